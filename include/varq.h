@@ -1,0 +1,152 @@
+/*
+ * varq.h -- C ABI of libvarq_hip.so: VAR-Q KV-cache quantization hot path for
+ * AMD MI355X (gfx950).
+ *
+ * The reference (lujiaji/VAR-Q) is pure Python and has no FFI; the interface
+ * replaced here is its Python surface.  Each entry point cites the reference
+ * lines whose work it performs.  Conventions common to every call:
+ *
+ *   - all pointers are DEVICE pointers unless named host_*; the library never
+ *     allocates, frees, synchronizes or keeps a pointer after returning;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - return value 0 = success, negative = one of varq_status; the message for
+ *     the calling thread's last failure is varq_last_error();
+ *   - shapes are validated on the host before any launch; nothing is launched
+ *     when validation fails;
+ *   - dtype codes: 0 = fp32, 1 = bf16, 2 = fp16;
+ *   - codes are signed two's complement in [-(2^(b-1)), 2^(b-1)-1]; packed
+ *     words hold 32/bits codes, code j of a word at bit j*bits, along the last
+ *     dimension (VAR_Q/pack_unpack.py:177-196).
+ */
+#ifndef VARQ_H
+#define VARQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VARQ_ABI_VERSION 1
+
+enum varq_status {
+  VARQ_OK = 0,
+  VARQ_ERR_INVALID = -1,     /* bad argument (shape, bits, dtype, null pointer) */
+  VARQ_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for      */
+  VARQ_ERR_LAUNCH = -3,      /* HIP reported an error at launch                 */
+  VARQ_ERR_WORKSPACE = -4    /* workspace too small                             */
+};
+
+enum varq_dtype { VARQ_F32 = 0, VARQ_BF16 = 1, VARQ_F16 = 2 };
+
+int varq_abi_version(void);
+const char *varq_last_error(void);
+
+/*
+ * Row mapping used by the calls that write into a pre-allocated packed cache.
+ * The input is seen as [n0, n1, n2] rows of `c` channels (the three leading
+ * dims of the 4-D K/V tensor).  Row (i0,i1,i2) is written to output row
+ *     s(i0,0)*os0 + s(i1,1)*os1 + s(i2,2)*os2 + off
+ * where s(i,d) = slot[i] if d == slot_dim (rows whose slot is negative are
+ * skipped) and i otherwise.  This is how a [B,H,n,c] step lands at token
+ * offset L0 of a [B,H',Lmax,...] cache, optionally only the heads of one
+ * bit-width class.  It replaces the torch.cat growth of VAR_Q/quant.py:200-201.
+ * Passed as 8 host int64: {n0,n1,n2,os0,os1,os2,off,slot_dim(-1 = none)}.
+ */
+
+/*
+ * One-pass quantize + pack for groups that are `group` contiguous channels of
+ * one row (group-wise along D; batch and tokens not reduced).  Performs
+ * VAR_Q/quant.py:112-121 (scale, codes) fused with VAR_Q/pack_unpack.py:177-196
+ * (pack); asym != 0 selects the min/max affine quantizer
+ * (scale=(max-min)/(2^b-1), zp=qmin-round(min/scale)).
+ *   x        [n_rows, c] row-major, dtype x_dtype (n_rows = n0*n1*n2 of rowmap)
+ *   words    [out_rows, c*bits/32] int32
+ *   scale,zp [out_rows, c/group] fp32 (zp may be NULL when asym == 0)
+ *   host_rowmap  NULL = dense (output row == input row), else 8 int64 as above
+ *   slot     device int32 table for slot_dim, or NULL
+ * Requires bits in {2,4,8}, c % 8 == 0, c*bits % 32 == 0, group % 8 == 0,
+ * c % group == 0 and group/8 a power of two <= 64.
+ */
+int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, int c, int group, int bits,
+                         int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
+                         int32_t *words, float *scale, float *zp, void *stream);
+
+/*
+ * General quantizer for the six grouping methods of VAR_Q/quant.py:75-95 and
+ * any other reduce set: a group is every element sharing the indices of the
+ * dims NOT in reduce_mask (bit d set = dim d reduced).  Two phases: group
+ * min/max into `workspace`, then scale/zp and codes (VAR_Q/quant.py:112-121).
+ *   x       [shape[0..3]] contiguous
+ *   scale   [n_groups] fp32 in the order of the kept dims; zp likewise or NULL
+ *   words   packed output [rows, ceil(c/(32/bits))] or NULL
+ *   codes   int8 output [rows, c] or NULL (the pack_to_int32=False mode,
+ *           VAR_Q/quant.py:174-175).  At least one of words/codes is non-NULL.
+ *   workspace  >= varq_quant_workspace_bytes(...) bytes, any contents
+ * bits in 2..8 when only codes are requested, {2,4,8} when words are.
+ */
+size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask);
+int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
+                    int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* VAR_Q/pack_unpack.py:107-134 (and its CPU twin 177-196): int8 codes [rows,c]
+ * -> int32 words [rows, ceil(c*bits/32)], zero padding in the last word. */
+int varq_pack(const int8_t *codes, int64_t rows, int c, int bits, int32_t *words, void *stream);
+
+/* VAR_Q/pack_unpack.py:136-162 (and 198-211): words -> sign-extended int8
+ * codes [rows, c]. */
+int varq_unpack(const int32_t *words, int64_t rows, int c, int bits, int8_t *codes, void *stream);
+
+/*
+ * Unpack + dequantize in one pass: VAR_Q/quant.py:216-224 (unpack, then
+ * q.float()*scale, 123-124), with the affine form (q - zp)*scale when zp is
+ * given.  The scale of element (i0,i1,i2,ch) of the [n0,n1,n2,c] code tensor
+ * is scale[i0*ss[0] + i1*ss[1] + i2*ss[2] + (ch/group)*ss[3]] (strides in
+ * elements, 0 = broadcast), so every layout the quantizer produces -- expanded
+ * per-step scales, per-token group scales, per-head tables -- is addressed
+ * without materializing it.
+ *   words  packed codes, or codes_i8 unpacked int8 codes (exactly one non-NULL)
+ *   in_row_stride  rows between consecutive i1 blocks is n2 unless the input
+ *                  is a window of a larger cache: host_in_rowmap as above maps
+ *                  (i0,i1,i2) to the INPUT row (NULL = dense)
+ *   out    [n0*n1*n2, c] dense, dtype out_dtype
+ */
+int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scale, const float *zp,
+                 const int64_t *host_shape4, const int64_t *host_scale_strides4, int group, int bits,
+                 const int64_t *host_in_rowmap, void *out, int out_dtype, void *stream);
+
+/*
+ * Fused dequant flash-attention (no counterpart in the reference, which
+ * dequantizes the whole cache to fp32 and calls an external attention backend:
+ * VAR_Q/quant.py:216-230, VAR/models/basic_var.py:156-162,
+ * Infinity/infinity/models/basic.py:339-351).
+ *
+ *   out[b,h,i,:] = softmax_j( softmax_scale * q[b,h,i,:] . K[b,h,j,:] + mask(i,j) ) V[b,h,j,:]
+ *   K = (k_codes - k_zp) * k_scale,  V likewise, never materialized.
+ *
+ *   q, out     bf16 [B, Hq, Lq, D]
+ *   k_words    int32 [B, Hkv, Lk_stride, D*k_bits/32]; only rows < Lk are read
+ *   k_scale/zp fp32  [B, Hkv, Lk_stride, D/k_group]   (zp NULL = symmetric)
+ *   v_*        same for V
+ *   head_map   device int32 [Hkv]: q/out head served by packed head slot s, or
+ *              NULL for identity (then Hkv == Hq).  One launch per bit-width
+ *              class serves a cache with mixed per-head bit-widths.
+ *   kv_limit   device int32 [Lq]: query i sees keys j < kv_limit[i]
+ *              (block-causal next-scale mask of VAR/models/var.py:110-114,
+ *              limit = end of the query's own scale); NULL = all Lk visible.
+ * Requires D in {64,128}, bits in {2,4,8}, k_group/v_group in {32,64,128}
+ * dividing D.
+ */
+int varq_fused_attn(const void *q, void *out,
+                    const int32_t *k_words, const float *k_scale, const float *k_zp, int k_bits, int k_group,
+                    const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
+                    int B, int Hq, int Hkv, const int32_t *head_map,
+                    int Lq, int Lk, int Lk_stride, int D,
+                    const int32_t *kv_limit, float softmax_scale, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VARQ_H */

@@ -1,0 +1,69 @@
+"""The C-ABI library loads and exports every symbol include/varq.h declares;
+argument validation rejects bad calls on the host, before anything is launched
+(so these run without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from var_q_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, 'include', 'varq.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(varq_[a-z_0-9]+)\s*\(', text)))
+
+
+def test_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared()
+    assert 'varq_quant_pack_rows' in names and 'varq_fused_attn' in names and len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
+    assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
+    assert lib.varq_abi_version() == 1
+
+
+def test_invalid_arguments_are_rejected_on_the_host():
+    lib = _lib.load()
+    i64 = _lib.i64arr
+    fake = ctypes.c_void_p(0x1000)     # never dereferenced: validation fails first
+    rc = lib.varq_quant_pack_rows(fake, 1, 4, 64, 64, 3, 1, 1e-12, None, None, fake, fake, fake, None)
+    assert rc == -1 and b'bits' in lib.varq_last_error()
+    rc = lib.varq_quant_pack_rows(fake, 1, 4, 60, 60, 4, 1, 1e-12, None, None, fake, fake, fake, None)
+    assert rc == -1
+    rc = lib.varq_quant_pack_rows(fake, 1, 4, 64, 24, 4, 1, 1e-12, None, None, fake, fake, fake, None)
+    assert rc == -1 and b'group' in lib.varq_last_error()
+    rc = lib.varq_quant_pack_rows(fake, 1, 4, 64, 64, 4, 1, 1e-12, None, None, fake, fake, None, None)
+    assert rc == -1 and b'zp' in lib.varq_last_error()
+    rc = lib.varq_pack(fake, 4, 16, 5, fake, None)
+    assert rc == -1
+    rc = lib.varq_unpack(fake, 4, 16, 3, fake, None)
+    assert rc == -1
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 9, 0, 1e-12, fake, None, fake, None, fake, 1 << 20, None)
+    assert rc == -1
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 3, 0, 1e-12, fake, None, fake, None, fake, 1 << 20, None)
+    assert rc == -1 and b'2/4/8' in lib.varq_last_error()
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 4, 0, 1e-12, fake, None, fake, None, fake, 4, None)
+    assert rc == -4
+    assert lib.varq_quant_workspace_bytes(i64([2, 5, 3, 8]), 0b0011) == 3 * 8 * 2 * 4
+    rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128,
+                             1, 2, 2, None, 16, 16, 16, 96, None, 1.0, None)
+    assert rc == -1 and b'D must be' in lib.varq_last_error()
+    rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 8, 128,
+                             1, 2, 2, None, 16, 16, 16, 128, None, 1.0, None)
+    assert rc == -2
+    # empty inputs are a no-op success
+    assert lib.varq_pack(None, 0, 16, 4, None, None) == 0
+    assert lib.varq_quant_pack_rows(fake, 1, 0, 64, 64, 4, 1, 1e-12, None, None, fake, fake, fake, None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, '_lib', None)
+    monkeypatch.setattr(_lib, 'LIB_PATH', str(tmp_path / 'nope.so'))
+    with pytest.raises(_lib.VarqError, match='no fallback'):
+        _lib.load()

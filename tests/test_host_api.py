@@ -1,0 +1,94 @@
+"""Host-side mirror of the reference's Python surface: constructor contract,
+derived fields, config loader, schedules -- and that CPU tensors are refused
+rather than silently computed somewhere else."""
+import json
+import os
+
+import pytest
+import torch
+
+import var_q_amd
+from var_q_amd import VAR_Q, VarqError, load_varq_config, schedules
+from var_q_amd import pack_unpack as PU
+
+PKG = os.path.dirname(var_q_amd.__file__)
+
+
+def test_constructor_contract_matches_reference():
+    q = VAR_Q()
+    assert (q.quant_bits, q.qkv_format, q.quant_method, q.cur_blk_idx, q.pack_to_int32, q.eps) == \
+        (8, 'BLHc', 'G_SCALE_HEAD_DIM', 0, True, 1e-12)
+    assert q.dim_cat == 1 and q.dim_map['G_TOKEN'] == (0, 2, 3) and q.dim_map['G_SCALE_HEAD_DIM'] == (0, 1)
+    assert (q.bound_min, q.bound_max) == (-128, 127)
+    assert q.cached_item is None and q.cached_scale is None and q.quantized_item is None and q.scale is None
+    assert q._pack_meta is None
+    q = VAR_Q(4, 'BHLc', 'G_TOKEN_HEAD', blk_idx=7)
+    assert q.dim_cat == 2 and q.dim_map['G_SCALE_HEAD_DIM'] == (0, 2) and q.dim_map['G_TOKEN'] == (0, 1, 3)
+    assert (q.bound_min, q.bound_max, q.cur_blk_idx) == (-8, 7, 7)
+    for bad in (dict(qkv_format='LBHc'), dict(quant_method='PER_DIM'), dict(quant_bits=1), dict(quant_bits=9)):
+        with pytest.raises(AssertionError):
+            VAR_Q(**bad)
+    with pytest.raises(AssertionError):
+        VAR_Q(quant_method='G_GROUP')          # needs group_size
+
+
+def test_qkv_format_assignment_rederives_layout():
+    q = VAR_Q(8, 'BLHc')
+    q.qkv_format = 'BHLc'                      # what Infinity's attention does every forward
+    assert q.dim_cat == 2 and q.dim_map['G_SCALE_HEAD_DIM'] == (0, 2)
+
+
+def test_cpu_tensors_are_refused():
+    q = VAR_Q(8, 'BLHc')
+    with pytest.raises(VarqError):
+        q.use_var_q(torch.randn(1, 2, 2, 8))
+    with pytest.raises(AssertionError):
+        PU.pack_last_dim_to_int32_triton(torch.zeros(2, 8, dtype=torch.int8), 4)
+    with pytest.raises(AssertionError):
+        PU.unpack_last_dim_from_int32_triton(torch.zeros(2, 1, dtype=torch.int32),
+                                             {'orig_c': 8, 'vals_per_word': 8, 'pad_len': 0, 'bits': 4})
+
+
+def test_reference_import_names_resolve():
+    from VAR_Q.quant import VAR_Q as A
+    from VAR_Q.pack_unpack import (pack_last_dim_to_int32_triton, unpack_last_dim_from_int32_triton,  # noqa: F401
+                                   pack_last_dim_to_int32_python, unpack_last_dim_from_int32_python)  # noqa: F401
+    from VAR_Q.config_loader import VARQConfig, load_varq_config as L  # noqa: F401
+    assert A is VAR_Q and L is load_varq_config
+
+
+@pytest.mark.parametrize('name,infinity', [('VAR-VAR_Q-8.json', False), ('Infinity-VAR_Q-8.json', True),
+                                           ('VAR-raw.json', False), ('Infinity-VAR_Q-4-g128.json', True)])
+def test_config_loader(name, infinity, tmp_path):
+    cfg = load_varq_config(os.path.join(PKG, name))
+    assert cfg.is_infinity_model() == infinity and cfg.is_var_model() != infinity
+    qc = cfg.get_quantization_config()
+    qc['enable'] = 'changed'
+    assert cfg.config['quantization']['enable'] != 'changed'       # getters return copies
+    assert cfg.get_device() in ('cuda', 'cpu')
+    assert cfg.get_batch_processing_config()['batch_size'] == 50
+    if infinity:
+        assert cfg.get_checkpoint_paths()[1].endswith('infinity_2b_reg.pth')
+    else:
+        assert cfg.get_checkpoint_paths(16)[1].endswith('var_d16.pth')
+        with pytest.raises(ValueError):
+            cfg.get_checkpoint_paths()
+    cfg.update_config({'quantization': {'q_bits': 4}, 'extra': {'a': 1}})
+    assert cfg.config['quantization']['q_bits'] == 4 and cfg.config['extra'] == {'a': 1}
+    if name != 'VAR-raw.json':
+        assert cfg.config['quantization']['quant_method'] in ('G_SCALE_HEAD_DIM', 'G_GROUP')
+        kw = cfg.quantizer_kwargs()
+        VAR_Q(**kw)
+    out = tmp_path / 'saved.json'
+    cfg.save_config(str(out))
+    assert json.load(open(out)) == cfg.config
+
+
+def test_schedules_and_kv_limit():
+    assert schedules.total_tokens(schedules.VAR_PATCH_NUMS) == 680
+    assert schedules.total_tokens(schedules.INFINITY_PATCH_NUMS) == 10521
+    lim = schedules.kv_limit((1, 2, 3))
+    assert lim.dtype == torch.int32 and lim.tolist() == [1] + [5] * 4 + [14] * 9
+    assert schedules.kv_limit((1, 2, 3), q_start=5).tolist() == [14] * 9
+    import varq_oracle as O
+    assert torch.equal(schedules.kv_limit(O.VAR_PATCH_NUMS), O.kv_limit_from_schedule(O.VAR_PATCH_NUMS))

@@ -1,0 +1,160 @@
+// Unpack + dequantize in one pass: what VAR_Q/quant.py:216-224 does with two
+// unpack launches per field, a stack, a sign-extension and a multiply
+// (VAR_Q/pack_unpack.py:198-211, VAR_Q/quant.py:123-124), plus the affine form
+// (q - zp) * scale.  HBM-bound; the output (fp32 in the reference, 4 B/element)
+// dominates the traffic, so bf16/fp16 outputs are offered too.
+//
+// One lane produces 8 consecutive channels.  A block stays inside one (i0,i1)
+// pair so the scale base and the input-window row base are block-uniform.
+#include "varq_common.h"
+
+namespace {
+
+struct DeqParams {
+  const int32_t *words;
+  const int8_t *codes;
+  const float *scale;
+  const float *zp;
+  void *out;
+  RowMap in_map;           // (i0,i1,i2) -> input row
+  int64_t n1, n2;
+  int64_t ss0, ss1, ss2, ss3;
+  int64_t octets_per_pair, blocks_per_pair;
+  int c, c8, wpr, bits, group;
+};
+
+template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t elem, const float (&f)[8], int n_valid) {
+  if (ODT == VARQ_F32) {
+    float *o = reinterpret_cast<float *>(out) + elem;
+    if (n_valid == 8) {
+      reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
+      reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
+    } else {
+      for (int j = 0; j < n_valid; ++j) o[j] = f[j];
+    }
+  } else {
+    uint16_t h[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) h[j] = (ODT == VARQ_BF16) ? f32_to_bf16_rne(f[j]) : f32_to_f16_rne(f[j]);
+    uint16_t *o = reinterpret_cast<uint16_t *>(out) + elem;
+    if (n_valid == 8) {
+      *reinterpret_cast<uint4 *>(o) = make_uint4(h[0] | ((u32)h[1] << 16), h[2] | ((u32)h[3] << 16),
+                                                 h[4] | ((u32)h[5] << 16), h[6] | ((u32)h[7] << 16));
+    } else {
+      for (int j = 0; j < n_valid; ++j) o[j] = h[j];
+    }
+  }
+}
+
+template <int ODT>
+__global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
+  const int64_t pair = blockIdx.x / p.blocks_per_pair;
+  const int64_t tile = blockIdx.x - pair * p.blocks_per_pair;
+  const int64_t o = tile * 256 + threadIdx.x;
+  if (o >= p.octets_per_pair) return;
+  const int64_t i0 = pair / p.n1, i1 = pair - i0 * p.n1;
+  const int64_t i2 = o / p.c8;
+  const int col = (int)(o - i2 * p.c8);
+  const int ch0 = col * 8;
+  const int n_valid = min(8, p.c - ch0);
+  const int64_t in_row = i0 * p.in_map.os0 + i1 * p.in_map.os1 + i2 * p.in_map.os2 + p.in_map.off;
+  const int64_t out_row = (i0 * p.n1 + i1) * p.n2 + i2;
+
+  int q[8];
+  if (p.codes) {
+    const int8_t *src = p.codes + in_row * p.c + ch0;
+    if (n_valid == 8 && (p.c & 7) == 0) {
+      uint2 b = *reinterpret_cast<const uint2 *>(src);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { q[j] = __builtin_amdgcn_sbfe((int)b.x, 8 * j, 8); q[4 + j] = __builtin_amdgcn_sbfe((int)b.y, 8 * j, 8); }
+    } else {
+      for (int j = 0; j < 8; ++j) q[j] = j < n_valid ? src[j] : 0;
+    }
+  } else {
+    const int32_t *src = p.words + in_row * p.wpr;
+    if (p.bits == 4) {
+      const int w = src[col];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_sbfe(w, 4 * j, 4);
+    } else if (p.bits == 8) {
+      const int w0 = src[col * 2];
+      const int w1 = (col * 2 + 1 < p.wpr) ? src[col * 2 + 1] : 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { q[j] = __builtin_amdgcn_sbfe(w0, 8 * j, 8); q[4 + j] = __builtin_amdgcn_sbfe(w1, 8 * j, 8); }
+    } else {
+      const int w = src[col >> 1] >> ((col & 1) * 16);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_sbfe(w, 2 * j, 2);
+    }
+  }
+
+  const int64_t sbase = i0 * p.ss0 + i1 * p.ss1 + i2 * p.ss2;
+  float f[8];
+  if ((p.group & 7) == 0) {
+    const int64_t g = sbase + (ch0 / p.group) * p.ss3;
+    const float s = p.scale[g];
+    if (p.zp) {
+      const float z = p.zp[g];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = ((float)q[j] - z) * s;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = (float)q[j] * s;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int ch = min(ch0 + j, p.c - 1);
+      const int64_t g = sbase + (ch / p.group) * p.ss3;
+      const float s = p.scale[g];
+      f[j] = p.zp ? ((float)q[j] - p.zp[g]) * s : (float)q[j] * s;
+    }
+  }
+  store8<ODT>(p.out, out_row * p.c + ch0, f, ((p.c & 7) == 0) ? 8 : n_valid);
+}
+
+}  // namespace
+
+extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scale, const float *zp,
+                            const int64_t *host_shape4, const int64_t *host_scale_strides4, int group, int bits,
+                            const int64_t *host_in_rowmap, void *out, int out_dtype, void *stream) {
+  VARQ_CHECK_ARG(host_shape4 && host_scale_strides4, "dequant: null shape/strides");
+  const int64_t *s = host_shape4;
+  VARQ_CHECK_ARG(s[0] >= 0 && s[1] >= 0 && s[2] >= 0 && s[3] > 0 && s[3] <= (1 << 20), "dequant: bad shape");
+  VARQ_CHECK_ARG((words != nullptr) != (codes_i8 != nullptr), "dequant: exactly one of words/codes must be given");
+  VARQ_CHECK_ARG(!words || bits == 2 || bits == 4 || bits == 8, "dequant: bits must be 2, 4 or 8 (got %d)", bits);
+  VARQ_CHECK_ARG(out_dtype >= 0 && out_dtype <= 2, "dequant: bad output dtype %d", out_dtype);
+  VARQ_CHECK_ARG(group >= 1 && group <= s[3], "dequant: bad group %d", group);
+  const int64_t rows = s[0] * s[1] * s[2];
+  if (rows == 0) return VARQ_OK;
+  VARQ_CHECK_ARG(scale && out, "dequant: null pointer");
+
+  DeqParams p;
+  p.words = words; p.codes = codes_i8; p.scale = scale; p.zp = zp; p.out = out;
+  p.n1 = s[1]; p.n2 = s[2];
+  p.c = (int)s[3];
+  p.c8 = (p.c + 7) / 8;
+  p.bits = bits; p.group = group;
+  p.wpr = words ? (p.c + 32 / bits - 1) / (32 / bits) : 0;
+  p.ss0 = host_scale_strides4[0]; p.ss1 = host_scale_strides4[1];
+  p.ss2 = host_scale_strides4[2]; p.ss3 = host_scale_strides4[3];
+  if (host_in_rowmap) {
+    p.in_map = varq_rowmap_from_host(host_in_rowmap, rows);
+    VARQ_CHECK_ARG(p.in_map.n0 == s[0] && p.in_map.n1 == s[1] && p.in_map.n2 == s[2], "dequant: row map dims differ from shape");
+    VARQ_CHECK_ARG(p.in_map.slot_dim < 0, "dequant: slot tables are not supported on input maps");
+  } else {
+    p.in_map.n0 = s[0]; p.in_map.n1 = s[1]; p.in_map.n2 = s[2];
+    p.in_map.os0 = s[1] * s[2]; p.in_map.os1 = s[2]; p.in_map.os2 = 1; p.in_map.off = 0; p.in_map.slot_dim = -1;
+  }
+  p.octets_per_pair = s[2] * p.c8;
+  p.blocks_per_pair = (p.octets_per_pair + 255) / 256;
+  const int64_t blocks = p.blocks_per_pair * s[0] * s[1];
+  VARQ_CHECK_ARG(blocks < (1ll << 31), "dequant: too many blocks");
+  dim3 grid((unsigned)blocks);
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == VARQ_F32) hipLaunchKernelGGL(dequant_kernel<VARQ_F32>, grid, dim3(256), 0, st, p);
+  else if (out_dtype == VARQ_BF16) hipLaunchKernelGGL(dequant_kernel<VARQ_BF16>, grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(dequant_kernel<VARQ_F16>, grid, dim3(256), 0, st, p);
+  VARQ_CHECK_LAUNCH("dequant");
+  return VARQ_OK;
+}

@@ -1,0 +1,241 @@
+"""Tensor-level entry points over the C ABI of libvarq_hip.so.
+
+torch is used here for device memory and the current stream only; all
+arithmetic happens in the HIP kernels.  Every function requires GPU tensors and
+raises otherwise -- there is no CPU path in the product.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import VarqError, check, i64arr
+
+_DT = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def _gpu(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        dev = getattr(t, 'device', type(t))
+        raise VarqError(f'{name} must be a GPU tensor (got {dev}); the VAR-Q HIP path has no CPU fallback')
+    return t
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise VarqError(f'unsupported dtype {t.dtype}; expected float32, bfloat16 or float16')
+    return _DT[t.dtype]
+
+
+# ---------------------------------------------------------------------------
+# row-local (group-wise along the last dim) quantize + pack
+# ---------------------------------------------------------------------------
+def quant_pack_rows(x: torch.Tensor, group: int, bits: int, asym: bool = True, eps: float = 1e-12
+                    ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """One-pass quantize+pack with one (scale[, zp]) per `group` contiguous
+    channels of each row.  x [..., c] -> (words [..., c*bits/32] int32,
+    scale [..., c/group] fp32, zp like scale or None)."""
+    _gpu(x, 'x')
+    x = x.contiguous()
+    *lead, c = x.shape
+    n_rows = x.numel() // c if c else 0
+    words = torch.empty((*lead, c * bits // 32), dtype=torch.int32, device=x.device)
+    scale = torch.empty((*lead, c // group), dtype=torch.float32, device=x.device)
+    zp = torch.empty_like(scale) if asym else None
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        check(lib.varq_quant_pack_rows(x.data_ptr(), _dt(x), n_rows, c, group, bits, int(asym), eps, None, None,
+                                       words.data_ptr(), scale.data_ptr(), _ptr(zp), _stream(x)), 'varq_quant_pack_rows')
+    return words, scale, zp
+
+
+def quant_pack_rows_into(x: torch.Tensor, group: int, bits: int, asym: bool, eps: float,
+                         words: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor],
+                         rowmap: Sequence[int], slot: Optional[torch.Tensor] = None) -> None:
+    """Same kernel writing into pre-allocated cache buffers through a row map
+    {n0,n1,n2,os0,os1,os2,off,slot_dim} (see include/varq.h)."""
+    _gpu(x, 'x'); _gpu(words, 'words'); _gpu(scale, 'scale')
+    assert x.is_contiguous() and words.is_contiguous() and scale.is_contiguous()
+    assert words.dtype == torch.int32 and scale.dtype == torch.float32
+    c = x.shape[-1]
+    n_rows = x.numel() // c
+    assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        check(lib.varq_quant_pack_rows(x.data_ptr(), _dt(x), n_rows, c, group, bits, int(asym), eps, i64arr(rowmap),
+                                       _ptr(slot), words.data_ptr(), scale.data_ptr(), _ptr(zp), _stream(x)),
+              'varq_quant_pack_rows')
+
+
+# ---------------------------------------------------------------------------
+# general (cross-row groups) quantize + pack
+# ---------------------------------------------------------------------------
+def quant_pack(x: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: bool = False, eps: float = 1e-12,
+               pack: bool = True) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Quantize a 4-D tensor with one group per index of the non-reduced dims.
+    Returns (packed int32 words or int8 codes, scale with keepdim shape, zp or None)."""
+    _gpu(x, 'x')
+    assert x.dim() == 4, 'expected a 4-D [B,L,H,c] / [B,H,L,c] tensor'
+    x = x.contiguous()
+    shape = list(x.shape)
+    mask = 0
+    for d in reduce_dims:
+        mask |= 1 << (d % 4)
+    sshape = [1 if (mask >> d) & 1 else shape[d] for d in range(4)]
+    scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    zp = torch.empty_like(scale) if asym else None
+    c = shape[3]
+    if pack:
+        vals = 32 // bits
+        q = torch.empty((*shape[:3], (c + vals - 1) // vals), dtype=torch.int32, device=x.device)
+    else:
+        q = torch.empty(shape, dtype=torch.int8, device=x.device)
+    lib = _lib.load()
+    sh = i64arr(shape)
+    ws_bytes = lib.varq_quant_workspace_bytes(sh, mask)
+    ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.varq_quant_pack(x.data_ptr(), _dt(x), sh, mask, bits, int(asym), eps,
+                                  q.data_ptr() if pack else None, None if pack else q.data_ptr(),
+                                  scale.data_ptr(), _ptr(zp), ws.data_ptr(), ws.numel(), _stream(x)), 'varq_quant_pack')
+    return q, scale, zp
+
+
+# ---------------------------------------------------------------------------
+# pack / unpack of int8 codes
+# ---------------------------------------------------------------------------
+def pack(codes: torch.Tensor, bits: int) -> torch.Tensor:
+    _gpu(codes, 'q_int8')
+    codes = codes.contiguous()
+    *lead, c = codes.shape
+    vals = 32 // bits
+    rows = codes.numel() // c if c else 0
+    words = torch.empty((*lead, (c + vals - 1) // vals), dtype=torch.int32, device=codes.device)
+    lib = _lib.load()
+    with torch.cuda.device(codes.device):
+        check(lib.varq_pack(codes.data_ptr(), rows, c, bits, words.data_ptr(), _stream(codes)), 'varq_pack')
+    return words
+
+
+def unpack(words: torch.Tensor, c: int, bits: int) -> torch.Tensor:
+    _gpu(words, 'packed')
+    words = words.contiguous()
+    *lead, w = words.shape
+    rows = words.numel() // w if w else 0
+    codes = torch.empty((*lead, c), dtype=torch.int8, device=words.device)
+    lib = _lib.load()
+    with torch.cuda.device(words.device):
+        check(lib.varq_unpack(words.data_ptr(), rows, c, bits, codes.data_ptr(), _stream(words)), 'varq_unpack')
+    return codes
+
+
+# ---------------------------------------------------------------------------
+# unpack + dequantize
+# ---------------------------------------------------------------------------
+def dequant(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], c: int, bits: int,
+            out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """q: packed int32 words [n0,n1,n2,W] or int8 codes [n0,n1,n2,c].  scale
+    (and zp) broadcast against [n0,n1,n2,c] in the first three dims and hold
+    1, c/g or c entries in the last (per-row, group-wise, per-channel); any
+    strides, including stride-0 expands, are used as they are."""
+    _gpu(q, 'q'); _gpu(scale, 'scale')
+    assert q.dim() == 4 and scale.dim() == 4
+    q = q.contiguous()
+    n0, n1, n2 = q.shape[:3]
+    packed = q.dtype == torch.int32
+    assert packed or q.dtype == torch.int8
+    if zp is not None and (zp.shape != scale.shape or zp.stride() != scale.stride()):
+        zp = zp.expand_as(scale).contiguous()
+        scale = scale.contiguous()
+    s3 = scale.shape[3]
+    assert c % s3 == 0, f'scale last dim {s3} does not divide c={c}'
+    group = c // s3
+    strides = []
+    for d in range(4):
+        if scale.shape[d] == 1:
+            strides.append(0)
+        else:
+            assert d == 3 or scale.shape[d] == q.shape[d], f'scale dim {d} = {scale.shape[d]} vs {q.shape[d]}'
+            strides.append(scale.stride(d))
+    out = torch.empty((n0, n1, n2, c), dtype=out_dtype, device=q.device)
+    lib = _lib.load()
+    # collapse the leading dims when the scale does not depend on them: fuller blocks
+    shape = [n0, n1, n2, c]
+    if strides[0] == 0 and strides[1] == 0 and strides[2] == 0:
+        shape = [1, 1, n0 * n1 * n2, c]
+    elif strides[0] == 0 and strides[1] == 0:
+        pass
+    with torch.cuda.device(q.device):
+        check(lib.varq_dequant(q.data_ptr() if packed else None, None if packed else q.data_ptr(),
+                               scale.data_ptr(), _ptr(zp), i64arr(shape), i64arr(strides), group, bits, None,
+                               out.data_ptr(), _DT[out_dtype], _stream(q)), 'varq_dequant')
+    return out
+
+
+def dequant_window(words: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], shape4: Sequence[int],
+                   scale_strides4: Sequence[int], group: int, bits: int, in_rowmap: Sequence[int],
+                   out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Dequantize a [n0,n1,n2,c] window of a larger packed cache; the window's
+    rows are located through in_rowmap, scales through explicit strides."""
+    _gpu(words, 'words'); _gpu(scale, 'scale')
+    packed = words.dtype == torch.int32
+    assert packed or words.dtype == torch.int8
+    out = torch.empty(tuple(shape4), dtype=out_dtype, device=words.device)
+    lib = _lib.load()
+    with torch.cuda.device(words.device):
+        check(lib.varq_dequant(words.data_ptr() if packed else None, None if packed else words.data_ptr(),
+                               scale.data_ptr(), _ptr(zp), i64arr(shape4),
+                               i64arr(scale_strides4), group, bits, i64arr(in_rowmap), out.data_ptr(),
+                               _DT[out_dtype], _stream(words)), 'varq_dequant')
+    return out
+
+
+# ---------------------------------------------------------------------------
+# fused dequant flash-attention
+# ---------------------------------------------------------------------------
+def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_zp: Optional[torch.Tensor],
+               v_words: torch.Tensor, v_scale: torch.Tensor, v_zp: Optional[torch.Tensor],
+               k_bits: int, v_bits: int, Lk: int, softmax_scale: float,
+               kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32;
+    k/v_scale (zp) [B,Hkv,Lstride,D/group] fp32; attends keys 0..Lk-1.
+    Returns out [B,Hq,Lq,D] bf16 (rows of heads not in head_map are untouched)."""
+    for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_scale, 'k_scale'), (v_scale, 'v_scale')):
+        _gpu(t, n)
+        assert t.is_contiguous(), f'{n} must be contiguous'
+    assert q.dtype == torch.bfloat16 and q.dim() == 4
+    B, Hq, Lq, D = q.shape
+    Bk, Hkv, Lstride, Wk = k_words.shape
+    assert Bk == B and v_words.shape[:3] == k_words.shape[:3]
+    assert Wk * 32 == D * k_bits and v_words.shape[3] * 32 == D * v_bits
+    assert k_scale.shape[:3] == (B, Hkv, Lstride) and v_scale.shape[:3] == (B, Hkv, Lstride)
+    k_group, v_group = D // k_scale.shape[3], D // v_scale.shape[3]
+    if out is None:
+        out = torch.empty_like(q)
+    if kv_limit is not None:
+        _gpu(kv_limit, 'kv_limit')
+        assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
+    if head_map is not None:
+        _gpu(head_map, 'head_map')
+        assert head_map.dtype == torch.int32 and head_map.numel() == Hkv
+    else:
+        assert Hkv == Hq
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        check(lib.varq_fused_attn(q.data_ptr(), out.data_ptr(),
+                                  k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp), k_bits, k_group,
+                                  v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), v_bits, v_group,
+                                  B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
+                                  _ptr(kv_limit), float(softmax_scale), _stream(q)), 'varq_fused_attn')
+    return out

@@ -1,0 +1,234 @@
+"""Drop-in for the reference class VAR_Q (VAR_Q/quant.py:52-230): quantizer plus
+per-step KV cache state machine, on HIP kernels.
+
+Same constructor arguments, methods (`quant`, `cache`, `dequant_current`,
+`dequant_all`, `use_var_q`), readable attributes and error behaviour.  What
+changes underneath:
+
+* scale + codes + packing is one kernel chain (ops.quant_pack /
+  ops.quant_pack_rows) instead of ~15 torch launches with fp32 temporaries;
+* unpack + dequant is one kernel (ops.dequant_window);
+* the cache lives in pre-allocated buffers that grow geometrically; a step is
+  written in place instead of re-copying the whole cache with torch.cat
+  (VAR_Q/quant.py:200-201).  `cached_item` / `cached_scale` are views of the
+  valid part and hold the same values the reference's concatenations hold.
+
+Behaviour kept on purpose, because callers can observe it:
+* every method reduces over the batch dim (VAR_Q/quant.py:78-95);
+* G_HEAD_DIM and G_TENSOR re-quantize cat(dequant_all(), item)
+  (VAR_Q/quant.py:149-159); G_TENSOR then *appends* that re-quantized
+  concatenation (the first branch of cache() matches it, VAR_Q/quant.py:196-201);
+* dequantized tensors are fp32 (VAR_Q/quant.py:123-124).
+
+Extensions (absent from the reference): `symmetric=False` selects the min/max
+affine quantizer (attributes `zp`, `cached_zp`); quant_method 'G_GROUP' with
+`group_size=g` quantizes g contiguous channels of each token independently
+(batch and tokens not reduced); 'G_HEAD' keeps one scale per head.
+GPU tensors only.
+"""
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import ops
+from ._lib import VarqError
+
+_REF_METHODS = ('G_TENSOR', 'G_SCALE_HEAD_DIM', 'G_HEAD_DIM', 'G_SCALE', 'G_TOKEN', 'G_TOKEN_HEAD')
+_EXT_METHODS = ('G_GROUP', 'G_HEAD')
+
+
+def _dim_map(qkv_format: str) -> Dict[str, Tuple[int, ...]]:
+    if qkv_format == 'BLHc':
+        return {'G_TENSOR': (0, 1, 2, 3), 'G_SCALE_HEAD_DIM': (0, 1), 'G_HEAD_DIM': (0, 1), 'G_TOKEN': (0, 2, 3),
+                'G_TOKEN_HEAD': (0, 3), 'G_SCALE': (0, 1, 2, 3), 'G_HEAD': (0, 1, 3), 'G_GROUP': (3,)}
+    return {'G_TENSOR': (0, 1, 2, 3), 'G_SCALE_HEAD_DIM': (0, 2), 'G_HEAD_DIM': (0, 2), 'G_TOKEN': (0, 1, 3),
+            'G_TOKEN_HEAD': (0, 3), 'G_SCALE': (0, 1, 2, 3), 'G_HEAD': (0, 2, 3), 'G_GROUP': (3,)}
+
+
+class _Growable:
+    """Buffer that grows along one dim; `view()` is the valid prefix."""
+
+    def __init__(self, dim: int):
+        self.dim, self.buf, self.len = dim, None, 0
+
+    def append(self, t: torch.Tensor):
+        n = t.size(self.dim)
+        if self.buf is None or self.len + n > self.buf.size(self.dim):
+            cap = max(2 * (self.len + n), 64)
+            shape = list(t.shape)
+            shape[self.dim] = cap
+            new = torch.empty(shape, dtype=t.dtype, device=t.device)
+            if self.buf is not None and self.len:
+                new.narrow(self.dim, 0, self.len).copy_(self.buf.narrow(self.dim, 0, self.len))
+            self.buf = new
+        self.buf.narrow(self.dim, self.len, n).copy_(t)
+        self.len += n
+
+    def replace(self, t: torch.Tensor):
+        self.buf, self.len = t, t.size(self.dim)
+
+    def view(self) -> Optional[torch.Tensor]:
+        return None if self.buf is None else self.buf.narrow(self.dim, 0, self.len)
+
+
+class VAR_Q:
+    def __init__(self, quant_bits: int = 8, qkv_format: str = 'BLHc', quant_method: str = 'G_SCALE_HEAD_DIM',
+                 blk_idx: int = 0, pack_to_int32: bool = True, eps: float = 1e-12, debug: bool = False,
+                 symmetric: bool = True, group_size: Optional[int] = None):
+        assert qkv_format in ('BLHc', 'BHLc'), f"Invalid qkv_format: {qkv_format}"
+        assert quant_method in _REF_METHODS + _EXT_METHODS, f"Invalid quant_method: {quant_method}"
+        assert 1 < quant_bits <= 8, "Only support (2..8] bits (common 2/4/8 bits); bit-pack implementation covers 2/4/8 bits"
+        if quant_method == 'G_GROUP':
+            assert group_size is not None and group_size > 0, "G_GROUP needs group_size"
+            assert pack_to_int32, "G_GROUP always packs"
+        self.quant_bits = quant_bits
+        self.quant_method = quant_method
+        self.cur_blk_idx = blk_idx
+        self.pack_to_int32 = pack_to_int32
+        self.eps = eps
+        self.debug = debug
+        self.symmetric = symmetric
+        self.group_size = group_size
+        self.qkv_format = qkv_format   # property: also derives dim_cat / dim_map
+        self.bound_min = -(2 ** (quant_bits - 1))
+        self.bound_max = (2 ** (quant_bits - 1)) - 1
+
+        self.quantized_item: Optional[torch.Tensor] = None
+        self.scale: Optional[torch.Tensor] = None
+        self.zp: Optional[torch.Tensor] = None
+        self._pack_meta: Optional[Dict[str, int]] = None
+        self._reset_cache()
+
+    # The reference derives dim_cat/dim_map once in __init__ and callers later
+    # assign `qkv_format` (Infinity/infinity/models/basic.py:309,314) without the
+    # derived fields following.  Here the assignment re-derives them.
+    @property
+    def qkv_format(self) -> str:
+        return self._qkv_format
+
+    @qkv_format.setter
+    def qkv_format(self, fmt: str):
+        assert fmt in ('BLHc', 'BHLc'), f"Invalid qkv_format: {fmt}"
+        self._qkv_format = fmt
+        self.dim_cat = 1 if fmt == 'BLHc' else 2
+        self.dim_map = _dim_map(fmt)
+
+    # ---------------- cache views ----------------
+    def _reset_cache(self):
+        self._c_item = _Growable(self.dim_cat)
+        self._c_scale = _Growable(self.dim_cat)
+        self._c_zp = _Growable(self.dim_cat)
+
+    @property
+    def cached_item(self) -> Optional[torch.Tensor]:
+        return self._c_item.view()
+
+    @property
+    def cached_scale(self) -> Optional[torch.Tensor]:
+        return self._c_scale.view()
+
+    @property
+    def cached_zp(self) -> Optional[torch.Tensor]:
+        return self._c_zp.view()
+
+    # ---------------- quantize ----------------
+    def _quantize(self, x: torch.Tensor):
+        if not isinstance(x, torch.Tensor) or not x.is_cuda:
+            raise VarqError('VAR_Q requires GPU tensors; there is no CPU path in this package')
+        m = self.quant_method
+        if m == 'G_GROUP':
+            q, s, z = ops.quant_pack_rows(x, self.group_size, self.quant_bits, asym=not self.symmetric, eps=self.eps)
+        else:
+            q, s, z = ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
+                                     pack=self.pack_to_int32)
+        return q, s, z
+
+    def quant(self, item: torch.Tensor):
+        m = self.quant_method
+        if m in ('G_HEAD_DIM', 'G_TENSOR') and self.cached_item is not None and self.cached_scale is not None:
+            item = torch.cat([self.dequant_all(), item], dim=self.dim_cat)
+        elif m not in _REF_METHODS + _EXT_METHODS:
+            raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
+        if self.pack_to_int32:
+            assert self.quant_bits in (2, 4, 8), "bit-pack only implements 2/4/8 bits"
+        q, s, z = self._quantize(item)
+        if self.pack_to_int32:
+            c, vals = item.shape[-1], 32 // self.quant_bits
+            meta = {'orig_c': int(c), 'vals_per_word': int(vals), 'pad_len': int((-c) % vals), 'bits': int(self.quant_bits)}
+            if self._pack_meta is not None:
+                assert meta['bits'] == self._pack_meta['bits']
+                assert meta['vals_per_word'] == self._pack_meta['vals_per_word']
+                assert meta['orig_c'] == self._pack_meta['orig_c']
+                assert meta['pad_len'] == self._pack_meta['pad_len']
+            self._pack_meta = meta
+        self.quantized_item, self.scale, self.zp = q, s, z
+
+    # ---------------- cache ----------------
+    def _expand_scale_like_L(self, q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+        d = 1 if self.qkv_format == 'BLHc' else 2
+        if scale.size(d) == 1 and q.size(d) > 1:
+            shape = [-1, -1, -1, -1]
+            shape[d] = q.size(d)
+            scale = scale.expand(*shape)
+        return scale
+
+    def cache(self):
+        m = self.quant_method
+        q_cur = self.quantized_item
+        s_cur = self._expand_scale_like_L(q_cur, self.scale)
+        z_cur = None if self.zp is None else self._expand_scale_like_L(q_cur, self.zp)
+        if m in ('G_SCALE_HEAD_DIM', 'G_SCALE', 'G_TOKEN', 'G_TOKEN_HEAD', 'G_TENSOR', 'G_GROUP', 'G_HEAD'):
+            if self._c_item.dim != self.dim_cat:   # layout was re-assigned before the first step
+                self._reset_cache()
+            self._c_item.append(q_cur)
+            self._c_scale.append(s_cur)
+            if z_cur is not None:
+                self._c_zp.append(z_cur)
+        elif m == 'G_HEAD_DIM':
+            self._c_item.replace(q_cur)
+            self._c_scale.replace(s_cur)
+            if z_cur is not None:
+                self._c_zp.replace(z_cur)
+        else:
+            raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
+
+    # ---------------- dequantize ----------------
+    def _dequant(self, q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor]) -> torch.Tensor:
+        if self.pack_to_int32:
+            assert self._pack_meta is not None, "pack meta is missing"
+            c = self._pack_meta['orig_c']
+        else:
+            c = q.shape[-1]
+        return _dequant_views(q, scale, zp, c, self.quant_bits)
+
+    def dequant_current(self) -> torch.Tensor:
+        return self._dequant(self.quantized_item, self.scale, self.zp)
+
+    def dequant_all(self) -> torch.Tensor:
+        if self.cached_item is None:
+            return self.dequant_current()
+        return self._dequant(self.cached_item, self.cached_scale, self.cached_zp)
+
+    def use_var_q(self, item: torch.Tensor) -> torch.Tensor:
+        self.quant(item)
+        self.cache()
+        return self.dequant_all()
+
+
+def _dequant_views(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], c: int, bits: int,
+                   out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Dequantize codes given as a (possibly strided) 4-D view of a cache buffer
+    whose rows are dense, with a scale that is any broadcastable strided view."""
+    assert q.dim() == 4 and scale.dim() == 4
+    n0, n1, n2, wq = q.shape
+    assert q.stride(3) == 1 and all(st % wq == 0 for st in q.stride()[:3]), 'rows of the code tensor must be dense'
+    rowmap = [n0, n1, n2, q.stride(0) // wq, q.stride(1) // wq, q.stride(2) // wq, 0, -1]
+    if zp is not None and (zp.shape != scale.shape or zp.stride() != scale.stride()):
+        scale, zp = scale.contiguous(), zp.expand_as(scale).contiguous()
+    s3 = scale.shape[3]
+    assert c % s3 == 0
+    group = c // s3
+    strides = [0 if scale.shape[d] == 1 else scale.stride(d) for d in range(4)]
+    for d in range(3):
+        assert scale.shape[d] in (1, q.shape[d]), f'scale dim {d}: {scale.shape[d]} vs {q.shape[d]}'
+    return ops.dequant_window(q, scale, zp, (n0, n1, n2, c), strides, group, bits, rowmap, out_dtype)
