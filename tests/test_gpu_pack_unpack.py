@@ -1,0 +1,90 @@
+"""Parity of the stand-alone pack / unpack / dequant kernels with the oracle,
+through the reference's function names."""
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import note
+from var_q_amd import ops
+from var_q_amd import pack_unpack as PU
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('shape', [(100, 680, 2, 64), (3, 7, 5, 128), (4, 10), (9, 33), (2, 3, 1), (1, 16), (0, 64)])
+def test_pack_unpack_roundtrip_and_layout(dev, bits, shape):
+    note('pack/unpack', bits, shape)
+    lo, hi = O.qrange(bits)
+    g = torch.Generator().manual_seed(bits)
+    q = torch.randint(lo, hi + 1, shape, generator=g, dtype=torch.int8)
+    want, meta = O.pack_last_dim(q, bits) if q.numel() else (torch.empty((*shape[:-1], -(-shape[-1] // (32 // bits))), dtype=torch.int32), None)
+    w, gmeta = PU.pack_last_dim_to_int32_triton(q.to(dev), bits)
+    assert w.dtype == torch.int32 and w.shape == want.shape
+    assert torch.equal(w.cpu(), want)
+    if meta is not None:
+        assert gmeta == meta
+    back = PU.unpack_last_dim_from_int32_triton(w, gmeta)
+    assert back.dtype == torch.int8 and torch.equal(back.cpu(), q)
+    # the _python names are the same kernels
+    w2, _ = PU.pack_last_dim_to_int32_python(q.to(dev), bits)
+    assert torch.equal(w2, w)
+    assert torch.equal(PU.unpack_last_dim_from_int32_python(w, gmeta), back)
+
+
+def test_known_answer_words_on_gpu(dev):
+    note('pack KAT')
+    w, _ = PU.pack_last_dim_to_int32_triton(torch.tensor([[-1, -128, 127, 5]], dtype=torch.int8, device=dev), 8)
+    assert w.tolist() == [[0x057F80FF]]
+    w, _ = PU.pack_last_dim_to_int32_triton(torch.tensor([[-2, -1, 0, 1] * 4], dtype=torch.int8, device=dev), 2)
+    assert w.tolist() == [[0x4E4E4E4E]]
+    w, _ = PU.pack_last_dim_to_int32_triton(torch.arange(8, dtype=torch.int8, device=dev).view(1, 8), 4)
+    assert w.tolist() == [[0x76543210]]
+
+
+def test_asserts_like_reference(dev):
+    with pytest.raises(AssertionError):
+        PU.pack_last_dim_to_int32_triton(torch.zeros(2, 8, dtype=torch.int32, device=dev), 4)
+    with pytest.raises(AssertionError):
+        PU.pack_last_dim_to_int32_triton(torch.zeros(2, 8, dtype=torch.int8, device=dev), 3)
+    with pytest.raises(AssertionError):
+        PU.unpack_last_dim_from_int32_triton(torch.zeros(2, 1, dtype=torch.int8, device=dev),
+                                             {'orig_c': 8, 'vals_per_word': 8, 'pad_len': 0, 'bits': 4})
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_dequant_matches_oracle(dev, bits, out_dtype):
+    g = torch.Generator().manual_seed(bits + 40)
+    lo, hi = O.qrange(bits)
+    B, H, L, c = 2, 3, 11, 64
+    q = torch.randint(lo, hi + 1, (B, H, L, c), generator=g, dtype=torch.int8)
+    words, _ = O.pack_last_dim(q, bits)
+    cases = {
+        'per-tensor': (1, 1, 1, 1), 'per-head-dim': (1, H, 1, c), 'token-head': (1, H, L, 1),
+        'token': (1, 1, L, 1), 'group32': (B, H, L, 2), 'group64': (B, H, L, 1), 'per-head': (1, H, 1, 1),
+    }
+    for name, sshape in cases.items():
+        for asym in (False, True):
+            note('dequant', bits, out_dtype, name, asym)
+            s = torch.rand(sshape, generator=g) + 0.01
+            z = torch.randint(-9, 9, sshape, generator=g).float() if asym else None
+            if sshape[3] in (1, c):
+                want = O.dequant_asym(q, s, z) if asym else O.dequant_sym(q, s)
+            else:
+                want = O.dequant_groupwise(q, s, z, c // sshape[3])
+            got = ops.dequant(words.to(dev), s.to(dev), None if z is None else z.to(dev), c, bits, out_dtype)
+            assert got.dtype == out_dtype
+            assert torch.equal(got.cpu(), want.to(out_dtype)), name
+            got8 = ops.dequant(q.to(dev), s.to(dev), None if z is None else z.to(dev), c, bits, out_dtype)
+            assert torch.equal(got8.cpu(), want.to(out_dtype)), name + ' (int8 codes)'
+
+
+def test_dequant_ragged_channels_and_expanded_scale(dev):
+    note('dequant ragged')
+    g = torch.Generator().manual_seed(9)
+    q = torch.randint(-8, 8, (2, 5, 3, 10), generator=g, dtype=torch.int8)
+    words, _ = O.pack_last_dim(q, 4)
+    s = (torch.rand(1, 1, 3, 10, generator=g) + 0.1).expand(1, 5, 3, 10)     # stride-0 expand along L
+    got = ops.dequant(words.to(dev), s.to(dev).expand(1, 5, 3, 10), None, 10, 4)
+    assert torch.equal(got.cpu(), O.dequant_sym(q, s))

@@ -1,0 +1,93 @@
+"""Parity of the one-pass row-local quantize+pack kernel (through the C ABI)
+with the CPU oracle: packed words, scales and zero-points bit-exact."""
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import adversarial_rows, note
+from var_q_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(x_cpu, group, bits, asym, dev):
+    q, s, z = O.quant_groupwise(x_cpu, group, bits, asym)
+    want_w, _ = O.pack_last_dim(q, bits)
+    w, gs, gz = ops.quant_pack_rows(x_cpu.to(dev), group, bits, asym)
+    torch.cuda.synchronize()
+    assert torch.equal(gs.cpu(), s), 'scale mismatch'
+    if asym:
+        assert torch.equal(gz.cpu(), z), 'zero-point mismatch'
+    else:
+        assert gz is None
+    bad = (w.cpu() != want_w)
+    assert not bool(bad.any()), f'{int(bad.sum())} packed words differ'
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('asym', [False, True])
+def test_random_shapes(dev, dtype, bits, asym):
+    g = torch.Generator().manual_seed(bits * 7 + int(asym))
+    for shape, group in [((3, 5, 7, 64), 64), ((3, 5, 7, 64), 32), ((2, 4, 33, 128), 128), ((2, 4, 33, 128), 64),
+                         ((1, 2, 9, 128), 16), ((300, 64), 8), ((5, 512), 512), ((7, 256), 256)]:
+        note('quant_rows', dtype, bits, asym, shape, group)
+        x = (torch.randn(*shape, generator=g) * 3).to(dtype)
+        x[..., 5] *= 15
+        _check(x, group, bits, asym, dev)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('asym', [False, True])
+@pytest.mark.parametrize('c,group', [(64, 64), (128, 128), (128, 32)])
+def test_adversarial_rows(dev, dtype, bits, asym, c, group):
+    note('quant_rows adversarial', dtype, bits, asym, c, group)
+    _check(adversarial_rows(c, dtype), group, bits, asym, dev)
+
+
+def test_empty_and_single_row(dev):
+    note('quant_rows empty')
+    w, s, z = ops.quant_pack_rows(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), 64, 4, True)
+    assert w.shape == (0, 8) and s.shape == (0, 1)
+    _check(torch.randn(1, 64).bfloat16(), 64, 4, True, dev)
+
+
+def test_infinity2b_full_shape_int4_g128(dev):
+    """BASELINE config 4 at full size: [2,16,10521,128] bf16, INT4 asym g=128."""
+    note('quant_rows c4 full')
+    x = O.synth_kv((2, 16, 10521, 128), seed=1004, dist='student4', outlier_frac=0.01, outlier_mul=20.0,
+                   dtype=torch.bfloat16)
+    _check(x, 128, 4, True, dev)
+
+
+def test_var_d16_batch_shape_int4(dev):
+    """BASELINE config 2 shapes (B reduced to 8 to keep the CPU oracle quick):
+    K group 32, V group 64."""
+    note('quant_rows c2')
+    k = O.synth_kv((8, 16, 680, 64), seed=1002, dtype=torch.bfloat16)
+    _check(k, 32, 4, True, dev)
+    _check(k, 64, 4, True, dev)
+
+
+def test_row_map_appends_into_cache(dev):
+    """Two steps written at token offsets of a [B,H,Lmax,...] cache equal the
+    concatenation of the steps quantized on their own (VAR_Q/quant.py:196-201)."""
+    B, H, D, Lmax, g, bits = 2, 3, 64, 40, 32, 4
+    gen = torch.Generator().manual_seed(3)
+    words = torch.zeros(B, H, Lmax, D * bits // 32, dtype=torch.int32, device=dev)
+    scale = torch.zeros(B, H, Lmax, D // g, device=dev)
+    zp = torch.zeros_like(scale)
+    off, parts = 0, []
+    for n in (1, 4, 9):
+        note('row map step', n)
+        x = torch.randn(B, H, n, D, generator=gen).bfloat16()
+        parts.append(x)
+        ops.quant_pack_rows_into(x.to(dev), g, bits, True, 1e-12, words, scale, zp,
+                                 [B, H, n, H * Lmax, Lmax, 1, off, -1])
+        off += n
+    cat = torch.cat(parts, dim=2)
+    q, s, z = O.quant_groupwise(cat, g, bits, True)
+    assert torch.equal(words[:, :, :off].cpu(), O.pack_last_dim(q, bits)[0])
+    assert torch.equal(scale[:, :, :off].cpu(), s) and torch.equal(zp[:, :, :off].cpu(), z)
+    assert int(words[:, :, off:].abs().sum()) == 0           # nothing written past the end

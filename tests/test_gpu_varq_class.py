@@ -1,0 +1,86 @@
+"""The drop-in VAR_Q class on the GPU against the oracle's restatement of the
+reference class, step by step: codes, scales, cache contents and the fp32
+tensors handed to attention are identical."""
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import note
+from var_q_amd import VAR_Q
+
+pytestmark = pytest.mark.gpu
+
+STEPS = (1, 4, 9, 16)
+
+
+def _steps(fmt, dtype, seed, H=3, c=64, B=2):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for n in STEPS:
+        x = (torch.randn(B, n, H, c, generator=g) * 2).to(dtype)
+        out.append(x if fmt == 'BLHc' else x.permute(0, 2, 1, 3).contiguous())
+    return out
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('method', list(O.METHODS))
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('pack', [True, False])
+def test_state_machine_matches_oracle(dev, fmt, method, bits, pack):
+    note('VAR_Q', fmt, method, bits, pack)
+    ref = O.OracleVARQ(bits, fmt, method, pack_to_int32=pack)
+    gpu = VAR_Q(bits, fmt, method, pack_to_int32=pack)
+    for i, x in enumerate(_steps(fmt, torch.bfloat16 if bits == 4 else torch.float32, seed=bits)):
+        want = ref.use_var_q(x)
+        got = gpu.use_var_q(x.to(dev))
+        assert got.dtype == torch.float32 and got.shape == want.shape, (i, got.shape, want.shape)
+        assert torch.equal(got.cpu(), want), f'step {i}: dequantized K/V differ'
+        assert torch.equal(gpu.scale.cpu(), ref.scale)
+        assert torch.equal(gpu.quantized_item.cpu(), ref.quantized_item)
+        assert torch.equal(gpu.cached_item.cpu(), ref.cached_item)
+        assert torch.equal(gpu.cached_scale.cpu(), ref.cached_scale.contiguous())
+        assert gpu._pack_meta == ref._pack_meta
+        assert torch.equal(gpu.dequant_current().cpu(), ref.dequant_current())
+
+
+def test_hook_usage_pattern(dev):
+    """Two quantizers per layer, k then v each step, as in
+    VAR/models/basic_var.py:109-110,146-147 (BLHc, 8-bit, the shipped rule)."""
+    note('VAR_Q hook pattern')
+    kq, vq = VAR_Q(8, 'BLHc', 'G_SCALE_HEAD_DIM', blk_idx=3), VAR_Q(8, 'BLHc', 'G_SCALE_HEAD_DIM', blk_idx=3)
+    kr, vr = O.OracleVARQ(8, 'BLHc'), O.OracleVARQ(8, 'BLHc')
+    g = torch.Generator().manual_seed(11)
+    for pn in (1, 2, 3, 4):
+        k = torch.randn(4, pn * pn, 16, 64, generator=g).half()
+        v = torch.randn(4, pn * pn, 16, 64, generator=g).half()
+        assert torch.equal(kq.use_var_q(k.to(dev)).cpu(), kr.use_var_q(k))
+        assert torch.equal(vq.use_var_q(v.to(dev)).cpu(), vr.use_var_q(v))
+    assert kq.cached_item.shape == (4, 30, 16, 16)
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('group', [32, 64])
+def test_groupwise_asymmetric_extension(dev, bits, group):
+    note('VAR_Q G_GROUP', bits, group)
+    gpu = VAR_Q(bits, 'BHLc', 'G_GROUP', symmetric=False, group_size=group)
+    g = torch.Generator().manual_seed(bits)
+    parts = []
+    for n in (1, 4, 9):
+        x = (torch.randn(2, 3, n, 64, generator=g) + 0.3).bfloat16()
+        parts.append(x)
+        got = gpu.use_var_q(x.to(dev))
+        cat = torch.cat(parts, dim=2)
+        q, s, z = O.quant_groupwise(cat, group, bits, True)
+        assert torch.equal(got.cpu(), O.dequant_groupwise(q, s, z, group))
+        assert torch.equal(gpu.cached_scale.cpu(), s) and torch.equal(gpu.cached_zp.cpu(), z)
+        assert torch.equal(gpu.cached_item.cpu(), O.pack_last_dim(q, bits)[0])
+
+
+def test_per_head_extension_single_call(dev):
+    note('VAR_Q G_HEAD')
+    x = O.synth_kv((2, 16, 100, 64), seed=5)
+    gpu = VAR_Q(8, 'BHLc', 'G_HEAD')
+    got = gpu.use_var_q(x.to(dev))
+    s = O.scale_sym(x, (0, 2, 3), 8)
+    assert torch.equal(got.cpu(), O.dequant_sym(O.codes_sym(x, s, 8), s))
+    assert gpu.scale.shape == (1, 16, 1, 1)

@@ -98,8 +98,8 @@ template <> struct KCodec<8> {
     float f[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      f[j] = (float)__builtin_amdgcn_sbfe((int)w0, 8 * j, 8);
-      f[4 + j] = (float)__builtin_amdgcn_sbfe((int)w1, 8 * j, 8);
+      f[j] = (float)(int)__builtin_amdgcn_sbfe((int)w0, 8 * j, 8);
+      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe((int)w1, 8 * j, 8);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = (f2u(f[2 * j]) >> 16) | (f2u(f[2 * j + 1]) & 0xffff0000u);
@@ -124,7 +124,7 @@ template <> struct VCodec<2> {
   __device__ static __forceinline__ void codes(const u32 *lds_row, int oct, float (&f)[8]) {
     const int w = (int)(lds_row[oct >> 1] >> ((oct & 1) * 16));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = (float)__builtin_amdgcn_sbfe(w, 2 * j, 2);
+    for (int j = 0; j < 8; ++j) f[j] = (float)(int)__builtin_amdgcn_sbfe(w, 2 * j, 2);
   }
 };
 template <> struct VCodec<8> {
@@ -133,8 +133,8 @@ template <> struct VCodec<8> {
     const int w0 = (int)lds_row[2 * oct], w1 = (int)lds_row[2 * oct + 1];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      f[j] = (float)__builtin_amdgcn_sbfe(w0, 8 * j, 8);
-      f[4 + j] = (float)__builtin_amdgcn_sbfe(w1, 8 * j, 8);
+      f[j] = (float)(int)__builtin_amdgcn_sbfe(w0, 8 * j, 8);
+      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe(w1, 8 * j, 8);
     }
   }
 };
@@ -398,17 +398,17 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
       }
 #pragma unroll
       for (int s = 0; s < NSV; ++s) {
-        float ps[16];
+        // The zero-point term must see the same bf16-rounded weights as the
+        // MFMA does, or the constant offset of the raw codes stops cancelling.
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i2 = 0; i2 < 8; ++i2) {
+          const int i = 2 * i2;
           const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          ps[i] = pv[i] * lds_sv[s][key];
-          r_run[s] += ps[i] * lds_zv[s][key];
+          const u32 pk = pack_bf16_rne(pv[i] * lds_sv[s][key], pv[i + 1] * lds_sv[s][key + 1]);
+          pop[s][kb * 2 + (i >> 3)][(i & 7) >> 1] = pk;
+          r_run[s] += u2f(pk << 16) * lds_zv[s][key];
+          r_run[s] += u2f(pk & 0xffff0000u) * lds_zv[s][key + 1];
         }
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) pop[s][kb * 2 + c][j] = pack_bf16_rne(ps[c * 8 + 2 * j], ps[c * 8 + 2 * j + 1]);
       }
     }
 

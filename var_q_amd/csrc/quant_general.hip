@@ -377,12 +377,12 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   VARQ_CHECK_ARG(s[0] >= 0 && s[1] >= 0 && s[2] >= 0 && s[3] > 0 && s[3] <= (1 << 20), "quant_pack: bad shape");
   VARQ_CHECK_ARG(x_dtype >= 0 && x_dtype <= 2, "quant_pack: bad dtype %d", x_dtype);
   VARQ_CHECK_ARG(reduce_mask >= 0 && reduce_mask < 16, "quant_pack: bad reduce mask");
-  VARQ_CHECK_ARG(words || codes, "quant_pack: no output requested");
   VARQ_CHECK_ARG(bits > 1 && bits <= 8, "quant_pack: bits must be in 2..8 (got %d)", bits);
   VARQ_CHECK_ARG(!words || bits == 2 || bits == 4 || bits == 8, "quant_pack: packing implements 2/4/8 bits only (got %d)", bits);
-  VARQ_CHECK_ARG(scale && (!asym || zp), "quant_pack: scale/zp output missing");
   const int64_t rows = s[0] * s[1] * s[2];
   if (rows == 0) return VARQ_OK;
+  VARQ_CHECK_ARG(words || codes, "quant_pack: no output requested");
+  VARQ_CHECK_ARG(scale && (!asym || zp), "quant_pack: scale/zp output missing");
   VARQ_CHECK_ARG(x && workspace, "quant_pack: null pointer");
   const int64_t ng = count_groups(s, reduce_mask);
   if (workspace_bytes < (size_t)ng * 2 * sizeof(u32))

@@ -175,8 +175,8 @@ int launch_dt(const RowsParams &p, int bits, int asym, int lpg, dim3 grid, hipSt
 extern "C" int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, int c, int group, int bits,
                                     int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
                                     int32_t *words, float *scale, float *zp, void *stream) {
-  VARQ_CHECK_ARG(x && words && scale, "quant_pack_rows: null pointer");
-  VARQ_CHECK_ARG(!asym || zp, "quant_pack_rows: asym needs zp output");
+  VARQ_CHECK_ARG(n_rows == 0 || (x && words && scale), "quant_pack_rows: null pointer");
+  VARQ_CHECK_ARG(n_rows == 0 || !asym || zp, "quant_pack_rows: asym needs zp output");
   VARQ_CHECK_ARG(bits == 2 || bits == 4 || bits == 8, "quant_pack_rows: bits must be 2, 4 or 8 (got %d)", bits);
   VARQ_CHECK_ARG(x_dtype >= 0 && x_dtype <= 2, "quant_pack_rows: bad dtype %d", x_dtype);
   VARQ_CHECK_ARG(n_rows >= 0 && c > 0, "quant_pack_rows: bad shape");
