@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the VAR-Q hot path on one MI355X.
+
+One step = one pass over BASELINE config 4 (Infinity-2B shape): quantize+pack K
+and V [2,16,10521,128] bf16 to INT4 group-128 asymmetric, then fused dequant
+attention of the final scale's 4096 queries over all 10521 packed keys.  Inputs
+are resident in HBM before the timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, 'oracle')):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
+
+B, H, L, D = 2, 16, 10521, 128
+LQ = 4096
+BITS, GROUP = 4, 128
+NBUF = 4   # distinct input sets cycled through, 4*2*86 MB > the 256 MB Infinity Cache
+
+
+def algorithmic_bytes():
+    n = B * H * L * D
+    groups = B * H * L * (D // GROUP)
+    quant_pack = n * 2 + n * BITS // 8 + groups * 8            # per tensor: bf16 in, packed out, scale+zp out
+    kv_read = 2 * (n * BITS // 8 + groups * 8)                  # packed K and V with scales/zps, read once
+    attn_flops = 4 * B * H * LQ * L * D
+    return quant_pack, kv_read, attn_flops
+
+
+def cpu_baseline(torch, O, k0, v0, q0, threads):
+    """The CPU oracle timed on this host: full-size quantize+pack of K and V,
+    unpack+dequant of both, and bf16 SDPA on a 512-query sample (scaled x8)."""
+    torch.set_num_threads(threads)
+    t0 = time.perf_counter()
+    kq, ks, kz = O.quant_groupwise(k0, GROUP, BITS, True)
+    kw, kmeta = O.pack_last_dim(kq, BITS)
+    t1 = time.perf_counter()
+    vq, vs, vz = O.quant_groupwise(v0, GROUP, BITS, True)
+    vw, vmeta = O.pack_last_dim(vq, BITS)
+    t2 = time.perf_counter()
+    kd = O.dequant_groupwise(O.unpack_last_dim(kw, kmeta), ks, kz, GROUP)
+    vd = O.dequant_groupwise(O.unpack_last_dim(vw, vmeta), vs, vz, GROUP)
+    t3 = time.perf_counter()
+    nq = 512
+    ref = O.attention_ref(q0[:, :, :nq], kd, vd, 1.0 / math.sqrt(D))
+    t4 = time.perf_counter()
+    t_quant = (t2 - t0) / 2
+    t_attn = (t3 - t2) + (t4 - t3) * (LQ / nq)
+    return {'kw': kw, 'ks': ks, 'kz': kz, 'vw': vw, 'ref': ref, 'nq': nq,
+            't_quant_pack_per_tensor_s': t_quant, 't_unpack_dequant_s': t3 - t2, 't_sdpa_sample_s': t4 - t3,
+            't_attn_equiv_s': t_attn}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=40)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py measures one GPU: this path has no collectives and is not sharded; '
+              'run with --gpus 1 (got --gpus %d)' % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import varq_oracle as O
+    from var_q_amd import _lib, ops
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    _lib.load()   # raises if the HIP library is missing: no fallback
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+
+    quant_bytes, kv_bytes, attn_flops = algorithmic_bytes()
+    scale = 1.0 / math.sqrt(D)
+
+    # ---- synthetic inputs (seeds as for the parity tests) --------------------
+    k0 = O.synth_kv((B, H, L, D), 1004, 'student4', 0.01, 20.0, torch.bfloat16, outlier_seed=4004)
+    v0 = O.synth_kv((B, H, L, D), 2004, 'student4', 0.01, 20.0, torch.bfloat16, outlier_seed=4004)
+    q0 = torch.randn(B, H, LQ, D, generator=torch.Generator().manual_seed(3004)).bfloat16()
+    ks_in, vs_in = [k0.to(dev)], [v0.to(dev)]
+    for i in range(1, NBUF):   # further sets: same distribution, different memory and values
+        ks_in.append(torch.roll(ks_in[0], shifts=i * 977, dims=2).contiguous())
+        vs_in.append(torch.roll(vs_in[0], shifts=i * 977, dims=2).contiguous())
+    q = q0.to(dev)
+
+    W = D * BITS // 32
+    mk = lambda last, dt: torch.empty((B, H, L, last), dtype=dt, device=dev)
+    outs = [dict(kw=mk(W, torch.int32), ks=mk(1, torch.float32), kz=mk(1, torch.float32),
+                 vw=mk(W, torch.int32), vs=mk(1, torch.float32), vz=mk(1, torch.float32)) for _ in range(NBUF)]
+    o = torch.empty_like(q)
+    rowmap = [1, 1, B * H * L, 0, 0, 1, 0, -1]
+
+    def step(i, ev=None):
+        s, t = i % NBUF, outs[i % NBUF]
+        if ev: ev[0].record()
+        ops.quant_pack_rows_into(ks_in[s], GROUP, BITS, True, 1e-12, t['kw'], t['ks'], t['kz'], rowmap)
+        if ev: ev[1].record()
+        ops.quant_pack_rows_into(vs_in[s], GROUP, BITS, True, 1e-12, t['vw'], t['vs'], t['vz'], rowmap)
+        if ev: ev[2].record()
+        ops.fused_attn(q, t['kw'], t['ks'], t['kz'], t['vw'], t['vs'], t['vz'], BITS, BITS, L, scale, out=o)
+        if ev: ev[3].record()
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    t_qk = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps * 1e-3
+    t_qv = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps * 1e-3
+    t_at = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps * 1e-3
+    t_quant = 0.5 * (t_qk + t_qv)
+
+    # ---- CPU baseline + parity of the timed results against it ------------------
+    cpu = None
+    checked = None
+    if not args.no_cpu:
+        threads = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
+        step(0)
+        torch.cuda.synchronize()
+        c = cpu_baseline(torch, O, k0, v0, q0, threads)
+        t = outs[0]
+        words_ok = bool(torch.equal(t['kw'].cpu(), c['kw']) and torch.equal(t['vw'].cpu(), c['vw'])
+                        and torch.equal(t['ks'].cpu(), c['ks']) and torch.equal(t['kz'].cpu(), c['kz']))
+        got, ref = o[:, :, :c['nq']].double().cpu(), c['ref'].double()
+        cosine = float(torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0))
+        checked = {'packed_words_scales_zps_bit_exact': words_ok, 'attn_cosine_vs_oracle': round(cosine, 6)}
+        if not words_ok or cosine < 0.9995:
+            print('bench.py: GPU results differ from the oracle: %r' % checked, file=sys.stderr)
+            sys.exit(1)
+        cpu = {
+            'value': round(kv_bytes / c['t_attn_equiv_s'] / 1e9, 4), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
+            'sample': ('torch-CPU oracle on this host: full-size INT4 g128 quantize+pack of K and V '
+                       '(%.3f s per tensor = %.2f GB/s), unpack+dequant of both (%.3f s), bf16 SDPA on 512 of the '
+                       '4096 queries (%.3f s, scaled x8); value = packed-KV bytes / (dequant + scaled SDPA)'
+                       % (c['t_quant_pack_per_tensor_s'], quant_bytes / c['t_quant_pack_per_tensor_s'] / 1e9,
+                          c['t_unpack_dequant_s'], c['t_sdpa_sample_s'])),
+            'pack_GBps': round(quant_bytes / c['t_quant_pack_per_tensor_s'] / 1e9, 3),
+        }
+
+    attn_tflops = attn_flops / t_at / 1e12
+    kv_gbps = kv_bytes / t_at / 1e9
+    pack_gbps = quant_bytes / t_quant / 1e9
+    traffic = None
+    tf = os.path.join(ROOT, 'profiles', 'traffic.json')   # HBM bytes per launch from the rocprofv3 --pmc runs
+    if os.path.exists(tf):
+        try:
+            traffic = json.load(open(tf))
+        except Exception:
+            traffic = None
+    line = {
+        'metric': 'fused dequant-attn KV-read GB/s (%HBM peak) + pack GB/s, Infinity-2B shape',
+        'value': round(kv_gbps, 3), 'unit': 'GB/s',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16 MFMA over int4 codes, fp32 scales', 'data': 'synthetic',
+        'config': {'workload': 'config 4: Infinity-2B KV [B=2,H=16,L=10521,D=128] bf16 -> INT4 group-128 asymmetric '
+                               'quantize+pack of K and V, then fused dequant attention of the final 4096 queries',
+                   'B': B, 'H': H, 'L': L, 'D': D, 'Lq': LQ, 'bits': BITS, 'group': GROUP, 'input_sets_cycled': NBUF},
+        'attn_kv_read_frac_hbm_peak': round(kv_gbps / HBM_PEAK_GBPS, 5),
+        'attn_ms': round(t_at * 1e3, 4), 'attn_TFLOPs': round(attn_tflops, 2),
+        'attn_query_tokens_per_s': round(B * LQ / t_at, 1),
+        'pack_GBps': round(pack_gbps, 2), 'pack_frac_hbm_peak': round(pack_gbps / HBM_PEAK_GBPS, 4),
+        'pack_us_per_tensor': round(t_quant * 1e6, 2), 'pack_tokens_per_s': round(B * L / t_quant, 1),
+        'roofline': {'kernel': 'fused_attn_kernel<128,4,128,128>', 'bound': 'mfma', 'achieved': round(attn_tflops, 2),
+                     'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s', 'frac': round(attn_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                     'traffic': None if not traffic else traffic.get('fused_attn')},
+        'roofline_pack': {'kernel': 'quant_pack_rows_kernel<bf16,4,asym,16>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
+                          'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(pack_gbps / HBM_PEAK_GBPS, 4),
+                          'traffic': None if not traffic else traffic.get('quant_pack_rows')},
+        'cpu_baseline': cpu, 'checked_against_oracle': checked,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == '__main__':
+    main()
