@@ -12,6 +12,7 @@
 // the min/max reduction is a DPP butterfly inside the wavefront and never
 // touches LDS.  A block covers octets of one (i0,i1) pair of the row map so
 // that the output row offset is block-uniform.
+#include <type_traits>
 #include "varq_common.h"
 
 namespace {
@@ -149,14 +150,220 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   }
 }
 
+// ---- wide variant: one lane owns 4 octets (32 channels) of one group ---------
+// Used for groups of 32 channels and more.  The per-group work (one IEEE fp32
+// division for the scale, one fp64 reciprocal, the cross-lane reduce) is
+// amortized over 32 elements instead of 8.  A group is LPG4 = group/32 adjacent
+// lanes; lane j owns octets j, j+LPG4, j+2*LPG4, j+3*LPG4 of its group.
+//
+// HBM side: every global load and (in the common dense-output case) every
+// global store instruction of a wavefront touches 1 KiB of contiguous memory.
+// The change of layout between "contiguous per instruction" and "32 channels of
+// one group per lane" goes through a 4 KiB wave-private LDS window, so there is
+// no workgroup barrier anywhere.
+//
+// Rounding: x/s is needed exactly as an IEEE fp32 division rounds it.  The fp64
+// product x * RN64(1/s) is within 2^-52 (relative) of the true quotient, and a
+// quotient of two fp32 numbers is never closer than 2^-49 (relative) to a point
+// where rounding to fp32 changes (such a point has 25 significant bits; x - m*s
+// is a non-zero multiple of ulp(m)*ulp(s)).  Narrowing the product to fp32
+// therefore yields the correctly rounded quotient for every finite input,
+// denormals included, at 3 full-rate instructions instead of a ~11-instruction
+// division sequence.
+template <int DT, int BITS, bool ASYM, int LPG4, bool DENSE>
+__global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
+  __shared__ Raw8<DT> lds_stage[4][256];   // per wave: 256 octets in, then packed words out
+
+  const int64_t i0 = blockIdx.z, i1 = blockIdx.y;
+  const int64_t pair = i0 * p.map.n1 + i1;
+  int64_t s0 = i0, s1 = i1;
+  if (p.map.slot_dim == 0) s0 = p.slot[i0];
+  if (p.map.slot_dim == 1) s1 = p.slot[i1];
+  if (s0 < 0 || s1 < 0) return;
+  const int64_t out_base = s0 * p.map.os0 + s1 * p.map.os1 + p.map.off;
+  const int64_t pair_elem0 = pair * p.octets_per_pair * 8;
+
+  const int n_oct = (int)p.octets_per_pair;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  Raw8<DT> *stage = lds_stage[wv];
+  constexpr float kMin = (float)QRange<BITS>::kMin, kMax = (float)QRange<BITS>::kMax;
+  const int w0 = blockIdx.x * 1024 + wv * 256;       // first octet of this wave's window, inside the pair
+
+  // 1 KiB contiguous per load instruction
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    int o = w0 + k * 64 + lane;
+    o = o < n_oct ? o : 0;                            // past the end: re-read octet 0, never stored
+    Raw8<DT> r;
+    r.load(p.x, pair_elem0 + (int64_t)o * 8);
+    stage[k * 64 + lane] = r;
+  }
+  __builtin_amdgcn_wave_barrier();
+
+  // lane-owned octets inside the wave window
+  const int j = lane & (LPG4 - 1);
+  const int loc0 = ((lane - j) << 2) + j;
+  float v[4][8];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) stage[loc0 + k * LPG4].widen(v[k]);
+
+  float mn = 0.f, mx;
+  if (ASYM) {
+    mn = v[0][0]; mx = v[0][0];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { mn = fminf(mn, v[k][e]); mx = fmaxf(mx, v[k][e]); }
+    mn = group_allreduce<LPG4, false>(mn);
+    mx = group_allreduce<LPG4, true>(mx);
+  } else {
+    mx = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[k][e]));
+    mx = group_allreduce<LPG4, true>(mx);
+  }
+
+  float s, zp = 0.f;
+  if (ASYM) s = fmaxf((mx - mn) / (float)QRange<BITS>::kLevels, p.eps);
+  else s = fmaxf(mx / kMax, p.eps);
+  const double rinv = 1.0 / (double)s;
+  if (ASYM) zp = kMin - rintf((float)((double)mn * rinv));
+
+  // clamp(t + zp, qmin, qmax) as clamp(t, qmin - zp, qmax - zp) + zp, with the
+  // final add also planting the integer in the low mantissa bits (1.5 * 2^23
+  // trick): exact whenever |zp| <= 2^22.  Larger zero-points (data offset by
+  // millions of quantization steps) take the literal sequence.
+  const bool big_zp = ASYM && !(fabsf(zp) <= 0x1p22f);
+  const float lo = kMin - zp, hi = kMax - zp, magic = zp + 12582912.f;
+  u32 w[4][2];
+  auto quantize_all = [&](auto literal) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      u32 acc = 0;
+      w[k][0] = 0; w[k][1] = 0;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float t = rintf((float)((double)v[k][e] * rinv));
+        u32 q;
+        if (decltype(literal)::value) q = (u32)(int)__builtin_amdgcn_fmed3f(ASYM ? t + zp : t, kMin, kMax);
+        else q = f2u(__builtin_amdgcn_fmed3f(t, lo, hi) + magic);
+        acc = __builtin_amdgcn_alignbit(q, acc, BITS);
+        if (BITS == 8 && e == 3) { w[k][0] = acc; acc = 0; }
+      }
+      if (BITS == 8) w[k][1] = acc;
+      else if (BITS == 4) w[k][0] = acc;
+      else w[k][0] = acc >> 16;
+    }
+  };
+  if (__builtin_amdgcn_ballot_w64(big_zp) != 0) quantize_all(std::true_type{});   // wave-uniform, rare
+  else quantize_all(std::false_type{});
+  if (BITS == 2 && LPG4 > 1) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      u32 other = (u32)__builtin_amdgcn_update_dpp(0, (int)w[k][0], 0xB1, 0xf, 0xf, false);
+      w[k][0] |= other << 16;
+    }
+  }
+
+  const int oct0 = w0 + loc0;                         // first owned octet, inside the pair
+  const bool live = oct0 < n_oct;                     // groups never straddle the end
+
+  if (DENSE) {
+    // output rows of the pair are consecutive: word, scale and zp indices follow
+    // the pair-local octet index directly
+    if (BITS == 4) {
+      // packed words back to global order through the same window, 16 B per lane
+      typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+      u32 *wstage = reinterpret_cast<u32 *>(stage);
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int k = 0; k < 4; ++k) wstage[loc0 + k * LPG4] = w[k][0];
+      __builtin_amdgcn_wave_barrier();
+      const u32x4 out4 = reinterpret_cast<const u32x4 *>(wstage)[lane];
+      const int o = w0 + 4 * lane;                    // octet == word index for 4-bit codes
+      if (o < n_oct)
+        __builtin_nontemporal_store(out4, reinterpret_cast<u32x4 *>(p.words + out_base * p.c8 + o));
+    } else if (live) {
+      const int64_t wbase = out_base * p.c8 + oct0;   // in octets
+      if (BITS == 8) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          *reinterpret_cast<uint2 *>(p.words + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
+      } else if (LPG4 == 1) {
+        *reinterpret_cast<uint2 *>(p.words + (wbase >> 1)) =
+            make_uint2(w[0][0] | (w[1][0] << 16), w[2][0] | (w[3][0] << 16));
+      } else if ((j & 1) == 0) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) p.words[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
+      }
+    }
+    if (live && j == 0) {
+      const int64_t g = out_base * p.nseg + oct0 / (4 * LPG4);
+      p.scale[g] = s;
+      if (ASYM) p.zp[g] = zp;
+    }
+    return;
+  }
+
+  if (!live) return;
+  int i2, col;
+  if (p.c8_shift >= 0) { i2 = oct0 >> p.c8_shift; col = oct0 & (p.c8 - 1); }
+  else { i2 = oct0 / p.c8; col = oct0 - i2 * p.c8; }
+  if (p.map.slot_dim == 2) i2 = p.slot[i2];
+  if (i2 < 0) return;
+  const int64_t out_row = out_base + (int64_t)i2 * p.map.os2;
+  const int64_t wbase = out_row * p.c8 + col;            // in octets
+  if (BITS == 8) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      *reinterpret_cast<uint2 *>(p.words + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
+  } else if (BITS == 4) {
+    if (LPG4 == 1) {
+      *reinterpret_cast<uint4 *>(p.words + wbase) = make_uint4(w[0][0], w[1][0], w[2][0], w[3][0]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) p.words[wbase + k * LPG4] = (int32_t)w[k][0];
+    }
+  } else {
+    if (LPG4 == 1) {
+      *reinterpret_cast<uint2 *>(p.words + (wbase >> 1)) =
+          make_uint2(w[0][0] | (w[1][0] << 16), w[2][0] | (w[3][0] << 16));
+    } else if ((j & 1) == 0) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) p.words[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
+    }
+  }
+  if (j == 0) {
+    const int64_t g = out_row * p.nseg + col / (4 * LPG4);
+    p.scale[g] = s;
+    if (ASYM) p.zp[g] = zp;
+  }
+}
+
 template <int DT, int BITS, bool ASYM>
 int launch_lpg(const RowsParams &p, int lpg, dim3 grid, hipStream_t st) {
+  if (lpg >= 4) {   // groups of >= 32 channels: 4 octets per lane, 1024 octets per workgroup
+    dim3 g32((unsigned)((p.octets_per_pair + 1023) / 1024), grid.y, grid.z);
+    const bool dense = (p.map.os2 == 1) && (p.map.slot_dim != 2);
+    switch (lpg / 4) {
+#define VARQ_CASE32(L)                                                                                            \
+  case L:                                                                                                         \
+    if (dense) hipLaunchKernelGGL((quant_pack_rows32_kernel<DT, BITS, ASYM, L, true>), g32, dim3(256), 0, st, p); \
+    else hipLaunchKernelGGL((quant_pack_rows32_kernel<DT, BITS, ASYM, L, false>), g32, dim3(256), 0, st, p);      \
+    return 0;
+      VARQ_CASE32(1) VARQ_CASE32(2) VARQ_CASE32(4) VARQ_CASE32(8) VARQ_CASE32(16)
+#undef VARQ_CASE32
+    }
+    return -1;
+  }
   switch (lpg) {
 #define VARQ_CASE(L)                                                                     \
   case L:                                                                                \
     hipLaunchKernelGGL((quant_pack_rows_kernel<DT, BITS, ASYM, L>), grid, dim3(256), 0, st, p); \
     return 0;
-    VARQ_CASE(1) VARQ_CASE(2) VARQ_CASE(4) VARQ_CASE(8) VARQ_CASE(16) VARQ_CASE(32) VARQ_CASE(64)
+    VARQ_CASE(1) VARQ_CASE(2)
 #undef VARQ_CASE
   }
   return -1;
@@ -183,7 +390,7 @@ extern "C" int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, 
   VARQ_CHECK_ARG(c % 8 == 0 && (c * bits) % 32 == 0, "quant_pack_rows: c=%d must be a multiple of 8 and fill whole words", c);
   VARQ_CHECK_ARG(group > 0 && group % 8 == 0 && c % group == 0, "quant_pack_rows: group=%d must be a multiple of 8 dividing c=%d", group, c);
   const int lpg = group / 8;
-  VARQ_CHECK_ARG(varq_log2_exact(lpg) >= 0 && lpg <= 64, "quant_pack_rows: group/8=%d must be a power of two <= 64", lpg);
+  VARQ_CHECK_ARG(varq_log2_exact(lpg) >= 0 && lpg <= 64, "quant_pack_rows: group/8=%d must be a power of two <= 64 (group <= 512)", lpg);
   RowMap m = varq_rowmap_from_host(host_rowmap, n_rows);
   VARQ_CHECK_ARG(m.n0 >= 0 && m.n1 >= 0 && m.n2 >= 0 && m.n0 * m.n1 * m.n2 == n_rows, "quant_pack_rows: row map does not cover n_rows");
   VARQ_CHECK_ARG(m.slot_dim >= -1 && m.slot_dim <= 2 && (m.slot_dim < 0 || slot), "quant_pack_rows: slot table missing");

@@ -105,6 +105,44 @@ template <> struct In8<VARQ_F16> {
   }
 };
 
+// Raw 8-element loads (no conversion) so that a kernel can issue the next
+// tile's loads before converting the current one.  Streaming data: marked
+// non-temporal, it is read exactly once.
+typedef float varq_f32x4 __attribute__((ext_vector_type(4)));
+template <int DT> struct Raw8;
+template <> struct Raw8<VARQ_F32> {
+  varq_f32x4 a, b;
+  __device__ __forceinline__ void load(const void *base, int64_t elem) {
+    const varq_f32x4 *p = reinterpret_cast<const varq_f32x4 *>(reinterpret_cast<const float *>(base) + elem);
+    a = __builtin_nontemporal_load(p);
+    b = __builtin_nontemporal_load(p + 1);
+  }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+  }
+};
+template <> struct Raw8<VARQ_BF16> {
+  varq_bf16x8 a;
+  __device__ __forceinline__ void load(const void *base, int64_t elem) {
+    a = __builtin_nontemporal_load(reinterpret_cast<const varq_bf16x8 *>(reinterpret_cast<const __bf16 *>(base) + elem));
+  }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+  }
+};
+template <> struct Raw8<VARQ_F16> {
+  varq_f16x8 a;
+  __device__ __forceinline__ void load(const void *base, int64_t elem) {
+    a = __builtin_nontemporal_load(reinterpret_cast<const varq_f16x8 *>(reinterpret_cast<const _Float16 *>(base) + elem));
+  }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+  }
+};
+
 // fp32 -> output dtype, round to nearest even (what tensor.to(dtype) does).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
   u32 u = f2u(f);
