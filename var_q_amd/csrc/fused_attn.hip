@@ -14,19 +14,27 @@
 //    S^T = K Q^T and O^T = V^T P^T, so that a lane owns one query column: row
 //    max/sum are per-lane (one cross-half exchange per tile) and the S^T
 //    accumulator registers are directly the B operand of the second MFMA.
-//  * Codes are never scaled before the MFMA.  They are widened to small exact
-//    bf16 integers; the affine map is applied in fp32 to the 32x32 results:
-//       S[l,q] = sum_seg  ks[l,seg] * (A_seg[l,q] - kzp'[l,seg] * qsum_seg[q])
-//       O[q,:] = sum_l (p[l,q] * vs[l,seg]) * vraw[l,:]  -  sum_l p' * vzp'
-//    which is cheaper than dequantizing every element and loses nothing to
-//    bf16 rounding of K/V.
-//  * K tile: packed words HBM -> LDS, expanded in registers by each wavefront
-//    straight into MFMA A operands (8 codes of one word = one lane's operand).
-//  * V tile: packed words HBM -> LDS -> expanded once per workgroup and written
-//    transposed (V^T, bf16) to LDS, because the PV contraction runs over keys.
+//  * The MFMA operands are exact small numbers derived from the codes, never
+//    scaled or rounded; scales are applied in fp32 to the 32x32 results:
+//       O[q,:] = sum_l (p[l,q] * vs[l]) * (vq - vzp)[l,:]
+//    (vq - vzp) is an integer that bf16 holds exactly when |vzp| <= 240.  Larger
+//    V zero-points (data offset by hundreds of quantization steps) are split
+//    zp = zp_c + zp_r; the remainder goes through a correction term on tiles
+//    that have one.
+//  * Packed K and V tiles go HBM -> LDS as they are (16-byte loads, prefetched
+//    one tile ahead).  K words are widened in registers by each wavefront
+//    straight into MFMA A operands, interleaved with the MFMAs (8 codes of one
+//    word = one lane's operand; the codes land in the mantissa of a bf16 1.x, an
+//    affine image of the code that the fp32 epilogue undoes together with the
+//    zero-point: S = ks*(kMul*A - (kzp+kOff)*sum(q))).  V is widened once per
+//    workgroup with its zero-point folded in and written transposed to LDS
+//    (the PV contraction runs over keys).
 //  * Key rows are fed to the first MFMA in a permuted order chosen so that each
 //    lane's accumulator registers hold 8 consecutive keys per 16-key chunk,
 //    which makes the V^T operand a single 16-byte LDS read.
+//  * Online softmax in the log2 domain against a reference that is only moved
+//    when some row's maximum exceeds it by 2^16: the common tile needs no
+//    subtraction and no rescale of the output accumulators.
 #include "varq_common.h"
 
 namespace {
@@ -38,6 +46,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(u32)))) u32 u32x4_t;
 constexpr int BM = 128;  // queries per workgroup (32 per wavefront)
 constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
 
 struct AttnParams {
   const __bf16 *q;
@@ -51,67 +60,14 @@ struct AttnParams {
   float scale_log2e;
 };
 
-// ---- code widening ---------------------------------------------------------
-// K side: 8 codes of one octet -> 8 bf16 (4 dwords) holding code*kMul'+const,
-// i.e. code = kMul * raw - kOff.  `slot_d(j)` is the channel (within the octet)
-// that lands in operand slot j; the Q operand is gathered in the same order.
-template <int BITS> struct KCodec;
-
-template <> struct KCodec<4> {
-  // nibble u = code+8 goes to the top 4 mantissa bits of bf16 1.0:
-  // raw = 1 + u/16 = (code + 24)/16.
-  static constexpr float kMul = 16.f, kOff = 24.f;
-  __device__ static __forceinline__ int slot_d(int j) { return (j >> 1) + 4 * (j & 1); }
-  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32 (&o)[4]) {
-    const u32 w = lds_row[oct] ^ 0x88888888u;
-    constexpr u32 M = 0x00780078u, B = 0x3f803f80u;
-    o[0] = ((w << 3) & M) | B;   // nibbles 0,4
-    o[1] = ((w >> 1) & M) | B;   // 1,5
-    o[2] = ((w >> 5) & M) | B;   // 2,6
-    o[3] = ((w >> 9) & M) | B;   // 3,7
-  }
-};
-
-template <> struct KCodec<2> {
-  // field u = code+2 goes to the top 2 mantissa bits: raw = 1 + u/4 = (code + 6)/4.
-  static constexpr float kMul = 4.f, kOff = 6.f;
-  // an octet is half a word: fields 0..7 of the half; dword m holds fields (m, m+4)
-  __device__ static __forceinline__ int slot_d(int j) { return (j >> 1) + 4 * (j & 1); }
-  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32 (&o)[4]) {
-    const u32 w = ((lds_row[oct >> 1] >> ((oct & 1) * 16)) & 0xffffu) ^ 0xaaaau;
-    // fields m (bits 2m) and m+4 (bits 2m+8): move to bits 5..6 and 21..22
-    const u32 t = (w & 0xffu) | ((w & 0xff00u) << 8);  // low byte: fields 0-3, byte 2: fields 4-7
-    constexpr u32 M = 0x00600060u, B = 0x3f803f80u;
-    o[0] = ((t << 5) & M) | B;
-    o[1] = ((t << 3) & M) | B;
-    o[2] = ((t << 1) & M) | B;
-    o[3] = ((t >> 1) & M) | B;
-  }
-};
-
-template <> struct KCodec<8> {
-  // bytes are widened through fp32 (exact), raw = code.
-  static constexpr float kMul = 1.f, kOff = 0.f;
-  __device__ static __forceinline__ int slot_d(int j) { return j; }
-  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32 (&o)[4]) {
-    const u32 w0 = lds_row[2 * oct], w1 = lds_row[2 * oct + 1];
-    float f[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f[j] = (float)(int)__builtin_amdgcn_sbfe((int)w0, 8 * j, 8);
-      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe((int)w1, 8 * j, 8);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) o[j] = (f2u(f[2 * j]) >> 16) | (f2u(f[2 * j + 1]) & 0xffff0000u);
-  }
-};
-
-// V side: the 8 codes of octet `oct` of one key as exact floats code + kOff.
-template <int BITS> struct VCodec;
-template <> struct VCodec<4> {
-  static constexpr float kOff = 8.f;
-  __device__ static __forceinline__ void codes(const u32 *lds_row, int oct, float (&f)[8]) {
-    const u32 w = lds_row[oct] ^ 0x88888888u;
+// The 8 codes of octet `oct` of one packed row as exact floats code + kOff, and
+// the largest |zp| that still folds exactly into bf16 (|code - zp| <= 256).
+template <int BITS> struct Codec;
+template <> struct Codec<4> {
+  static constexpr float kOff = 8.f, kZmax = 240.f;
+  static constexpr u32 kStageXor = 0x88888888u;   // applied once when the tile is staged: nibble -> code + 8
+  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
+    const u32 w = row[oct];
     const u32 e = w & 0x0f0f0f0fu, o = (w >> 4) & 0x0f0f0f0fu;
     f[0] = (float)(e & 0xffu); f[1] = (float)(o & 0xffu);
     f[2] = (float)((e >> 8) & 0xffu); f[3] = (float)((o >> 8) & 0xffu);
@@ -119,18 +75,20 @@ template <> struct VCodec<4> {
     f[6] = (float)(e >> 24); f[7] = (float)(o >> 24);
   }
 };
-template <> struct VCodec<2> {
-  static constexpr float kOff = 0.f;
-  __device__ static __forceinline__ void codes(const u32 *lds_row, int oct, float (&f)[8]) {
-    const int w = (int)(lds_row[oct >> 1] >> ((oct & 1) * 16));
+template <> struct Codec<2> {
+  static constexpr float kOff = 0.f, kZmax = 250.f;
+  static constexpr u32 kStageXor = 0u;
+  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
+    const int w = (int)(row[oct >> 1] >> ((oct & 1) * 16));
 #pragma unroll
     for (int j = 0; j < 8; ++j) f[j] = (float)(int)__builtin_amdgcn_sbfe(w, 2 * j, 2);
   }
 };
-template <> struct VCodec<8> {
-  static constexpr float kOff = 0.f;
-  __device__ static __forceinline__ void codes(const u32 *lds_row, int oct, float (&f)[8]) {
-    const int w0 = (int)lds_row[2 * oct], w1 = (int)lds_row[2 * oct + 1];
+template <> struct Codec<8> {
+  static constexpr float kOff = 0.f, kZmax = 127.f;
+  static constexpr u32 kStageXor = 0u;
+  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
+    const int w0 = (int)row[2 * oct], w1 = (int)row[2 * oct + 1];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f[j] = (float)(int)__builtin_amdgcn_sbfe(w0, 8 * j, 8);
@@ -140,7 +98,7 @@ template <> struct VCodec<8> {
 };
 
 __device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
-  return (f2u(lo) >> 16) | (f2u(hi) & 0xffff0000u);
+  return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);   // {hi[31:16], lo[31:16]} in one v_perm_b32
 }
 __device__ __forceinline__ u32 pack_bf16_rne(float lo, float hi) {
   typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
@@ -155,6 +113,67 @@ __device__ __forceinline__ u32 pack_bf16_rne(float lo, float hi) {
 // holds key 16*(i/8) + 8*h + i%8.
 __device__ __forceinline__ int kperm(int r) { return (r & 0x13) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
+// ---- code widening ---------------------------------------------------------
+// K side: 8 codes of one octet -> 8 bf16 (4 dwords) holding code*kMul'+const,
+// i.e. code = kMul * raw - kOff.  `slot_d(j)` is the channel (within the octet)
+// that lands in operand slot j; the Q operand is gathered in the same order.
+template <int BITS> struct KCodec;
+
+template <> struct KCodec<4> {
+  // nibble u = code+8 goes to the top 4 mantissa bits of bf16 1.0:
+  // raw = 1 + u/16 = (code + 24)/16.
+  static constexpr float kMul = 16.f, kOff = 24.f;
+  __device__ static __forceinline__ int slot_d(int j) { return (j >> 1) + 4 * (j & 1); }
+  static constexpr u32 kStageXor = 0x88888888u;   // applied once when the tile is staged
+  static constexpr u32 kMask = 0x00780078u;
+  // `M` is kMask held in a vector register, which lets each output be one shift and one v_and_or_b32
+  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32 M, u32 (&o)[4]) {
+    const u32 w = lds_row[oct];
+    constexpr u32 B = 0x3f803f80u;
+    o[0] = ((w << 3) & M) | B;   // nibbles 0,4
+    o[1] = ((w >> 1) & M) | B;   // 1,5
+    o[2] = ((w >> 5) & M) | B;   // 2,6
+    o[3] = ((w >> 9) & M) | B;   // 3,7
+  }
+};
+
+template <> struct KCodec<2> {
+  // field u = code+2 goes to the top 2 mantissa bits: raw = 1 + u/4 = (code + 6)/4.
+  static constexpr float kMul = 4.f, kOff = 6.f;
+  // an octet is half a word: fields 0..7 of the half; dword m holds fields (m, m+4)
+  __device__ static __forceinline__ int slot_d(int j) { return (j >> 1) + 4 * (j & 1); }
+  static constexpr u32 kStageXor = 0xaaaaaaaau;
+  static constexpr u32 kMask = 0x00600060u;
+  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32 M, u32 (&o)[4]) {
+    const u32 w = (lds_row[oct >> 1] >> ((oct & 1) * 16)) & 0xffffu;
+    // fields m (bits 2m) and m+4 (bits 2m+8): move to bits 5..6 and 21..22
+    const u32 t = (w & 0xffu) | ((w & 0xff00u) << 8);  // low byte: fields 0-3, byte 2: fields 4-7
+    constexpr u32 B = 0x3f803f80u;
+    o[0] = ((t << 5) & M) | B;
+    o[1] = ((t << 3) & M) | B;
+    o[2] = ((t << 1) & M) | B;
+    o[3] = ((t >> 1) & M) | B;
+  }
+};
+
+template <> struct KCodec<8> {
+  // bytes are widened through fp32 (exact), raw = code.
+  static constexpr float kMul = 1.f, kOff = 0.f;
+  __device__ static __forceinline__ int slot_d(int j) { return j; }
+  static constexpr u32 kStageXor = 0u, kMask = 0u;
+  __device__ static __forceinline__ void expand(const u32 *lds_row, int oct, u32, u32 (&o)[4]) {
+    const u32 w0 = lds_row[2 * oct], w1 = lds_row[2 * oct + 1];
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[j] = (float)(int)__builtin_amdgcn_sbfe((int)w0, 8 * j, 8);
+      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe((int)w1, 8 * j, 8);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = pack_bf16_hi(f[2 * j], f[2 * j + 1]);
+  }
+};
+
 // octet (8-channel unit) of K that lane-half h contracts in 16-channel chunk ch;
 // chunks never straddle a scale group of `G` channels.
 template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
@@ -163,22 +182,43 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
   return seg * (G / 8) + h * CPS + cl;
 }
 
+// LDS layout of the attention kernel (bytes), shared by kernel and launcher.
+template <int D, int BITS, int GK, int GV> struct AttnLds {
+  static constexpr int WPR = D * BITS / 32;
+  static constexpr int RSK = WPR + 4;       // packed K row stride (words): 16-byte rows
+  static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
+  static constexpr int kParFloats = (2 * (D / GK) + 3 * (D / GV)) * 64;
+  static constexpr int kKp = 0;
+  static constexpr int kVp = kKp + 3 * 64 * RSK * 4;
+  static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
+  static constexpr int kPar = kVt + 2 * D * (64 + 8) * 2;
+  static constexpr int kFlag = kPar + 3 * kParFloats * 4;
+  static constexpr int kBytes = kFlag + 16;
+};
+
 template <int D, int BITS, int GK, int GV>
 __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   constexpr int NSK = D / GK, NSV = D / GV;
   constexpr int WPR = D * BITS / 32;        // packed words per key row
-  constexpr int RS = WPR + 4;               // LDS row stride of packed tiles (words)
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
   constexpr int NDB = D / 32;               // 32-row blocks of O^T
   constexpr int VTS = BN + 8;               // V^T row stride (bf16 elements)
+  using L = AttnLds<D, BITS, GK, GV>;
 
-  __shared__ u32 lds_k[BN * RS];
-  __shared__ u32 lds_vp[BN * RS];
-  __shared__ __attribute__((aligned(16))) uint16_t lds_vt[D * VTS];
-  __shared__ __attribute__((aligned(16))) float lds_ck[NSK][BN];   // ks * scale * log2e * kMul
-  __shared__ __attribute__((aligned(16))) float lds_dk[NSK][BN];   // -ks * scale * log2e * (kzp + kOff)
-  __shared__ __attribute__((aligned(16))) float lds_sv[NSV][BN];   // vs
-  __shared__ __attribute__((aligned(16))) float lds_zv[NSV][BN];   // vzp + vOff
+  // Pipelined LDS buffers (one workgroup barrier per tile):
+  //   packed K, packed V and the per-key parameters of tile t live in slot t % 3,
+  //   the widened V^T of tile t in slot t % 2.
+  // While tile t is being attended, V of tile t+1 is widened and tile t+2 is
+  // written from the registers it was loaded into one iteration earlier.
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  u32 *const lds_kp = reinterpret_cast<u32 *>(lds_raw + L::kKp);          // [3][BN][RSK]
+  u32 *const lds_vp = reinterpret_cast<u32 *>(lds_raw + L::kVp);          // [3][BN][RSV]
+  uint16_t *const lds_vt = reinterpret_cast<uint16_t *>(lds_raw + L::kVt);  // [2][D][VTS]  (vq - vzp_c), transposed
+  float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
+  int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
+  constexpr int RSK = L::RSK, RSV = L::RSV;
+  // parameter block of one tile: ck, dk [NSK][BN]; sv, vr, vz [NSV][BN]
+  constexpr int P_CK = 0, P_DK = NSK * BN, P_SV = 2 * NSK * BN, P_VR = P_SV + NSV * BN, P_VZ = P_VR + NSV * BN;
 
   // XCD-aware decode: consecutive workgroup ids go to different XCDs (8 of
   // them), so ids congruent mod 8 share an L2.  All query tiles of one
@@ -204,7 +244,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   if (limit < 0) limit = 0;
 
   // Q^T operands, gathered in the slot order of the K codec
-  u32 qb[NCH][4];
+  u32x4_t qb[NCH];
   float qsum[NSK];
 #pragma unroll
   for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
@@ -223,8 +263,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
 
-  // ---- tile range -------------------------------------------------------------
-  // every lane of the workgroup must run the same number of tiles
+  // ---- tile range: every lane of the workgroup runs the same number of tiles ----
   __shared__ int lds_maxlim;
   if (tid == 0) lds_maxlim = 0;
   __syncthreads();
@@ -240,8 +279,8 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   for (int i = 0; i < NDB; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) oacc[i][j] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  float r_run[NSV];
+  float m_ref = 0.f, l_run = 0.f;    // softmax reference (log2 domain) and running sum
+  float r_run[NSV];                  // sum_l p' * vzp_r, only fed on tiles with a remainder
 #pragma unroll
   for (int s = 0; s < NSV; ++s) r_run[s] = 0.f;
 
@@ -266,7 +305,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
         vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + off);
       }
     }
-    // scales: thread t < 64*NS handles (key = t % 64, seg = t / 64)
+    // scales: thread t handles (key = t % 64, seg = t / 64)
     {
       const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6;
       if (seg < NSK) {
@@ -282,149 +321,202 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
     }
   };
 
-  if (n_tiles > 0) prefetch(0);
-
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const int t0 = tile * BN;
-    __syncthreads();  // previous tile's LDS reads are finished
+  // registers -> LDS slot of `tile` (packed words as they are, parameters precombined)
+  auto stage = [&](int tile) {
+    const int sl = tile % 3;
+    u32 *kp = lds_kp + sl * BN * RSK, *vp = lds_vp + sl * BN * RSV;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * 256;
       if (LPT * 256 == QUADS || piece < QUADS) {
         const int key = piece / (WPR / 4), w4 = (piece % (WPR / 4)) * 4;
-        *reinterpret_cast<u32x4_t *>(&lds_k[key * RS + w4]) = kreg[i];
-        *reinterpret_cast<u32x4_t *>(&lds_vp[key * RS + w4]) = vreg[i];
+        constexpr u32 KX = KCodec<BITS>::kStageXor, VX = Codec<BITS>::kStageXor;
+        const u32x4_t kx = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
+        *reinterpret_cast<u32x4_t *>(&kp[key * RSK + w4]) = kx;
+        // V rows use an odd stride (bank spread for the column reads of the widening step)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) vp[key * RSV + w4 + j] = vreg[i][j] ^ VX;
       }
     }
-    {
-      const int key = tid & 63, seg = tid >> 6;
-      if (seg < NSK) {
-        const float c = ksc * p.scale_log2e;
-        lds_ck[seg][key] = c * KCodec<BITS>::kMul;
-        lds_dk[seg][key] = -c * (kzp + KCodec<BITS>::kOff);
-      }
-      if (seg < NSV) {
-        lds_sv[seg][key] = vsc;
-        lds_zv[seg][key] = vzp + VCodec<BITS>::kOff;
-      }
+    float *par = lds_par + sl * L::kParFloats;
+    const int key = tid & 63, seg = tid >> 6;
+    if (seg < NSK) {
+      const float c = ksc * p.scale_log2e;
+      par[P_CK + seg * BN + key] = c * KCodec<BITS>::kMul;
+      par[P_DK + seg * BN + key] = -c * (kzp + KCodec<BITS>::kOff);
     }
-    __syncthreads();
-    if (tile + 1 < n_tiles) prefetch(tile + 1);
+    if (seg < NSV) {
+      const float zc = __builtin_amdgcn_fmed3f(vzp, -Codec<BITS>::kZmax, Codec<BITS>::kZmax);
+      const float zr = vzp - zc;
+      par[P_SV + seg * BN + key] = vsc;
+      par[P_VR + seg * BN + key] = zr;
+      par[P_VZ + seg * BN + key] = zc + Codec<BITS>::kOff;
+      if (!(zr == 0.f)) lds_flag[sl] = tile + 1;   // benign race: every writer stores the same tag
+    }
+  };
 
-    // ---- V: packed -> V^T bf16 (each thread: 4 keys x 8 channels) ---------------
+  // packed V of `tile` -> V^T bf16: each thread takes 4 keys x 8 channels
+  auto widen_v = [&](int tile) {
+    const u32 *vp = lds_vp + (tile % 3) * BN * RSV;
+    const float *par = lds_par + (tile % 3) * L::kParFloats;
+    uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
     for (int blk = tid; blk < (BN / 4) * (D / 8); blk += 256) {
       const int kq = blk & (BN / 4 - 1), oct = blk / (BN / 4);
       float f[4][8];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) VCodec<BITS>::codes(&lds_vp[(kq * 4 + kk) * RS], oct, f[kk]);
+      for (int kk = 0; kk < 4; ++kk) {
+        const int key = kq * 4 + kk;
+        Codec<BITS>::codes(&vp[key * RSV], oct, f[kk]);
+        const float z = par[P_VZ + (oct * 8 / GV) * BN + key];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[kk][j] -= z;
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         uint2 v = make_uint2(pack_bf16_hi(f[0][j], f[1][j]), pack_bf16_hi(f[2][j], f[3][j]));
-        *reinterpret_cast<uint2 *>(&lds_vt[(oct * 8 + j) * VTS + kq * 4]) = v;
+        *reinterpret_cast<uint2 *>(&vt[(oct * 8 + j) * VTS + kq * 4]) = v;
       }
     }
-    __syncthreads();
+  };
 
-    // ---- S^T = K Q^T for the two 32-key blocks -----------------------------------
-    float x[2][16];
+  // ---- prologue: tiles 0 and 1 staged, V of tile 0 widened, tile 2 in registers ------
+  if (tid < 3) lds_flag[tid] = 0;
+  __syncthreads();
+  if (n_tiles > 0) { prefetch(0); stage(0); }
+  if (n_tiles > 1) { prefetch(1); stage(1); }
+  __syncthreads();
+  if (n_tiles > 0) widen_v(0);
+  if (n_tiles > 2) prefetch(2);
+  __syncthreads();
+
+  u32 kmask = KCodec<BITS>::kMask;
+  asm volatile("" : "+v"(kmask));   // keep the mask in a vector register (see KCodec::expand)
+
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int t0 = tile * BN;
+    const u32 *kp = lds_kp + (tile % 3) * BN * RSK;
+    const float *par = lds_par + (tile % 3) * L::kParFloats;
+    const uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
+    const bool tile_rem = lds_flag[tile % 3] == tile + 1;   // tagged with the tile, so stale tags never match
+
+    // slot (tile+2)%3 was last read during tile-1 (before the barrier): refill it
+    if (tile + 2 < n_tiles) stage(tile + 2);
+    if (tile + 3 < n_tiles) prefetch(tile + 3);
+
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
+      // ---- S^T = K Q^T for this 32-key block, K widened in registers -------------------
       floatx16_t sacc[NSK];
 #pragma unroll
       for (int s = 0; s < NSK; ++s)
 #pragma unroll
         for (int j = 0; j < 16; ++j) sacc[s][j] = 0.f;
-      const u32 *krow = &lds_k[(kb * 32 + kperm(col)) * RS];
+      const u32 *krow = &kp[(kb * 32 + kperm(col)) * RSK];
 #pragma unroll
       for (int ch = 0; ch < NCH; ++ch) {
         u32 a[4];
-        KCodec<BITS>::expand(krow, k_octet<GK>(ch, half), a);
-        u32x4_t av = {a[0], a[1], a[2], a[3]};
-        u32x4_t bv = {qb[ch][0], qb[ch][1], qb[ch][2], qb[ch][3]};
+        KCodec<BITS>::expand(krow, k_octet<GK>(ch, half), kmask, a);
+        const u32x4_t av = {a[0], a[1], a[2], a[3]};
         sacc[ch / (GK / 16)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, bv), sacc[ch / (GK / 16)], 0, 0, 0);
+            __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[ch / (GK / 16)], 0, 0, 0);
       }
-      // affine map: register i <-> key kb*32 + 16*(i/8) + 8*half + i%8
+
+      // ---- logits of this block in the log2 domain, relative to the reference --------
+      // register i <-> key kb*32 + 16*(i/8) + 8*half + i%8
+      float z[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        float v = 0.f;
+        float v = -m_ref;
 #pragma unroll
-        for (int s = 0; s < NSK; ++s) v += lds_ck[s][key] * sacc[s][i] + lds_dk[s][key] * qsum[s];
-        x[kb][i] = v;
+        for (int s = 0; s < NSK; ++s) v = __builtin_fmaf(par[P_DK + s * BN + key], qsum[s], v);
+#pragma unroll
+        for (int s = 0; s < NSK; ++s) v = __builtin_fmaf(par[P_CK + s * BN + key], sacc[s][i], v);
+        z[i] = v;
       }
-    }
-
-    // ---- mask (block-causal key limit, and the ragged last tile) -----------------
-    if (t0 + BN > wave_minlim) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      // mask: block-causal key limit, and the ragged last tile
+      if (t0 + BN > wave_minlim) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int key = t0 + kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          if (key >= limit) x[kb][i] = -INFINITY;
+          if (key >= limit) z[i] = -INFINITY;
         }
-    }
+      }
 
-    // ---- online softmax ---------------------------------------------------------
-    float mt = x[0][0];
+      // ---- online softmax against a lazily moved reference --------------------------
+      float zmax = z[0];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
+      zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+      const bool first = (tile == 0 && kb == 0);
+      if (first || __any(zmax > kRescaleAt)) {
+        // Move the reference to the row's current maximum: up only (never down) once
+        // something has been accumulated; the very first block takes its maximum as it
+        // is, negative or not (the accumulators are still zero, so alpha = 1 is exact).
+        const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
+        const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+        m_ref += delta;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mt = fmaxf(mt, x[kb][i]);
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {
+        for (int i = 0; i < 16; ++i) z[i] -= delta;
 #pragma unroll
-      for (int d = 0; d < NDB; ++d)
+        for (int d = 0; d < NDB; ++d)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
+          for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
 #pragma unroll
-      for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
-      l_run *= alpha;
-    }
-    // P'^T operands: for each V scale group, p * vs as bf16; 8 registers -> 4 dwords per 16-key chunk
-    u32 pop[NSV][4][4];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+        for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
+        l_run *= alpha;
+      }
+
+      // P'^T operands: for each V scale group, p * vs as bf16; 16 registers -> 2 chunks of 4 dwords
       float pv[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        pv[i] = __builtin_amdgcn_exp2f(x[kb][i] - m_use);
+        pv[i] = __builtin_amdgcn_exp2f(z[i]);
         l_run += pv[i];
       }
+      u32 pop[NSV][2][4];
 #pragma unroll
-      for (int s = 0; s < NSV; ++s) {
-        // The zero-point term must see the same bf16-rounded weights as the
-        // MFMA does, or the constant offset of the raw codes stops cancelling.
+      for (int s = 0; s < NSV; ++s)
 #pragma unroll
         for (int i2 = 0; i2 < 8; ++i2) {
           const int i = 2 * i2;
           const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          const u32 pk = pack_bf16_rne(pv[i] * lds_sv[s][key], pv[i + 1] * lds_sv[s][key + 1]);
-          pop[s][kb * 2 + (i >> 3)][(i & 7) >> 1] = pk;
-          r_run[s] += u2f(pk << 16) * lds_zv[s][key];
-          r_run[s] += u2f(pk & 0xffff0000u) * lds_zv[s][key + 1];
+          pop[s][i >> 3][(i & 7) >> 1] =
+              pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
         }
+      if (tile_rem) {
+        // the remainder term must see the same bf16-rounded weights as the MFMA
+#pragma unroll
+        for (int s = 0; s < NSV; ++s)
+#pragma unroll
+          for (int i2 = 0; i2 < 8; ++i2) {
+            const int i = 2 * i2;
+            const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+            const u32 pk = pop[s][i >> 3][(i & 7) >> 1];
+            r_run[s] = __builtin_fmaf(u2f(pk << 16), par[P_VR + s * BN + key], r_run[s]);
+            r_run[s] = __builtin_fmaf(u2f(pk & 0xffff0000u), par[P_VR + s * BN + key + 1], r_run[s]);
+          }
       }
-    }
 
-    // ---- O^T += V^T P'^T -----------------------------------------------------------
+      // ---- O^T += V^T P'^T for the 32 keys of this block ------------------------------
 #pragma unroll
-    for (int d = 0; d < NDB; ++d) {
-      constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
-      const int s = d / DBS;
+      for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&lds_vt[(d * 32 + col) * VTS + c * 16 + half * 8]);
-        u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
-        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                          __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
-      }
+        for (int d = 0; d < NDB; ++d) {
+          constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
+          const int s = d / DBS;
+          const u32x4_t av =
+              *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
+          u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
+          oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                            __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
+        }
+
+      // between the two key blocks, with the first block's PV MFMAs in flight: widen
+      // the next tile's V into the other V^T slot
+      if (kb == 0 && tile + 1 < n_tiles) widen_v(tile + 1);
     }
+    __syncthreads();   // the one barrier per tile
   }
 
   // ---- epilogue -------------------------------------------------------------------
@@ -452,9 +544,16 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
 
 template <int D, int BITS, int GK, int GV>
 void launch(const AttnParams &p, hipStream_t st) {
+  constexpr int lds_bytes = AttnLds<D, BITS, GK, GV>::kBytes;
+  static bool configured = false;   // above 64 KiB the limit has to be raised once per process
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    configured = true;
+  }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV>), grid, dim3(256), 0, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV>), grid, dim3(256), lds_bytes, st, p);
 }
 
 template <int D, int BITS>
@@ -492,6 +591,7 @@ extern "C" int varq_fused_attn(const void *q, void *out,
     return VARQ_OK;
   }
   VARQ_CHECK_ARG((int64_t)B * Hkv * Lk_stride * D < (1ll << 40), "fused_attn: cache too large");
+  VARQ_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0, "fused_attn: q must be 16-byte and out 8-byte aligned");
 
   AttnParams p;
   p.q = reinterpret_cast<const __bf16 *>(q);
