@@ -15,20 +15,28 @@
 //    max/sum are per-lane (one cross-half exchange per tile) and the S^T
 //    accumulator registers are directly the B operand of the second MFMA.
 //  * The MFMA operands are exact small numbers derived from the codes, never
-//    scaled or rounded; scales are applied in fp32 to the 32x32 results:
-//       O[q,:] = sum_l (p[l,q] * vs[l]) * (vq - vzp)[l,:]
-//    (vq - vzp) is an integer that bf16 holds exactly when |vzp| <= 240.  Larger
-//    V zero-points (data offset by hundreds of quantization steps) are split
-//    zp = zp_c + zp_r; the remainder goes through a correction term on tiles
-//    that have one.
-//  * Packed K and V tiles go HBM -> LDS as they are (16-byte loads, prefetched
-//    one tile ahead).  K words are widened in registers by each wavefront
-//    straight into MFMA A operands, interleaved with the MFMAs (8 codes of one
-//    word = one lane's operand; the codes land in the mantissa of a bf16 1.x, an
-//    affine image of the code that the fp32 epilogue undoes together with the
-//    zero-point: S = ks*(kMul*A - (kzp+kOff)*sum(q))).  V is widened once per
-//    workgroup with its zero-point folded in and written transposed to LDS
-//    (the PV contraction runs over keys).
+//    scaled or rounded: a code lands in the top mantissa bits of a bf16 1.x
+//    (raw = (code + kOff) / kMul), which costs one shift and one and-or per two
+//    elements.  Scales are applied in fp32, zero-points ride on extra MFMA work:
+//       S[l,q]  = ck[l] * ( sum_d rawK[l,d] q[d]  -  (kzp[l]+kOff)/kMul * sum_d q[d] )
+//       O[q,:]  = ( kMul * sum_l p'[l,q] rawV[l,:]  -  sum_l p'[l,q] (vzp[l]+kOff) ) / sum_l p[l,q]
+//    The second term of S is a rank-1 update: both factors are split into three
+//    bf16 pieces and laid on the 16 contraction slots of one more MFMA per key
+//    block.  The second term of O is one more row of V^T (one more 32-row MFMA
+//    block whose row s carries vzp+kOff of V group s).  p' = bf16(p * vs[l]); with a
+//    single V group log2(vs)/ck is added to S through spare slots of the rank-1
+//    MFMA, so exp2 yields p * vs directly, and the denominator is accumulated as
+//    sum_l p'[l,q] / vs[l] by rows 4..6 of the extra block (1/vs in three bf16
+//    pieces): numerator and denominator then use the same rounded weights.
+//    V zero-points beyond +-kZmax (data offset by hundreds of quantization steps)
+//    or with a fractional part are split zp = zp_c + zp_r; the remainder goes
+//    through an fp32 correction term on tiles that have one.
+//  * Packed K and V tiles go HBM -> registers -> LDS as they are (16-byte loads,
+//    issued three tiles ahead, one workgroup barrier per tile).  K words are
+//    widened in registers by each wavefront straight into MFMA A operands,
+//    interleaved with the MFMAs (8 codes of one word = one lane's operand).  V is
+//    widened once per workgroup and written transposed to LDS (the PV contraction
+//    runs over keys).
 //  * Key rows are fed to the first MFMA in a permuted order chosen so that each
 //    lane's accumulator registers hold 8 consecutive keys per 16-key chunk,
 //    which makes the V^T operand a single 16-byte LDS read.
@@ -60,52 +68,81 @@ struct AttnParams {
   float scale_log2e;
 };
 
-// The 8 codes of octet `oct` of one packed row as exact floats code + kOff, and
-// the largest |zp| that still folds exactly into bf16 (|code - zp| <= 256).
-template <int BITS> struct Codec;
-template <> struct Codec<4> {
-  static constexpr float kOff = 8.f, kZmax = 240.f;
+__device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
+  return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);   // {hi[31:16], lo[31:16]} in one v_perm_b32
+}
+
+// ---- V side code widening ----------------------------------------------------
+// The V^T operand of the second MFMA holds, like the K operand of the first, an
+// affine image `raw` of the code (code = kMul * raw - kOff) that costs one shift
+// and one and-or per two elements.  `pairs` widens octet `oct` of two adjacent key
+// rows at once: out[j] = {raw(row0, channel j), raw(row1, channel j)} as a bf16
+// pair, which is one dword of the transposed tile.  The zero-point is not folded
+// in here; it rides on an extra MFMA row (see the kernel).  kZmax bounds the
+// part of the zero-point handled that way: kOff + zp must be a bf16-exact integer.
+template <int BITS> struct VCodec;
+template <> struct VCodec<4> {
+  static constexpr float kMul = 16.f, kOff = 24.f, kZmax = 232.f;
   static constexpr u32 kStageXor = 0x88888888u;   // applied once when the tile is staged: nibble -> code + 8
-  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
-    const u32 w = row[oct];
-    const u32 e = w & 0x0f0f0f0fu, o = (w >> 4) & 0x0f0f0f0fu;
-    f[0] = (float)(e & 0xffu); f[1] = (float)(o & 0xffu);
-    f[2] = (float)((e >> 8) & 0xffu); f[3] = (float)((o >> 8) & 0xffu);
-    f[4] = (float)((e >> 16) & 0xffu); f[5] = (float)((o >> 16) & 0xffu);
-    f[6] = (float)(e >> 24); f[7] = (float)(o >> 24);
+  __device__ static __forceinline__ void pairs(const u32 *row0, const u32 *row1, int oct, u32 M, u32 (&o)[8]) {
+    const u32 w0 = row0[oct], w1 = row1[oct];
+    constexpr u32 B = 0x3f803f80u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      // byte k of both rows, 16 bits apart: nibbles 2k and 2k+1
+      const u32 x = __builtin_amdgcn_perm(w1, w0, 0x0c000c00u | (u32)k | ((u32)(4 + k) << 16));
+      o[2 * k] = ((x << 3) & M) | B;
+      o[2 * k + 1] = ((x >> 1) & M) | B;
+    }
   }
 };
-template <> struct Codec<2> {
-  static constexpr float kOff = 0.f, kZmax = 250.f;
-  static constexpr u32 kStageXor = 0u;
-  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
-    const int w = (int)(row[oct >> 1] >> ((oct & 1) * 16));
-#pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = (float)(int)__builtin_amdgcn_sbfe(w, 2 * j, 2);
+template <> struct VCodec<2> {
+  static constexpr float kMul = 4.f, kOff = 6.f, kZmax = 250.f;
+  static constexpr u32 kStageXor = 0xaaaaaaaau;
+  __device__ static __forceinline__ void pairs(const u32 *row0, const u32 *row1, int oct, u32 M, u32 (&o)[8]) {
+    // the octet is half a word: put the two rows' halves side by side
+    const u32 x = __builtin_amdgcn_perm(row1[oct >> 1], row0[oct >> 1], 0x05040100u + (u32)(oct & 1) * 0x02020202u);
+    constexpr u32 B = 0x3f803f80u;
+    o[0] = ((x << 5) & M) | B;
+    o[1] = ((x << 3) & M) | B;
+    o[2] = ((x << 1) & M) | B;
+    o[3] = ((x >> 1) & M) | B;
+    o[4] = ((x >> 3) & M) | B;
+    o[5] = ((x >> 5) & M) | B;
+    o[6] = ((x >> 7) & M) | B;
+    o[7] = ((x >> 9) & M) | B;
   }
 };
-template <> struct Codec<8> {
-  static constexpr float kOff = 0.f, kZmax = 127.f;
+template <> struct VCodec<8> {
+  static constexpr float kMul = 1.f, kOff = 0.f, kZmax = 256.f;
   static constexpr u32 kStageXor = 0u;
-  __device__ static __forceinline__ void codes(const u32 *row, int oct, float (&f)[8]) {
-    const int w0 = (int)row[2 * oct], w1 = (int)row[2 * oct + 1];
+  __device__ static __forceinline__ void pairs(const u32 *row0, const u32 *row1, int oct, u32, u32 (&o)[8]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f[j] = (float)(int)__builtin_amdgcn_sbfe(w0, 8 * j, 8);
-      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe(w1, 8 * j, 8);
+    for (int h = 0; h < 2; ++h) {
+      const int w0 = (int)row0[2 * oct + h], w1 = (int)row1[2 * oct + h];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        o[4 * h + j] = pack_bf16_hi((float)(int)__builtin_amdgcn_sbfe(w0, 8 * j, 8),
+                                    (float)(int)__builtin_amdgcn_sbfe(w1, 8 * j, 8));
     }
   }
 };
 
-__device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
-  return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);   // {hi[31:16], lo[31:16]} in one v_perm_b32
-}
 __device__ __forceinline__ u32 pack_bf16_rne(float lo, float hi) {
   typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
   typedef float f2 __attribute__((ext_vector_type(2)));
   f2 v = {lo, hi};
   bf2 b = __builtin_convertvector(v, bf2);
   return __builtin_bit_cast(u32, b);
+}
+// x = h0 + h1 + h2 exactly, each piece a bf16 (returned as its 16 bits): three
+// 8-bit slices of the 24-bit significand
+__device__ __forceinline__ void split3_bf16(float x, u32 &h0, u32 &h1, u32 &h2) {
+  const float x0 = u2f(f2u(x) & 0xffff0000u);
+  const float r1 = x - x0;
+  const float x1 = u2f(f2u(r1) & 0xffff0000u);
+  const float x2 = r1 - x1;
+  h0 = f2u(x0) >> 16; h1 = f2u(x1) >> 16; h2 = f2u(x2) >> 16;
 }
 
 // MFMA row r (0..31) of the S^T block carries key kperm(r) of the 32-key block
@@ -187,11 +224,15 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSK = WPR + 4;       // packed K row stride (words): 16-byte rows
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
-  static constexpr int kParFloats = (2 * (D / GK) + 3 * (D / GV)) * 64;
+  static constexpr bool kFoldSv = (D / GV == 1);   // one V group: its scale rides inside the logits
+  static constexpr int kParFloats = ((D / GK) + (kFoldSv ? 1 : 2) * (D / GV)) * 64;
+  static constexpr int RSR = 64 + 8;        // stride (bf16) of the rows feeding the extra PV MFMA
   static constexpr int kKp = 0;
   static constexpr int kVp = kKp + 3 * 64 * RSK * 4;
   static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
-  static constexpr int kPar = kVt + 2 * D * (64 + 8) * 2;
+  static constexpr int kKz = kVt + 2 * D * (64 + 8) * 2;          // rank-1 operands of S^T, 2 x 16 bytes per key and group
+  static constexpr int kWz = kKz + 3 * (D / GK) * 64 * 32;        // 8 rows per slot for the extra PV MFMA
+  static constexpr int kPar = kWz + 3 * 8 * RSR * 2;
   static constexpr int kFlag = kPar + 3 * kParFloats * 4;
   static constexpr int kBytes = kFlag + 16;
 };
@@ -213,12 +254,18 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u32 *const lds_kp = reinterpret_cast<u32 *>(lds_raw + L::kKp);          // [3][BN][RSK]
   u32 *const lds_vp = reinterpret_cast<u32 *>(lds_raw + L::kVp);          // [3][BN][RSV]
-  uint16_t *const lds_vt = reinterpret_cast<uint16_t *>(lds_raw + L::kVt);  // [2][D][VTS]  (vq - vzp_c), transposed
+  uint16_t *const lds_vt = reinterpret_cast<uint16_t *>(lds_raw + L::kVt);  // [2][D][VTS]  raw V codes, transposed
+  u32x4_t *const lds_kz = reinterpret_cast<u32x4_t *>(lds_raw + L::kKz);  // [3][NSK][BN][2] rank-1 A operands (per lane half)
+  // [3][8][RSR] bf16 rows of the extra PV MFMA: row s < NSV = vzp_c + kOff of group s,
+  // rows 4..6 = the three bf16 pieces of 1/vs of group 0, row 7 = zeros
+  uint16_t *const lds_wz = reinterpret_cast<uint16_t *>(lds_raw + L::kWz);
   float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
   int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
   constexpr int RSK = L::RSK, RSV = L::RSV;
-  // parameter block of one tile: ck, dk [NSK][BN]; sv, vr, vz [NSV][BN]
-  constexpr int P_CK = 0, P_DK = NSK * BN, P_SV = 2 * NSK * BN, P_VR = P_SV + NSV * BN, P_VZ = P_VR + NSV * BN;
+  // parameter block of one tile: ck [NSK][BN]; vr [NSV][BN]; sv [NSV][BN] unless folded
+  constexpr bool FOLD_SV = L::kFoldSv;
+  constexpr int RSR = L::RSR;
+  constexpr int P_CK = 0, P_VR = NSK * BN, P_SV = P_VR + NSV * BN;
 
   // XCD-aware decode: consecutive workgroup ids go to different XCDs (8 of
   // them), so ids congruent mod 8 share an L2.  All query tiles of one
@@ -262,6 +309,23 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   }
 #pragma unroll
   for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
+  // The K zero-point term -(kzp+kOff)/kMul * sum(q) is a rank-1 update of S^T and
+  // rides on one more MFMA per key block and group.  Both factors are split into
+  // three bf16 pieces (a0+a1+a2, b0+b1+b2, exact) and the 9 products are laid on
+  // the 16 contraction slots: slots 0..7 (lower lane half) carry
+  // A = a0 a0 a0 a1 a1 a1 a2 a2 against B = b0 b1 b2 b0 b1 b2 b0 b1 (a2*b2, 2^-32 of
+  // the term, is dropped).  With a single V group, slots 0..2 of the upper half add
+  // log2(vs)/ck (three pieces against 1.0), which makes exp2(logit) come out as
+  // p * vs without a multiplication; the other upper slots are zero.
+  u32x4_t bq[NSK];
+#pragma unroll
+  for (int s = 0; s < NSK; ++s) {
+    u32 b0, b1, b2;
+    split3_bf16(qsum[s], b0, b1, b2);
+    if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
+    else if (FOLD_SV && s == 0) bq[s] = u32x4_t{0x3f803f80u, 0x00003f80u, 0u, 0u};
+    else bq[s] = u32x4_t{0u, 0u, 0u, 0u};
+  }
 
   // ---- tile range: every lane of the workgroup runs the same number of tiles ----
   __shared__ int lds_maxlim;
@@ -279,7 +343,12 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   for (int i = 0; i < NDB; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) oacc[i][j] = 0.f;
-  float m_ref = 0.f, l_run = 0.f;    // softmax reference (log2 domain) and running sum
+  // extra O^T block: row s < NSV: sum_l p'_s * (vzp_c + kOff); rows 4..6: pieces of the
+  // softmax denominator sum_l p'_0 / vs_0, i.e. the sum of the weights as rounded for the MFMA
+  floatx16_t racc;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) racc[j] = 0.f;
+  float m_ref = 0.f;                 // softmax reference (log2 domain)
   float r_run[NSV];                  // sum_l p' * vzp_r, only fed on tiles with a remainder
 #pragma unroll
   for (int s = 0; s < NSV; ++s) r_run[s] = 0.f;
@@ -291,7 +360,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   constexpr int QUADS = BN * WPR / 4;                 // 16-byte pieces per packed tile
   constexpr int LPT = (QUADS + 255) / 256;            // pieces per thread
   u32x4_t kreg[LPT], vreg[LPT];
-  float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f;
+  float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
 
   auto prefetch = [&](int tile) {
     const int t0 = tile * BN;
@@ -305,18 +374,21 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
         vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + off);
       }
     }
-    // scales: thread t handles (key = t % 64, seg = t / 64)
+    // scales: thread t handles key t % 64; wavefront w takes K group w and V group
+    // 3 - w, which puts the K and the V arithmetic of the single-group case on
+    // different wavefronts
     {
-      const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6;
+      const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = 3 - seg;
       if (seg < NSK) {
         const int64_t g = (kv_row0 + key) * NSK + seg;
         ksc = p.k_scale[g];
         kzp = p.k_zp ? p.k_zp[g] : 0.f;
       }
-      if (seg < NSV) {
-        const int64_t g = (kv_row0 + key) * NSV + seg;
+      if (vseg < NSV) {
+        const int64_t g = (kv_row0 + key) * NSV + vseg;
         vsc = p.v_scale[g];
         vzp = p.v_zp ? p.v_zp[g] : 0.f;
+        if (FOLD_SV) ksc0 = p.k_scale[(kv_row0 + key) * NSK];
       }
     }
   };
@@ -330,7 +402,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
       const int piece = tid + i * 256;
       if (LPT * 256 == QUADS || piece < QUADS) {
         const int key = piece / (WPR / 4), w4 = (piece % (WPR / 4)) * 4;
-        constexpr u32 KX = KCodec<BITS>::kStageXor, VX = Codec<BITS>::kStageXor;
+        constexpr u32 KX = KCodec<BITS>::kStageXor, VX = VCodec<BITS>::kStageXor;
         const u32x4_t kx = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
         *reinterpret_cast<u32x4_t *>(&kp[key * RSK + w4]) = kx;
         // V rows use an odd stride (bank spread for the column reads of the widening step)
@@ -339,48 +411,73 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
       }
     }
     float *par = lds_par + sl * L::kParFloats;
-    const int key = tid & 63, seg = tid >> 6;
+    const int key = tid & 63, seg = tid >> 6, vseg = 3 - seg;
+    // |ck| is kept away from zero so that log2(vs)/ck stays finite for a constant group
+    auto ck_of = [&](float ks) {
+      const float c = ks * p.scale_log2e * KCodec<BITS>::kMul;
+      return __builtin_fabsf(c) < 1e-30f ? 1e-30f : c;
+    };
     if (seg < NSK) {
-      const float c = ksc * p.scale_log2e;
-      par[P_CK + seg * BN + key] = c * KCodec<BITS>::kMul;
-      par[P_DK + seg * BN + key] = -c * (kzp + KCodec<BITS>::kOff);
+      par[P_CK + seg * BN + key] = ck_of(ksc);
+      u32 a0, a1, a2;
+      split3_bf16(-(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
+      u32x4_t *dst = &lds_kz[((sl * NSK + seg) * BN + key) * 2];
+      dst[0] = u32x4_t{a0 | (a0 << 16), a0 | (a1 << 16), a1 | (a1 << 16), a2 | (a2 << 16)};
+      if (!(FOLD_SV && seg == 0)) dst[1] = u32x4_t{0u, 0u, 0u, 0u};
     }
-    if (seg < NSV) {
-      const float zc = __builtin_amdgcn_fmed3f(vzp, -Codec<BITS>::kZmax, Codec<BITS>::kZmax);
+    if (vseg < NSV) {
+      const int seg = vseg;
+      if (FOLD_SV) {
+        u32 l0, l1, l2;
+        split3_bf16(__builtin_amdgcn_logf(vsc) * __builtin_amdgcn_rcpf(ck_of(ksc0)), l0, l1, l2);
+        lds_kz[(sl * NSK * BN + key) * 2 + 1] = u32x4_t{l0 | (l1 << 16), l2, 0u, 0u};
+      }
+      // integer part of the zero-point within +-kZmax rides on the MFMA, the rest (none
+      // for zero-points produced by the quantizer of ordinary data) on the fp32 remainder
+      const float zc = __builtin_amdgcn_fmed3f(__builtin_rintf(vzp), -VCodec<BITS>::kZmax, VCodec<BITS>::kZmax);
       const float zr = vzp - zc;
-      par[P_SV + seg * BN + key] = vsc;
+      if (!FOLD_SV) par[P_SV + seg * BN + key] = vsc;
       par[P_VR + seg * BN + key] = zr;
-      par[P_VZ + seg * BN + key] = zc + Codec<BITS>::kOff;
+      uint16_t *rows = lds_wz + sl * 8 * RSR;
+      rows[seg * RSR + key] = (uint16_t)(f2u(zc + VCodec<BITS>::kOff) >> 16);
+      if (seg == 0) {
+        u32 i0, i1, i2;
+        split3_bf16(__builtin_amdgcn_rcpf(vsc), i0, i1, i2);
+        rows[4 * RSR + key] = (uint16_t)i0;
+        rows[5 * RSR + key] = (uint16_t)i1;
+        rows[6 * RSR + key] = (uint16_t)i2;
+      }
       if (!(zr == 0.f)) lds_flag[sl] = tile + 1;   // benign race: every writer stores the same tag
     }
   };
 
+  u32 kmask = KCodec<BITS>::kMask;
+  asm volatile("" : "+v"(kmask));   // keep the mask in a vector register (see KCodec::expand)
+
+  // row of the extra PV block this lane feeds in the MFMA of V group s (as element offset)
+  int rowsel[NSV];
+#pragma unroll
+  for (int s = 0; s < NSV; ++s) rowsel[s] = ((col == s) ? s : (s == 0 && col >= 4 && col < 7) ? col : 7) * RSR;
+
   // packed V of `tile` -> V^T bf16: each thread takes 4 keys x 8 channels
   auto widen_v = [&](int tile) {
     const u32 *vp = lds_vp + (tile % 3) * BN * RSV;
-    const float *par = lds_par + (tile % 3) * L::kParFloats;
     uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
     for (int blk = tid; blk < (BN / 4) * (D / 8); blk += 256) {
       const int kq = blk & (BN / 4 - 1), oct = blk / (BN / 4);
-      float f[4][8];
+      const u32 *row = &vp[kq * 4 * RSV];
+      u32 lo[8], hi[8];
+      VCodec<BITS>::pairs(row, row + RSV, oct, kmask, lo);
+      VCodec<BITS>::pairs(row + 2 * RSV, row + 3 * RSV, oct, kmask, hi);
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const int key = kq * 4 + kk;
-        Codec<BITS>::codes(&vp[key * RSV], oct, f[kk]);
-        const float z = par[P_VZ + (oct * 8 / GV) * BN + key];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[kk][j] -= z;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        uint2 v = make_uint2(pack_bf16_hi(f[0][j], f[1][j]), pack_bf16_hi(f[2][j], f[3][j]));
-        *reinterpret_cast<uint2 *>(&vt[(oct * 8 + j) * VTS + kq * 4]) = v;
-      }
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<uint2 *>(&vt[(oct * 8 + j) * VTS + kq * 4]) = make_uint2(lo[j], hi[j]);
     }
   };
 
   // ---- prologue: tiles 0 and 1 staged, V of tile 0 widened, tile 2 in registers ------
   if (tid < 3) lds_flag[tid] = 0;
+  if (tid < 3 * RSR) lds_wz[((tid / RSR) * 8 + 7) * RSR + tid % RSR] = 0;   // the all-zero row of each slot
   __syncthreads();
   if (n_tiles > 0) { prefetch(0); stage(0); }
   if (n_tiles > 1) { prefetch(1); stage(1); }
@@ -389,14 +486,13 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   if (n_tiles > 2) prefetch(2);
   __syncthreads();
 
-  u32 kmask = KCodec<BITS>::kMask;
-  asm volatile("" : "+v"(kmask));   // keep the mask in a vector register (see KCodec::expand)
-
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int t0 = tile * BN;
     const u32 *kp = lds_kp + (tile % 3) * BN * RSK;
     const float *par = lds_par + (tile % 3) * L::kParFloats;
     const uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
+    const u32x4_t *kz = lds_kz + (tile % 3) * NSK * BN * 2;
+    const uint16_t *wz = lds_wz + (tile % 3) * 8 * RSR;
     const bool tile_rem = lds_flag[tile % 3] == tile + 1;   // tagged with the tile, so stale tags never match
 
     // slot (tile+2)%3 was last read during tile-1 (before the barrier): refill it
@@ -405,13 +501,34 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
 
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
+      // LDS operands are requested well ahead of their use (the scheduling fences keep
+      // the requests where they are written): with two wavefronts per SIMD there is
+      // little else to cover the LDS latency.  Only where the registers allow it.
+      constexpr bool HOIST = (NSK == 1 && NSV == 1);
+      // register i of this lane <-> key kb*32 + 16*(i/8) + 8*half + i%8 of the tile
+      float ckv[NSK][16];
+#pragma unroll
+      for (int s = 0; s < (HOIST ? NSK : 0); ++s)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
+          const float4 t = *reinterpret_cast<const float4 *>(&par[P_CK + s * BN + key]);
+          ckv[s][4 * i4] = t.x; ckv[s][4 * i4 + 1] = t.y; ckv[s][4 * i4 + 2] = t.z; ckv[s][4 * i4 + 3] = t.w;
+        }
+
       // ---- S^T = K Q^T for this 32-key block, K widened in registers -------------------
       floatx16_t sacc[NSK];
+      const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
-      for (int s = 0; s < NSK; ++s)
+      for (int s = 0; s < NSK; ++s) {
+        // starts the accumulator with the zero-point term (see bq above)
+        floatx16_t zero;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) sacc[s][j] = 0.f;
-      const u32 *krow = &kp[(kb * 32 + kperm(col)) * RSK];
+        for (int j = 0; j < 16; ++j) zero[j] = 0.f;
+        sacc[s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
+                                                          __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+      }
+      const u32 *krow = &kp[krow_i * RSK];
 #pragma unroll
       for (int ch = 0; ch < NCH; ++ch) {
         u32 a[4];
@@ -421,17 +538,40 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
             __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[ch / (GK / 16)], 0, 0, 0);
       }
 
+      // requested now, used after the softmax arithmetic: V scales and the V^T operands
+      // of the first 16-key chunk
+      float svv[NSV][16];
+#pragma unroll
+      for (int s = 0; s < ((HOIST && !FOLD_SV) ? NSV : 0); ++s)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
+          const float4 t = *reinterpret_cast<const float4 *>(&par[P_SV + s * BN + key]);
+          svv[s][4 * i4] = t.x; svv[s][4 * i4 + 1] = t.y; svv[s][4 * i4 + 2] = t.z; svv[s][4 * i4 + 3] = t.w;
+        }
+      u32x4_t vta[NDB], wza[NSV];
+      auto load_v_operands = [&](int c) {
+#pragma unroll
+        for (int d = 0; d < NDB; ++d)
+          vta[d] = *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
+#pragma unroll
+        for (int s = 0; s < NSV; ++s) {
+          wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
+        }
+      };
+      if constexpr (HOIST) load_v_operands(0);
+      if constexpr (HOIST) __builtin_amdgcn_sched_barrier(0);
+
       // ---- logits of this block in the log2 domain, relative to the reference --------
-      // register i <-> key kb*32 + 16*(i/8) + 8*half + i%8
       float z[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
         float v = -m_ref;
 #pragma unroll
-        for (int s = 0; s < NSK; ++s) v = __builtin_fmaf(par[P_DK + s * BN + key], qsum[s], v);
-#pragma unroll
-        for (int s = 0; s < NSK; ++s) v = __builtin_fmaf(par[P_CK + s * BN + key], sacc[s][i], v);
+        for (int s = 0; s < NSK; ++s) {
+          const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+          v = __builtin_fmaf(HOIST ? ckv[s][i] : par[P_CK + s * BN + key], sacc[s][i], v);
+        }
         z[i] = v;
       }
       // mask: block-causal key limit, and the ragged last tile
@@ -463,17 +603,15 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
           for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
 #pragma unroll
+        for (int j = 0; j < 16; ++j) racc[j] *= alpha;
+#pragma unroll
         for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
-        l_run *= alpha;
       }
 
       // P'^T operands: for each V scale group, p * vs as bf16; 16 registers -> 2 chunks of 4 dwords
       float pv[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        pv[i] = __builtin_amdgcn_exp2f(z[i]);
-        l_run += pv[i];
-      }
+      for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
       u32 pop[NSV][2][4];
 #pragma unroll
       for (int s = 0; s < NSV; ++s)
@@ -481,7 +619,9 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
         for (int i2 = 0; i2 < 8; ++i2) {
           const int i = 2 * i2;
           const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          pop[s][i >> 3][(i & 7) >> 1] =
+          if constexpr (FOLD_SV) pop[s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
+          else if constexpr (HOIST) pop[s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[s][i], pv[i + 1] * svv[s][i + 1]);
+          else pop[s][i >> 3][(i & 7) >> 1] =
               pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
         }
       if (tile_rem) {
@@ -498,19 +638,36 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
           }
       }
 
-      // ---- O^T += V^T P'^T for the 32 keys of this block ------------------------------
+      // ---- O^T += V^T P'^T for the 32 keys of this block; one more MFMA per chunk and
+      //      V group feeds the extra block: its row s collects the zero-point sum of group
+      //      s and rows 4..6 (group 0 only) the softmax denominator ------------------------
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+      for (int c = 0; c < 2; ++c) {
+        u32x4_t av[NDB], aw[NSV];
+        if constexpr (!HOIST) load_v_operands(c);
+#pragma unroll
+        for (int d = 0; d < NDB; ++d) av[d] = vta[d];
+#pragma unroll
+        for (int s = 0; s < NSV; ++s) aw[s] = wza[s];
+        if (HOIST && c == 0) {
+          load_v_operands(1);   // in flight under this chunk's MFMAs
+          if constexpr (HOIST) __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int d = 0; d < NDB; ++d) {
           constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
           const int s = d / DBS;
-          const u32x4_t av =
-              *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
           u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
-          oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+          oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[d]),
                                                             __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
         }
+#pragma unroll
+        for (int s = 0; s < NSV; ++s) {
+          u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
+          racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
+                                                         __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
+        }
+      }
 
       // between the two key blocks, with the first block's PV MFMAs in flight: widen
       // the next tile's V into the other V^T slot
@@ -520,21 +677,26 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   }
 
   // ---- epilogue -------------------------------------------------------------------
-  l_run += __shfl_xor(l_run, 32, 64);
 #pragma unroll
   for (int s = 0; s < NSV; ++s) r_run[s] += __shfl_xor(r_run[s], 32, 64);
-  const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+  // rows 4..6 of racc are registers 0..2 of the upper lane half, rows 0..3 registers 0..3 of the lower
+  const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
+  const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
+  float rq[NSV];
+#pragma unroll
+  for (int s = 0; s < NSV; ++s) rq[s] = __shfl(racc[s], col, 64) + r_run[s];
   if (q_live) {
     __bf16 *optr = p.out + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow) * D;
 #pragma unroll
     for (int d = 0; d < NDB; ++d) {
       constexpr int DBS = GV / 32;
-      const float r = r_run[d / DBS];
+      const float r = rq[d / DBS];
+      constexpr float VM = VCodec<BITS>::kMul;
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
-        const float o0 = (oacc[d][4 * g4 + 0] - r) * inv, o1 = (oacc[d][4 * g4 + 1] - r) * inv;
-        const float o2 = (oacc[d][4 * g4 + 2] - r) * inv, o3 = (oacc[d][4 * g4 + 3] - r) * inv;
+        const float o0 = (VM * oacc[d][4 * g4 + 0] - r) * inv, o1 = (VM * oacc[d][4 * g4 + 1] - r) * inv;
+        const float o2 = (VM * oacc[d][4 * g4 + 2] - r) * inv, o3 = (VM * oacc[d][4 * g4 + 3] - r) * inv;
         uint2 v = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
         *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = v;
       }
