@@ -162,14 +162,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
 // one group per lane" goes through a 4 KiB wave-private LDS window, so there is
 // no workgroup barrier anywhere.
 //
-// Rounding: x/s is needed exactly as an IEEE fp32 division rounds it.  The fp64
-// product x * RN64(1/s) is within 2^-52 (relative) of the true quotient, and a
-// quotient of two fp32 numbers is never closer than 2^-49 (relative) to a point
-// where rounding to fp32 changes (such a point has 25 significant bits; x - m*s
-// is a non-zero multiple of ulp(m)*ulp(s)).  Narrowing the product to fp32
-// therefore yields the correctly rounded quotient for every finite input,
-// denormals included, at 3 full-rate instructions instead of a ~11-instruction
-// division sequence.
+// Rounding: x/s is needed exactly as an IEEE fp32 division rounds it; see the
+// two routes (fp32 correction step, fp64 product) in the kernel body.
 template <int DT, int BITS, bool ASYM, int LPG4, bool DENSE>
 __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   __shared__ Raw8<DT> lds_stage[4][256];   // per wave: 256 octets in, then packed words out
@@ -228,36 +222,68 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   float s, zp = 0.f;
   if (ASYM) s = fmaxf((mx - mn) / (float)QRange<BITS>::kLevels, p.eps);
   else s = fmaxf(mx / kMax, p.eps);
-  const double rinv = 1.0 / (double)s;
-  if (ASYM) zp = kMin - rintf((float)((double)mn * rinv));
 
-  // clamp(t + zp, qmin, qmax) as clamp(t, qmin - zp, qmax - zp) + zp, with the
-  // final add also planting the integer in the low mantissa bits (1.5 * 2^23
-  // trick): exact whenever |zp| <= 2^22.  Larger zero-points (data offset by
-  // millions of quantization steps) take the literal sequence.
+  // x/s exactly as an IEEE fp32 division rounds it, in three full-rate
+  // instructions: with r = RN(1/s), q0 = RN(x*r) is within an ulp of the quotient,
+  // e = x - q0*s is exact in one fma, and RN(q0 + e*r) is the correctly rounded
+  // quotient (Markstein's correction step).  That holds for every finite x unless
+  // the significand of s is all ones or the residual can underflow; such groups,
+  // and zero-points beyond 2^22, take the fp64 route below.
+  const float r = 1.0f / s;
+  const bool plain = s > 0x1p-96f && s < 0x1p96f && (f2u(s) & 0x7fffffu) != 0x7fffffu;
+  auto quotient = [&](float x) {
+    const float q0 = x * r;
+    const float e = __builtin_fmaf(-q0, s, x);
+    return __builtin_fmaf(e, r, q0);
+  };
+  const bool wave_plain = __builtin_amdgcn_ballot_w64(!plain) == 0;
+  if (ASYM) zp = kMin - rintf(wave_plain ? quotient(mn) : mn / s);
   const bool big_zp = ASYM && !(fabsf(zp) <= 0x1p22f);
-  const float lo = kMin - zp, hi = kMax - zp, magic = zp + 12582912.f;
+
+  // Codes: clamp(rint(t) + zp, qmin, qmax) = rint(clamp(t, qmin - zp, qmax - zp)) + zp
+  // (the bounds are integers).  Adding 1.5 * 2^23 rounds the clamped quotient to
+  // nearest-even and leaves the integer in the low mantissa bits; the zero-point
+  // is then added to all fields of a packed word at once, modulo the field width
+  // (the sum is known to fit the field).
+  const float lo = kMin - zp, hi = kMax - zp;
+  constexpr u32 kFieldHi = BITS == 8 ? 0x80808080u : BITS == 4 ? 0x88888888u : 0xaaaaaaaau;
+  constexpr u32 kFieldLsb = BITS == 8 ? 0x01010101u : BITS == 4 ? 0x11111111u : 0x55555555u;
+  const u32 zrep = ((u32)(int)zp & ((1u << BITS) - 1u)) * kFieldLsb;
+  const u32 zlo = zrep & ~kFieldHi, zhi = zrep & kFieldHi;
+  auto add_zp = [&](u32 wd) { return ASYM ? (((wd & ~kFieldHi) + zlo) ^ (wd & kFieldHi) ^ zhi) : wd; };
   u32 w[4][2];
-  auto quantize_all = [&](auto literal) {
+  auto quantize_all = [&](auto exact64) {
+    double rinv = 0.0;
+    if (decltype(exact64)::value) rinv = 1.0 / (double)s;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       u32 acc = 0;
       w[k][0] = 0; w[k][1] = 0;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float t = rintf((float)((double)v[k][e] * rinv));
         u32 q;
-        if (decltype(literal)::value) q = (u32)(int)__builtin_amdgcn_fmed3f(ASYM ? t + zp : t, kMin, kMax);
-        else q = f2u(__builtin_amdgcn_fmed3f(t, lo, hi) + magic);
+        if (decltype(exact64)::value) {
+          // fp64 product x * RN64(1/s): within 2^-52 of the quotient, which is never that
+          // close to a point where rounding to fp32 changes, so narrowing it is exact too
+          const float t = rintf((float)((double)v[k][e] * rinv));
+          q = (u32)(int)__builtin_amdgcn_fmed3f(ASYM ? t + zp : t, kMin, kMax);
+        } else {
+          q = f2u(__builtin_amdgcn_fmed3f(quotient(v[k][e]), lo, hi) + 12582912.f);
+        }
         acc = __builtin_amdgcn_alignbit(q, acc, BITS);
         if (BITS == 8 && e == 3) { w[k][0] = acc; acc = 0; }
       }
       if (BITS == 8) w[k][1] = acc;
       else if (BITS == 4) w[k][0] = acc;
       else w[k][0] = acc >> 16;
+      if (!decltype(exact64)::value) {
+        w[k][0] = add_zp(w[k][0]);
+        if (BITS == 8) w[k][1] = add_zp(w[k][1]);
+        if (BITS == 2) w[k][0] &= 0xffffu;
+      }
     }
   };
-  if (__builtin_amdgcn_ballot_w64(big_zp) != 0) quantize_all(std::true_type{});   // wave-uniform, rare
+  if (!wave_plain || __builtin_amdgcn_ballot_w64(big_zp) != 0) quantize_all(std::true_type{});   // wave-uniform, rare
   else quantize_all(std::false_type{});
   if (BITS == 2 && LPG4 > 1) {
 #pragma unroll
