@@ -6,7 +6,11 @@ and V [2,16,10521,128] bf16 to INT4 group-128 asymmetric, then fused dequant
 attention of the final scale's 4096 queries over all 10521 packed keys.  Inputs
 are resident in HBM before the timed region.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+After the timed region (and outside `value`) it also replays BASELINE config 5,
+one image batch of the Infinity schedule through the pre-allocated mixed-bit
+cache (append + attend per scale), and reports its latency per image.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5]
 """
 import argparse
 import json
@@ -62,12 +66,48 @@ def cpu_baseline(torch, O, k0, v0, q0, threads):
             't_attn_equiv_s': t_attn}
 
 
+def c5_latency(torch, dev, passes=10, warm=3):
+    """Config 5: B=8 (4 images x CFG pair), H=16, D=128, the 13 Infinity scales; heads carry
+    2/4/8-bit codes (seeded), group 64 asymmetric.  Per scale: quantize+pack the step's K and V
+    in place into the pre-allocated cache, then fused attention of that scale's queries over
+    the prefix.  Returns seconds per pass (all scales, one layer)."""
+    from var_q_amd import PackedKVCache
+    from var_q_amd.schedules import INFINITY_PATCH_NUMS
+    B5, H5, D5 = 8, 16, 128
+    ns = [pn * pn for pn in INFINITY_PATCH_NUMS]
+    g = torch.Generator().manual_seed(5000)
+    bits = [(2, 4, 8)[int(i)] for i in torch.randint(0, 3, (H5,), generator=g)]
+    cache = PackedKVCache(B5, H5, sum(ns), D5, bits, 64, dev)
+    gd = torch.Generator(device=dev).manual_seed(5005)
+    steps = [tuple(torch.randn(B5, H5, n, D5, device=dev, generator=gd).bfloat16() for _ in range(3)) for n in ns]
+    outs = [torch.empty_like(s[0]) for s in steps]
+    def one_pass():
+        cache.reset()
+        for (q, k, v), o in zip(steps, outs):
+            cache.append(k, v)
+            cache.attend(q, 1.0 / math.sqrt(D5), out=o)
+    for _ in range(warm):
+        one_pass()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        one_pass()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / passes
+    flops = sum(4 * B5 * H5 * n * sum(ns[:i + 1]) * D5 for i, n in enumerate(ns))
+    return {'workload': 'config 5: 13-scale Infinity schedule, B=8 H=16 D=128, per-head bits %s, group 64 asymmetric, '
+                        'in-place append + fused attention per scale, one layer' % ''.join(str(b) for b in bits),
+            'ms_per_layer_pass': round(dt * 1e3, 4), 'ms_per_image_per_layer': round(dt * 1e3 / 4, 4),
+            'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=40)
-    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
+    ap.add_argument('--no-c5', action='store_true', help='skip the config-5 latency leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -193,10 +233,11 @@ def main():
         'roofline': {'kernel': 'fused_attn_kernel<128,4,128,128>', 'bound': 'mfma', 'achieved': round(attn_tflops, 2),
                      'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s', 'frac': round(attn_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
                      'traffic': None if not traffic else traffic.get('fused_attn')},
-        'roofline_pack': {'kernel': 'quant_pack_rows_kernel<bf16,4,asym,16>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
+        'roofline_pack': {'kernel': 'quant_pack_rows32_kernel<bf16,4,asym,4 lanes per group,dense>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
                           'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(pack_gbps / HBM_PEAK_GBPS, 4),
                           'traffic': None if not traffic else traffic.get('quant_pack_rows')},
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
+        'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
     }
     print(json.dumps(line), flush=True)
 

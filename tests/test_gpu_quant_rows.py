@@ -46,6 +46,50 @@ def test_adversarial_rows(dev, dtype, bits, asym, c, group):
     _check(adversarial_rows(c, dtype), group, bits, asym, dev)
 
 
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('asym', [False, True])
+@pytest.mark.parametrize('c,group', [(128, 128), (64, 32), (16, 16)])
+def test_scale_with_all_ones_significand(dev, bits, asym, c, group):
+    """Scales of the form (2 - 2^-23) * 2^e are the one case where correcting x * (1/s)
+    by a single residual step does not reproduce the IEEE quotient (x just above
+    s/2 yields 0.5 instead of 0.50000006 and rounds to 0 instead of 1): the
+    kernel must route such groups through its exact fallback."""
+    import numpy as np
+    levels = float((1 << bits) - 1) if asym else float((1 << (bits - 1)) - 1)
+    rows = []
+    for e in range(-6, 4):
+        s_star = np.float32((2 - 2.0 ** -23) * 2.0 ** e)
+        a = np.float32(np.float64(s_star) * levels)
+        cands = [a]
+        for _ in range(16):
+            cands.append(np.nextafter(cands[-1], np.float32(np.inf)))
+        lo = a
+        for _ in range(16):
+            lo = np.nextafter(lo, np.float32(-np.inf))
+            cands.append(lo)
+        hit = [v for v in cands if np.float32(v) / np.float32(levels) == s_star]
+        assert hit, 'no range value gives the wanted scale'
+        top = float(hit[0])
+        half = np.float32(np.float64(s_star) * 0.5)
+        x = np.zeros(c, dtype=np.float32)
+        vals = [np.nextafter(half, np.float32(np.inf)), half, np.nextafter(half, np.float32(0)),
+                np.float32(np.float64(s_star) * 1.5), np.nextafter(np.float32(np.float64(s_star) * 2.5), np.float32(np.inf))]
+        vals = [v for v in vals if float(v) < top]
+        for gi in range(c // group):
+            base = gi * group
+            x[base] = top                       # fixes the scale of the group (min stays 0 for asym)
+            for j, v in enumerate(vals):
+                x[base + 1 + j] = v
+                if not asym and base + 8 + j < base + group:
+                    x[base + 8 + j] = -v
+        rows.append(torch.from_numpy(x))
+    x = torch.stack(rows)
+    q, sc, _ = O.quant_groupwise(x, group, bits, asym)
+    assert bool(((sc.view(torch.int32) & 0x7fffff) == 0x7fffff).all()), 'test construction: scale significand not all ones'
+    note('quant_rows all-ones scale', bits, asym, c, group)
+    _check(x, group, bits, asym, dev)
+
+
 def test_empty_and_single_row(dev):
     note('quant_rows empty')
     w, s, z = ops.quant_pack_rows(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), 64, 4, True)
