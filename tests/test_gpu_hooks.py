@@ -1,0 +1,121 @@
+"""Self-attention hook modules on the GPU: the drop-in (unfused) backend against
+the same module on the CPU with the oracle quantizer, and the fused backend
+(packed cache + fused attention) A/B against the unfused one.
+
+Tolerances: the fused and unfused backends quantize with the same kernels, so
+their caches must dequantize to identical values; their outputs differ by the
+attention arithmetic only (bf16 SDPA on dequantized K/V vs exact codes), for
+which the bound is max-abs 2e-2 on unit-range attention outputs scaled by the
+output range, cosine >= 0.9995."""
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import note
+from var_q_amd import hooks
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _inference_mode():
+    with torch.no_grad():
+        yield
+
+
+def _cos(a, b):
+    return float(torch.nn.functional.cosine_similarity(a.double().flatten(), b.double().flatten(), dim=0))
+
+
+@pytest.mark.parametrize('layout', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('method,bits', [('G_SCALE_HEAD_DIM', 8), ('G_TOKEN_HEAD', 4), ('G_HEAD_DIM', 8)])
+def test_var_dropin_matches_cpu_oracle_module(dev, layout, method, bits):
+    torch.manual_seed(3)
+    C, H = 256, 4
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, q_bits=bits, quant_method=method, enable_quantization=True,
+              max_tokens=30)
+    cpu = hooks.VarSelfAttention(0, quantizer_factory=O.OracleVARQ, **kw)
+    gpu = hooks.VarSelfAttention(0, **kw).to(dev)
+    gpu.load_state_dict(cpu.state_dict())
+    cpu.kv_caching(True)
+    gpu.kv_caching(True)
+    for n in (1, 4, 9, 16):
+        note('hooks var dropin', layout, method, bits, n)
+        x = torch.randn(2, n, C)
+        a, b = cpu(x), gpu(x.to(dev)).cpu()
+        # the two differ by fp32 GEMM summation order, which can move a code by one step
+        step = a.abs().max().item() / (2 ** (bits - 1))
+        assert (a - b).abs().max().item() <= 2 * step + 1e-3, (n, (a - b).abs().max().item(), step)
+        assert _cos(a, b) > (0.999 if bits == 8 else 0.99)
+
+
+@pytest.mark.parametrize('layout', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('bits,sym', [(4, False), (8, True), (2, False)])
+def test_var_fused_vs_unfused(dev, layout, bits, sym):
+    torch.manual_seed(4)
+    C, H = 512, 8        # head_dim 64 as in VAR
+    pn = (1, 2, 3, 4, 5, 6, 8, 10, 13, 16)
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, q_bits=bits, quant_method='G_GROUP', group_size=64,
+              symmetric=sym, enable_quantization=True, max_tokens=680)
+    a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.VarSelfAttention(0, fused=True, **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    for p in pn:
+        note('hooks var fused', layout, bits, sym, p)
+        x = torch.randn(4, p * p, C, device=dev, dtype=torch.bfloat16)
+        a, b = a_mod(x).float(), b_mod(x).float()
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995
+    # both backends hold the same quantized cache
+    ka = a_mod.k_quant.dequant_all()
+    ka = ka if layout == 'BHLc' else ka.transpose(1, 2)
+    assert torch.equal(ka.contiguous(), b_mod.packed_cache.dequant('k'))
+    va = a_mod.v_quant.dequant_all()
+    va = va if layout == 'BHLc' else va.transpose(1, 2)
+    assert torch.equal(va.contiguous(), b_mod.packed_cache.dequant('v'))
+
+
+def test_infinity_fused_vs_unfused_with_rope(dev):
+    torch.manual_seed(5)
+    C, H = 1024, 8       # head_dim 128 as in Infinity-2B
+    hw = [(p, p) for p in (1, 2, 4, 6, 8, 12, 16, 20)]
+    total = sum(h * w for h, w in hw)
+    rope = hooks.rope2d_tables(C // H, hw)
+    kw = dict(embed_dim=C, num_heads=H, layout='BHLc', q_bits=4, quant_method='G_GROUP', group_size=128,
+              symmetric=False, enable_quantization=True, max_tokens=total)
+    a_mod = hooks.InfinitySelfAttention(fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.InfinitySelfAttention(fused=True, **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    start = 0
+    for h, w in hw:
+        note('hooks infinity fused', h, w)
+        x = torch.randn(2, h * w, C, device=dev, dtype=torch.bfloat16)
+        a = a_mod(x, rope=rope, token_start=start).float()
+        b = b_mod(x, rope=rope, token_start=start).float()
+        start += h * w
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), ((h, w), (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995
+    assert torch.equal(a_mod.k_quant.dequant_all(), b_mod.packed_cache.dequant('k'))
+
+
+def test_unquantized_cache_path_matches_full_sequence_attention(dev):
+    """Caching without quantization equals one full-sequence call under the
+    block-causal mask of VAR/models/var.py:110-114."""
+    torch.manual_seed(6)
+    C, H = 128, 2
+    pn = (1, 2, 3)
+    m = hooks.VarSelfAttention(0, C, H, layout='BHLc', max_tokens=14).to(dev)
+    xs = [torch.randn(1, p * p, C, device=dev) for p in pn]
+    m.kv_caching(True)
+    steps = torch.cat([m(x) for x in xs], dim=1)
+    m.kv_caching(False)
+    L = sum(p * p for p in pn)
+    bias = O.block_causal_bias(pn).to(dev).view(1, 1, L, L)
+    full = m(torch.cat(xs, dim=1), attn_bias=bias)
+    assert torch.allclose(steps, full, atol=2e-5)

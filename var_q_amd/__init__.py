@@ -9,4 +9,4 @@ from ._lib import VarqError, load as load_library  # noqa: F401
 from .quant import VAR_Q  # noqa: F401
 from .config_loader import VARQConfig, load_varq_config  # noqa: F401
 from .kv_cache import PackedKVCache  # noqa: F401
-from . import ops, schedules  # noqa: F401
+from . import hooks, ops, schedules  # noqa: F401

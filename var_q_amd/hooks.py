@@ -1,0 +1,232 @@
+"""Self-attention modules that carry the VAR-Q hook, on random weights.
+
+They reproduce the inference-time contract of the two call sites of the
+reference quantizer,
+
+  * VAR:       VAR/models/basic_var.py:70-165  (`SelfAttention`)
+  * Infinity:  Infinity/infinity/models/basic.py:205-351 (`SelfAttention`),
+               2-D rotary embedding basic.py:44-123
+
+i.e. `kv_caching(True)` creates one K and one V quantizer, `forward` projects
+x to q/k/v, normalises (and rotates) q and k, pushes k and v through the
+quantized cache and attends with the current scale's queries over everything
+cached.  Two backends behind the same interface:
+
+  * `fused=False`: the drop-in `VAR_Q.use_var_q` (dequantized full-length K/V
+    out) followed by scaled-dot-product attention, which is what the reference
+    modules do with flash-attn / xformers / their `slow_attn`;
+  * `fused=True`: `PackedKVCache.append` + `PackedKVCache.attend`: the step is
+    quantized in place into a pre-allocated packed cache and attention reads the
+    packed codes; no dequantized K/V exists.  Needs a row-local quantizer
+    (`quant_method='G_GROUP'`).
+
+The transformer blocks around the attention (AdaLN, FFN, cross-attention) are
+outside this package.
+"""
+import math
+from typing import Callable, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .kv_cache import PackedKVCache
+from .quant import VAR_Q
+
+
+def rope2d_tables(head_dim: int, scale_hw: Sequence[Tuple[int, int]], normalized_by_hw: int = 2,
+                  base: float = 10000.0, max_hw: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos, sin [sum(h*w), head_dim/2] of the 2-D rotary embedding for a scale
+    schedule [(h, w), ...]: the first half of the rotated pairs turns with the
+    token's row, the second half with its column, frequencies
+    base^(-2j/(head_dim/2)) (Infinity/infinity/models/basic.py:44-97).
+    normalized_by_hw = 0: grid coordinates as they are; 2: coordinates scaled to
+    the last scale's grid and rounded (the released models' setting); 1
+    (bilinear resampling of the table) is not provided."""
+    assert head_dim % 4 == 0
+    if normalized_by_hw not in (0, 2):
+        raise ValueError('normalized_by_hw must be 0 or 2 (got %r)' % (normalized_by_hw,))
+    half = head_dim // 2
+    inv_freq = 1.0 / (base ** (torch.arange(0, half, 2, dtype=torch.int64).float() / half))   # [half/2]
+    pos = torch.arange(max_hw, dtype=torch.int64).float()
+    ang = torch.outer(pos, inv_freq)                                                         # [max_hw, half/2]
+    uh, uw = scale_hw[-1]
+    cos, sin = [], []
+    for h, w in scale_hw:
+        if normalized_by_hw == 2:
+            ys = (torch.arange(h) * (uh / h)).round().long()
+            xs = (torch.arange(w) * (uw / w)).round().long()
+        else:
+            ys, xs = torch.arange(h), torch.arange(w)
+        a = torch.cat([ang[ys][:, None, :].expand(h, w, -1), ang[xs][None, :, :].expand(h, w, -1)], dim=-1)
+        a = a.reshape(h * w, half)
+        cos.append(torch.cos(a))
+        sin.append(torch.sin(a))
+    return torch.cat(cos), torch.cat(sin)
+
+
+def apply_rope2d(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, start: int, l_dim: int) -> torch.Tensor:
+    """Rotate adjacent channel pairs (2i, 2i+1) of x (fp32) by the angles of tokens
+    start..start+L (basic.py:103-123).  l_dim is the token axis of x."""
+    L = x.shape[l_dim]
+    shape = [1] * x.dim()
+    shape[l_dim], shape[-1] = L, x.shape[-1] // 2
+    c = cos[start:start + L].to(x.device).view(shape)
+    s = sin[start:start + L].to(x.device).view(shape)
+    x2 = x.float().reshape(*x.shape[:-1], -1, 2)
+    out = torch.stack([c * x2[..., 0] - s * x2[..., 1], s * x2[..., 0] + c * x2[..., 1]], dim=-1)
+    return out.reshape(x.shape)
+
+
+class _QuantizedSelfAttention(nn.Module):
+    """Common part: qkv projection, quantized cache, attention, output projection."""
+
+    def __init__(self, embed_dim: int, num_heads: int, layout: str, q_bits, quant_method: str, enable_quantization: bool,
+                 fused: bool, group_size: Optional[int], symmetric: bool, max_tokens: int, block_idx: int,
+                 quantizer_factory: Optional[Callable] = None):
+        super().__init__()
+        assert embed_dim % num_heads == 0 and layout in ('BLHc', 'BHLc')
+        self.num_heads, self.head_dim = num_heads, embed_dim // num_heads
+        self.layout, self.block_idx = layout, block_idx
+        self.q_bits, self.quant_method, self.enable_quantization = q_bits, quant_method, enable_quantization
+        self.fused, self.group_size, self.symmetric, self.max_tokens = fused, group_size, symmetric, max_tokens
+        self._quantizer_factory = quantizer_factory or VAR_Q
+        if fused:
+            assert enable_quantization and quant_method == 'G_GROUP' and group_size, \
+                'the fused backend needs the row-local group-wise quantizer (quant_method="G_GROUP", group_size=g)'
+        self.mat_qkv = nn.Linear(embed_dim, embed_dim * 3, bias=False)
+        self.q_bias, self.v_bias = nn.Parameter(torch.zeros(embed_dim)), nn.Parameter(torch.zeros(embed_dim))
+        self.register_buffer('zero_k_bias', torch.zeros(embed_dim))
+        self.proj = nn.Linear(embed_dim, embed_dim)
+        self.caching, self.cached_k, self.cached_v = False, None, None
+        self.k_quant = self.v_quant = None
+        self.packed_cache: Optional[PackedKVCache] = None
+
+    # -- cache life cycle (basic_var.py:104-117, basic.py:254-271) ---------------------
+    def kv_caching(self, enable: bool):
+        self.caching, self.cached_k, self.cached_v = enable, None, None
+        self.k_quant = self.v_quant = None
+        self.packed_cache = None
+        if enable and self.enable_quantization and not self.fused:
+            kw = dict(quant_bits=self.q_bits, qkv_format=self.layout, quant_method=self.quant_method, blk_idx=self.block_idx)
+            if self.quant_method == 'G_GROUP' or not self.symmetric:
+                kw.update(group_size=self.group_size, symmetric=self.symmetric)
+            self.k_quant = self._quantizer_factory(**kw)
+            self.v_quant = self._quantizer_factory(**kw)
+
+    def _project(self, x):
+        B, L, _ = x.shape
+        bias = torch.cat((self.q_bias, self.zero_k_bias, self.v_bias))
+        qkv = F.linear(x, self.mat_qkv.weight.to(x.dtype), bias.to(x.dtype)).view(B, L, 3, self.num_heads, self.head_dim)
+        if self.layout == 'BLHc':
+            return qkv.unbind(dim=2)                       # each [B,L,H,c]
+        return qkv.permute(2, 0, 3, 1, 4).unbind(dim=0)     # each [B,H,L,c]
+
+    def _attend(self, q, k, v, scale: float, attn_bias, out_dtype):
+        """q, k, v in self.layout (k, v full length); returns [B,L,C]."""
+        B = q.shape[0]
+        if self.layout == 'BLHc':
+            q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+        L = q.shape[2]
+        o = F.scaled_dot_product_attention(q.to(out_dtype), k.to(out_dtype), v.to(out_dtype), scale=scale,
+                                           attn_mask=None if attn_bias is None else attn_bias.to(out_dtype))
+        return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim)
+
+    def _cache_and_attend(self, q, k, v, scale: float, attn_bias, out_dtype):
+        B = q.shape[0]
+        l_dim = 1 if self.layout == 'BLHc' else 2
+        L = q.shape[l_dim]
+        if self.caching and self.fused:
+            if attn_bias is not None:
+                raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')
+            if self.packed_cache is None:
+                self.packed_cache = PackedKVCache(B, self.num_heads, self.max_tokens, self.head_dim, self.q_bits,
+                                                  self.group_size, q.device, symmetric=self.symmetric)
+            self.packed_cache.append(k, v, layout=self.layout)
+            qh = q if self.layout == 'BHLc' else q.transpose(1, 2)
+            o = self.packed_cache.attend(qh.to(torch.bfloat16).contiguous(), scale)       # [B,H,L,c]
+            return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
+        if self.caching:
+            if self.enable_quantization:
+                k = self.k_quant.use_var_q(k)
+                v = self.v_quant.use_var_q(v)
+            elif self.cached_k is None:
+                self.cached_k, self.cached_v = k, v
+            else:
+                k = self.cached_k = torch.cat((self.cached_k, k), dim=l_dim)
+                v = self.cached_v = torch.cat((self.cached_v, v), dim=l_dim)
+        return self._attend(q, k, v, scale, attn_bias, out_dtype)
+
+
+class VarSelfAttention(_QuantizedSelfAttention):
+    """VAR/models/basic_var.py:70-165.  attn_l2_norm=True (the released VAR-d16..d30
+    setting): q and k are l2-normalised, q is multiplied by a per-head
+    exp(min(param, ln 100)), softmax scale 1; else scale 0.25/sqrt(c)."""
+
+    def __init__(self, block_idx: int, embed_dim: int = 1024, num_heads: int = 16, attn_l2_norm: bool = True,
+                 layout: str = 'BLHc', q_bits=8, quant_method: str = 'G_SCALE_HEAD_DIM', enable_quantization: bool = False,
+                 fused: bool = False, group_size: Optional[int] = None, symmetric: bool = True, max_tokens: int = 680,
+                 quantizer_factory: Optional[Callable] = None):
+        super().__init__(embed_dim, num_heads, layout, q_bits, quant_method, enable_quantization, fused, group_size,
+                         symmetric, max_tokens, block_idx, quantizer_factory)
+        self.attn_l2_norm = attn_l2_norm
+        if attn_l2_norm:
+            self.scale = 1.0
+            self.scale_mul_1H11 = nn.Parameter(torch.full((1, num_heads, 1, 1), 4.0).log())
+            self.max_scale_mul = math.log(100.0)
+        else:
+            self.scale = 0.25 / math.sqrt(self.head_dim)
+
+    def forward(self, x: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        q, k, v = self._project(x)
+        main_type = x.dtype
+        if self.attn_l2_norm:
+            scale_mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp()
+            if self.layout == 'BLHc':
+                scale_mul = scale_mul.transpose(1, 2)
+            q = F.normalize(q.float(), dim=-1).mul(scale_mul)
+            k = F.normalize(k.float(), dim=-1)
+        o = self._cache_and_attend(q, k, v, self.scale, attn_bias, main_type)
+        return self.proj(o.to(self.proj.weight.dtype))
+
+
+class InfinitySelfAttention(_QuantizedSelfAttention):
+    """Infinity/infinity/models/basic.py:205-351: cos_attn (l2-normalised q, k with
+    a per-head multiplier, scale 1) or scale 1/sqrt(c)/tau; 2-D rotary embedding of
+    q and k before the cache; K reaches the quantizer in fp32, V in the compute
+    dtype."""
+
+    def __init__(self, embed_dim: int = 2048, num_heads: int = 16, tau: float = 1.0, cos_attn: bool = True,
+                 layout: str = 'BHLc', q_bits=8, quant_method: str = 'G_SCALE_HEAD_DIM', enable_quantization: bool = False,
+                 fused: bool = False, group_size: Optional[int] = None, symmetric: bool = True, max_tokens: int = 10521,
+                 block_idx: int = 0, quantizer_factory: Optional[Callable] = None):
+        super().__init__(embed_dim, num_heads, layout, q_bits, quant_method, enable_quantization, fused, group_size,
+                         symmetric, max_tokens, block_idx, quantizer_factory)
+        self.tau, self.cos_attn = tau, cos_attn
+        if cos_attn:
+            self.scale = 1.0
+            size = (1, 1, num_heads, 1) if layout == 'BLHc' else (1, num_heads, 1, 1)
+            self.scale_mul_1H11 = nn.Parameter(torch.full(size, 4.0).log())
+            self.max_scale_mul = math.log(100.0)
+        else:
+            self.scale = 1.0 / math.sqrt(self.head_dim) / tau
+
+    def forward(self, x: torch.Tensor, attn_bias: Optional[torch.Tensor] = None,
+                rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, token_start: int = 0) -> torch.Tensor:
+        """rope = (cos, sin) from rope2d_tables for the whole schedule; token_start =
+        number of tokens of the scales before this one."""
+        q, k, v = self._project(x)
+        main_type = x.dtype
+        if self.cos_attn:
+            scale_mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp()
+            q = F.normalize(q.float(), dim=-1, eps=1e-12).mul(scale_mul).contiguous()
+            k = F.normalize(k.float(), dim=-1, eps=1e-12).contiguous()
+            v = v.contiguous()
+        else:
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if rope is not None:
+            l_dim = 1 if self.layout == 'BLHc' else 2
+            q = apply_rope2d(q, rope[0], rope[1], token_start, l_dim)
+            k = apply_rope2d(k, rope[0], rope[1], token_start, l_dim)
+        o = self._cache_and_attend(q, k, v, self.scale, attn_bias, main_type)
+        return self.proj(o.to(self.proj.weight.dtype))

@@ -44,15 +44,25 @@ class PackedKVCache:
     def reset(self):
         self.len = 0
 
-    def append(self, k: torch.Tensor, v: torch.Tensor):
-        """Quantize + pack one step [B,H,n,D] into tokens len..len+n of the cache."""
-        B, H, n, D = k.shape
+    def append(self, k: torch.Tensor, v: torch.Tensor, layout: str = 'BHLc'):
+        """Quantize + pack one step into tokens len..len+n of the cache.  The step is
+        [B,H,n,D] (layout 'BHLc') or [B,n,H,D] ('BLHc', the flash-attention layout of
+        VAR/models/basic_var.py:127-131); either is read where it lies."""
+        assert layout in ('BHLc', 'BLHc')
+        if layout == 'BHLc':
+            B, H, n, D = k.shape
+        else:
+            B, n, H, D = k.shape
         assert (B, H, D) == (self.B, self.H, self.D) and v.shape == k.shape
         assert self.len + n <= self.Lmax, 'cache overflow'
         k, v = k.contiguous(), v.contiguous()
         for c in self.classes:
             hc = len(c.heads)
-            rowmap = [B, H, n, hc * self.Lmax, self.Lmax, 1, self.len, 1]
+            # input rows in memory order -> output row b*hc*Lmax + slot(h)*Lmax + len + l
+            if layout == 'BHLc':
+                rowmap = [B, H, n, hc * self.Lmax, self.Lmax, 1, self.len, 1]
+            else:
+                rowmap = [B, n, H, hc * self.Lmax, 1, self.Lmax, self.len, 2]
             asym = not self.symmetric
             ops.quant_pack_rows_into(k, self.group, c.bits, asym, self.eps, c.k_words, c.k_scale,
                                      c.k_zp if asym else None, rowmap, c.slot)
