@@ -58,3 +58,35 @@ def test_overflow_is_refused(dev):
     cache.append(x, x)
     with pytest.raises(AssertionError):
         cache.append(x, x)
+
+
+def test_descriptor_save_load_round_trip(dev, tmp_path):
+    """The hand-over format: descriptor + named buffers; a cache written to a file and
+    read back (into a larger capacity) holds the same codes and attends identically."""
+    import json
+    g = torch.Generator().manual_seed(77)
+    B, H, D = 2, 6, 64
+    bits = [8, 4, 2, 4, 8, 2]
+    cache = PackedKVCache(B, H, 40, D, bits, 32, dev)
+    for n in (1, 4, 9, 16):
+        note('kv_cache save/load append', n)
+        cache.append(torch.randn(B, H, n, D, generator=g).to(dev), torch.randn(B, H, n, D, generator=g).to(dev))
+    d = cache.descriptor()
+    json.dumps(d)                                     # serialisable
+    assert d['len'] == 30 and d['per_head_bits'] == bits and [c['bits'] for c in d['classes']] == [2, 4, 8]
+    for c in d['classes']:
+        assert c['meta'] == {'orig_c': D, 'vals_per_word': 32 // c['bits'], 'pad_len': 0, 'bits': c['bits']}
+        assert c['words']['shape'] == [B, len(c['heads']), 40, D * c['bits'] // 32]
+        assert tuple(cache.tensors()['b%d.k_words' % c['bits']].shape) == tuple(c['words']['shape'])
+    path = str(tmp_path / 'cache.safetensors')
+    cache.save(path)
+    back = PackedKVCache.load(path, dev, Lmax=64)
+    assert back.len == 30 and back.Lmax == 64 and back.per_head_bits == bits
+    assert torch.equal(back.dequant('k'), cache.dequant('k')) and torch.equal(back.dequant('v'), cache.dequant('v'))
+    q = torch.randn(B, H, 16, D, generator=g).to(dev).bfloat16()
+    assert torch.equal(back.attend(q, 0.125), cache.attend(q, 0.125))
+    # and it keeps growing where the saved one stopped
+    k, v = torch.randn(B, H, 5, D, generator=g).to(dev), torch.randn(B, H, 5, D, generator=g).to(dev)
+    back.append(k, v)
+    cache.append(k, v)
+    assert torch.equal(back.dequant('k'), cache.dequant('k'))

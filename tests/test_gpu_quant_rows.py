@@ -135,3 +135,25 @@ def test_row_map_appends_into_cache(dev):
     assert torch.equal(words[:, :, :off].cpu(), O.pack_last_dim(q, bits)[0])
     assert torch.equal(scale[:, :, :off].cpu(), s) and torch.equal(zp[:, :, :off].cpu(), z)
     assert int(words[:, :, off:].abs().sum()) == 0           # nothing written past the end
+
+
+@pytest.mark.parametrize('bits,sym', [(8, True), (4, False), (2, False)])
+def test_error_statistics_match_the_oracle(dev, bits, sym, tmp_path):
+    """Range and L2-normalised error figures (var_q_amd/stats.py) against the same
+    quantities computed from the oracle's codes on the CPU."""
+    from var_q_amd.stats import CsvReport, quant_error_stats
+    g = torch.Generator().manual_seed(bits)
+    x = O.synth_kv((2, 3, 50, 128), 11, 'student4', 0.01, 20.0, torch.bfloat16, outlier_seed=12)
+    note('quant stats', bits, sym)
+    st = quant_error_stats(x.to(dev), 64, bits, sym, tag='k')
+    q, s, z = O.quant_groupwise(x, 64, bits, not sym)
+    deq = O.dequant_groupwise(q, s, z, 64)
+    want = (torch.linalg.vector_norm((x.float() - deq).double()) / torch.linalg.vector_norm(x.double())).item()
+    assert st['l2_norm_error'] == pytest.approx(want, rel=1e-6)
+    assert st['max_abs_error'] == pytest.approx((x.float() - deq).abs().max().item(), rel=1e-6)
+    assert st['scale_max'] == s.max().item() and st['scale_min'] == s.min().item()
+    assert st['x_min'] == x.float().min().item() and st['x_max'] == x.float().max().item()
+    assert st['n_groups'] == s.numel() and st['max_abs_error_in_steps'] <= 0.5 + 1e-3 or not sym
+    rep = CsvReport(str(tmp_path / 'r.csv'))
+    rep.add(st)
+    assert float(rep.rows()[0]['l2_norm_error']) == pytest.approx(want, rel=1e-6)

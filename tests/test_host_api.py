@@ -58,7 +58,8 @@ def test_reference_import_names_resolve():
 
 
 @pytest.mark.parametrize('name,infinity', [('VAR-VAR_Q-8.json', False), ('Infinity-VAR_Q-8.json', True),
-                                           ('VAR-raw.json', False), ('Infinity-VAR_Q-4-g128.json', True)])
+                                           ('VAR-raw.json', False), ('Infinity-VAR_Q-4-g128.json', True),
+                                           ('Infinity-VAR_Q-mixed-g64.json', True)])
 def test_config_loader(name, infinity, tmp_path):
     cfg = load_varq_config(os.path.join(PKG, name))
     assert cfg.is_infinity_model() == infinity and cfg.is_var_model() != infinity
@@ -84,6 +85,26 @@ def test_config_loader(name, infinity, tmp_path):
     assert json.load(open(out)) == cfg.config
 
 
+def test_extended_quantization_schema_is_validated(tmp_path):
+    cfg = load_varq_config(os.path.join(PKG, 'Infinity-VAR_Q-mixed-g64.json'))
+    kw = cfg.packed_cache_kwargs(B=2, H=16, Lmax=100, D=128)
+    assert kw['bits'] == cfg.config['quantization']['per_head_bits'] and kw['group_size'] == 64 and kw['symmetric'] is False
+    with pytest.raises(ValueError, match='16 entries for 8 heads'):
+        cfg.packed_cache_kwargs(B=2, H=8, Lmax=100, D=128)
+    for bad, pat in (({'q_bits': 9}, 'q_bits'), ({'qkv_format': 'LBHc'}, 'qkv_format'), ({'symmetric': 'no'}, 'symmetric'),
+                     ({'group_size': 0}, 'group_size'), ({'per_head_bits': [4, 3]}, 'per_head_bits'),
+                     ({'quant_method': 'G_TOKEN_HEAD'}, 'per_head_bits')):
+        c = load_varq_config(os.path.join(PKG, 'Infinity-VAR_Q-mixed-g64.json'))
+        c.update_config({'quantization': bad})
+        with pytest.raises(ValueError, match=pat):
+            c.validate_quantization()
+    # the reference's rule files stay valid and do not describe a packed cache
+    ref = load_varq_config(os.path.join(PKG, 'Infinity-VAR_Q-8.json'))
+    ref.validate_quantization()
+    with pytest.raises(ValueError, match='G_GROUP'):
+        ref.packed_cache_kwargs(2, 16, 100, 128)
+
+
 def test_schedules_and_kv_limit():
     assert schedules.total_tokens(schedules.VAR_PATCH_NUMS) == 680
     assert schedules.total_tokens(schedules.INFINITY_PATCH_NUMS) == 10521
@@ -92,3 +113,14 @@ def test_schedules_and_kv_limit():
     assert schedules.kv_limit((1, 2, 3), q_start=5).tolist() == [14] * 9
     import varq_oracle as O
     assert torch.equal(schedules.kv_limit(O.VAR_PATCH_NUMS), O.kv_limit_from_schedule(O.VAR_PATCH_NUMS))
+
+
+def test_csv_report_appends_rows(tmp_path):
+    from var_q_amd.stats import CsvReport, FIELDS
+    path = str(tmp_path / 'q.csv')
+    rep = CsvReport(path)
+    rep.add({'tag': 'k', 'bits': 4, 'l2_norm_error': 0.125})
+    CsvReport(path).add({'tag': 'v', 'bits': 2})          # reopening keeps the header and the rows
+    rows = rep.rows()
+    assert [r['tag'] for r in rows] == ['k', 'v'] and rows[0]['l2_norm_error'] == '0.125' and rows[1]['bits'] == '2'
+    assert list(rows[0].keys()) == FIELDS

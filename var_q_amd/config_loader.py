@@ -74,17 +74,53 @@ class VARQConfig:
         with open(save_path, 'w') as f:
             json.dump(self.config, f, indent=2)
 
+    # -- extended `quantization` keys (a superset of the reference's JSON rule files) ---
+    #   symmetric      bool, default true    max-abs (reference) or min-max affine codes
+    #   group_size     int                   channels per group for quant_method "G_GROUP"
+    #   per_head_bits  list of H ints in {2,4,8}: mixed precision, packed cache only
+    def validate_quantization(self) -> Dict[str, Any]:
+        """The `quantization` section, checked; raises ValueError naming the bad key."""
+        qc = self.get_quantization_config()
+        bits = qc.get('q_bits', 8)
+        if not (isinstance(bits, int) and 1 < bits <= 8):
+            raise ValueError('quantization.q_bits must be an int in (1, 8], got %r' % (bits,))
+        if qc.get('qkv_format', 'BLHc') not in ('BLHc', 'BHLc'):
+            raise ValueError('quantization.qkv_format must be "BLHc" or "BHLc", got %r' % (qc.get('qkv_format'),))
+        if 'symmetric' in qc and not isinstance(qc['symmetric'], bool):
+            raise ValueError('quantization.symmetric must be true or false')
+        if qc.get('quant_method') == 'G_GROUP' and not (isinstance(qc.get('group_size'), int) and qc['group_size'] > 0):
+            raise ValueError('quantization.quant_method "G_GROUP" needs a positive integer group_size')
+        if 'per_head_bits' in qc:
+            phb = qc['per_head_bits']
+            if not (isinstance(phb, list) and phb and all(b in (2, 4, 8) for b in phb)):
+                raise ValueError('quantization.per_head_bits must be a non-empty list over {2, 4, 8}')
+            if qc.get('quant_method') != 'G_GROUP':
+                raise ValueError('quantization.per_head_bits needs quant_method "G_GROUP" (packed cache)')
+        return qc
+
     def quantizer_kwargs(self) -> Dict[str, Any]:
         """Constructor arguments for quant.VAR_Q from the `quantization` section
         (the four keys the reference threads into its attention blocks,
         VAR/models/__init__.py:108-111, plus the extended keys)."""
-        qc = self.get_quantization_config()
+        qc = self.validate_quantization()
         kw = {'quant_bits': qc.get('q_bits', 8), 'qkv_format': qc.get('qkv_format', 'BLHc'),
               'quant_method': qc.get('quant_method', 'G_SCALE_HEAD_DIM')}
         for src, dst in (('symmetric', 'symmetric'), ('group_size', 'group_size')):
             if src in qc:
                 kw[dst] = qc[src]
         return kw
+
+    def packed_cache_kwargs(self, B: int, H: int, Lmax: int, D: int) -> Dict[str, Any]:
+        """Constructor arguments for kv_cache.PackedKVCache (needs the row-local
+        group-wise quantizer, i.e. quant_method "G_GROUP")."""
+        qc = self.validate_quantization()
+        if qc.get('quant_method') != 'G_GROUP':
+            raise ValueError('the packed cache needs quantization.quant_method "G_GROUP"')
+        bits = qc.get('per_head_bits', qc.get('q_bits', 8))
+        if isinstance(bits, list) and len(bits) != H:
+            raise ValueError('quantization.per_head_bits has %d entries for %d heads' % (len(bits), H))
+        return {'B': B, 'H': H, 'Lmax': Lmax, 'D': D, 'bits': bits, 'group_size': qc['group_size'],
+                'symmetric': qc.get('symmetric', True)}
 
 
 def load_varq_config(config_path: str = None) -> VARQConfig:

@@ -7,7 +7,8 @@ quantized straight into its slot of the cache.  Heads may carry different
 bit-widths; heads of equal width share one dense buffer ("class") and a table
 maps each head to (class, slot).  Layout BHLc: K/V steps are [B, H, n, D].
 """
-from typing import List, Optional, Sequence, Union
+import json
+from typing import Any, Dict, List, Optional, Sequence, Union
 
 import torch
 
@@ -43,6 +44,72 @@ class PackedKVCache:
 
     def reset(self):
         self.len = 0
+
+    # -- hand-over format ---------------------------------------------------------------
+    FORMAT_VERSION = 1
+
+    def descriptor(self) -> Dict[str, Any]:
+        """JSON-serialisable description of the packed cache: everything a consumer
+        needs to address and decode the buffers of `tensors()`.  Per bit-width class it
+        repeats the `meta` dictionary of the reference's pack functions
+        (VAR_Q/pack_unpack.py:133: orig_c, vals_per_word, pad_len, bits)."""
+        ns = self.D // self.group
+        return {
+            'format': 'varq-packed-kv', 'version': self.FORMAT_VERSION, 'layout': 'BHLc',
+            'B': self.B, 'H': self.H, 'Lmax': self.Lmax, 'D': self.D, 'len': self.len,
+            'group_size': self.group, 'symmetric': self.symmetric, 'eps': self.eps,
+            'per_head_bits': list(self.per_head_bits),
+            'field_order': 'code j of a word at bits [j*bits, (j+1)*bits), two\'s complement',
+            'dequant': '(code - zp) * scale' if not self.symmetric else 'code * scale',
+            'classes': [{
+                'bits': c.bits, 'heads': list(c.heads),
+                'words': {'name': f'b{c.bits}.{{k,v}}_words', 'dtype': 'int32',
+                          'shape': [self.B, len(c.heads), self.Lmax, self.D * c.bits // 32]},
+                'scale': {'name': f'b{c.bits}.{{k,v}}_scale', 'dtype': 'float32',
+                          'shape': [self.B, len(c.heads), self.Lmax, ns]},
+                'zp': None if self.symmetric else {'name': f'b{c.bits}.{{k,v}}_zp', 'dtype': 'float32',
+                                                   'shape': [self.B, len(c.heads), self.Lmax, ns]},
+                'meta': {'orig_c': self.D, 'vals_per_word': 32 // c.bits, 'pad_len': 0, 'bits': c.bits},
+            } for c in self.classes],
+        }
+
+    def tensors(self) -> Dict[str, torch.Tensor]:
+        """The cache buffers under the names the descriptor uses (no copies)."""
+        out = {}
+        for c in self.classes:
+            for kv in 'kv':
+                out[f'b{c.bits}.{kv}_words'] = getattr(c, f'{kv}_words')
+                out[f'b{c.bits}.{kv}_scale'] = getattr(c, f'{kv}_scale')
+                if not self.symmetric:
+                    out[f'b{c.bits}.{kv}_zp'] = getattr(c, f'{kv}_zp')
+        return out
+
+    def save(self, path: str):
+        """Write the filled part of the cache (tokens 0..len-1) as one safetensors
+        file; the descriptor travels in the file's metadata."""
+        from safetensors.torch import save_file
+        desc = self.descriptor()
+        desc['Lmax_saved'] = self.len
+        data = {k: t[:, :, :self.len].contiguous().cpu() for k, t in self.tensors().items()}
+        save_file(data, path, metadata={'varq': json.dumps(desc)})
+
+    @classmethod
+    def load(cls, path: str, device, Lmax: Optional[int] = None) -> 'PackedKVCache':
+        """Rebuild a cache from `save`'s file (room for Lmax tokens, default: as saved
+        cache's capacity)."""
+        from safetensors import safe_open
+        with safe_open(path, framework='pt', device='cpu') as f:
+            desc = json.loads(f.metadata()['varq'])
+            if desc.get('format') != 'varq-packed-kv' or desc.get('version') != cls.FORMAT_VERSION:
+                raise ValueError('not a version-%d varq packed cache: %r' % (cls.FORMAT_VERSION, desc.get('format')))
+            cache = cls(desc['B'], desc['H'], Lmax or desc['Lmax'], desc['D'], desc['per_head_bits'], desc['group_size'],
+                        device, symmetric=desc['symmetric'], eps=desc['eps'])
+            n = desc['len']
+            assert n <= cache.Lmax, 'saved cache longer than the requested capacity'
+            for name, dst in cache.tensors().items():
+                dst[:, :, :n].copy_(f.get_tensor(name))
+            cache.len = n
+        return cache
 
     def append(self, k: torch.Tensor, v: torch.Tensor, layout: str = 'BHLc'):
         """Quantize + pack one step into tokens len..len+n of the cache.  The step is
