@@ -9,7 +9,7 @@
 // next-scale rule of VAR/models/var.py:110-114 expressed as a per-query key
 // limit.
 //
-// Design (one workgroup = 4 wavefronts = 128 queries of one (batch, head)):
+// Design (one workgroup = 8 wavefronts = 256 queries of one (batch, head)):
 //  * Both contractions run on v_mfma_f32_32x32x16_bf16 in transposed form,
 //    S^T = K Q^T and O^T = V^T P^T, so that a lane owns one query column: row
 //    max/sum are per-lane (one cross-half exchange per tile) and the S^T
@@ -51,7 +51,9 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(u32)))) u32 u32x4_t;
 
-constexpr int BM = 128;  // queries per workgroup (32 per wavefront)
+constexpr int NW = 8;          // wavefronts per workgroup
+constexpr int NT = NW * 64;    // threads per workgroup
+constexpr int BM = NW * 32;    // queries per workgroup (32 per wavefront)
 constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
@@ -238,7 +240,7 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
 };
 
 template <int D, int BITS, int GK, int GV>
-__global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
+__global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   constexpr int NSK = D / GK, NSV = D / GV;
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
@@ -285,6 +287,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   // ---- this lane's query ----------------------------------------------------
   const int qrow = qt * BM + wave * 32 + col;
   const bool q_live = qrow < p.Lq;
+  const bool wave_live = qt * BM + wave * 32 < p.Lq;   // wave-uniform
   const int qrow_c = q_live ? qrow : p.Lq - 1;
   const __bf16 *qptr = p.q + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow_c) * D;
   int limit = p.kv_limit ? min(p.kv_limit[qrow_c], p.Lk) : p.Lk;
@@ -358,7 +361,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   const u32 *vw = p.v_words + kv_row0 * WPR;
 
   constexpr int QUADS = BN * WPR / 4;                 // 16-byte pieces per packed tile
-  constexpr int LPT = (QUADS + 255) / 256;            // pieces per thread
+  constexpr int LPT = (QUADS + NT - 1) / NT;          // pieces per thread
   u32x4_t kreg[LPT], vreg[LPT];
   float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
 
@@ -366,8 +369,8 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
     const int t0 = tile * BN;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
-      const int piece = tid + i * 256;
-      if (LPT * 256 == QUADS || piece < QUADS) {
+      const int piece = tid + i * NT;
+      if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
         const int64_t off = (int64_t)key * WPR + (piece % (WPR / 4)) * 4;
         kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + off);
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
     // 3 - w, which puts the K and the V arithmetic of the single-group case on
     // different wavefronts
     {
-      const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = 3 - seg;
+      const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = NW - 1 - seg;
       if (seg < NSK) {
         const int64_t g = (kv_row0 + key) * NSK + seg;
         ksc = p.k_scale[g];
@@ -399,8 +402,8 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
     u32 *kp = lds_kp + sl * BN * RSK, *vp = lds_vp + sl * BN * RSV;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
-      const int piece = tid + i * 256;
-      if (LPT * 256 == QUADS || piece < QUADS) {
+      const int piece = tid + i * NT;
+      if (LPT * NT == QUADS || piece < QUADS) {
         const int key = piece / (WPR / 4), w4 = (piece % (WPR / 4)) * 4;
         constexpr u32 KX = KCodec<BITS>::kStageXor, VX = VCodec<BITS>::kStageXor;
         const u32x4_t kx = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
@@ -411,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
       }
     }
     float *par = lds_par + sl * L::kParFloats;
-    const int key = tid & 63, seg = tid >> 6, vseg = 3 - seg;
+    const int key = tid & 63, seg = tid >> 6, vseg = NW - 1 - seg;
     // |ck| is kept away from zero so that log2(vs)/ck stays finite for a constant group
     auto ck_of = [&](float ks) {
       const float c = ks * p.scale_log2e * KCodec<BITS>::kMul;
@@ -459,19 +462,18 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int s = 0; s < NSV; ++s) rowsel[s] = ((col == s) ? s : (s == 0 && col >= 4 && col < 7) ? col : 7) * RSR;
 
-  // packed V of `tile` -> V^T bf16: each thread takes 4 keys x 8 channels
+  // packed V of `tile` -> V^T bf16: a work item is 2 adjacent keys x 8 channels (one
+  // packed word of each key), written as 8 dwords of the transposed tile
   auto widen_v = [&](int tile) {
     const u32 *vp = lds_vp + (tile % 3) * BN * RSV;
     uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
-    for (int blk = tid; blk < (BN / 4) * (D / 8); blk += 256) {
-      const int kq = blk & (BN / 4 - 1), oct = blk / (BN / 4);
-      const u32 *row = &vp[kq * 4 * RSV];
-      u32 lo[8], hi[8];
-      VCodec<BITS>::pairs(row, row + RSV, oct, kmask, lo);
-      VCodec<BITS>::pairs(row + 2 * RSV, row + 3 * RSV, oct, kmask, hi);
+    for (int item = tid; item < (BN / 2) * (D / 8); item += NT) {
+      const int kp2 = item & (BN / 2 - 1), oct = item / (BN / 2);
+      const u32 *row = &vp[kp2 * 2 * RSV];
+      u32 pr[8];
+      VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        *reinterpret_cast<uint2 *>(&vt[(oct * 8 + j) * VTS + kq * 4]) = make_uint2(lo[j], hi[j]);
+      for (int j = 0; j < 8; ++j) *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * VTS + kp2 * 2]) = pr[j];
     }
   };
 
@@ -485,6 +487,18 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
   if (n_tiles > 0) widen_v(0);
   if (n_tiles > 2) prefetch(2);
   __syncthreads();
+
+  if (!wave_live) {
+    // a wavefront without queries (short query blocks) only helps with staging and
+    // widening, at the same barrier count as the others
+    for (int tile = 0; tile < n_tiles; ++tile) {
+      if (tile + 2 < n_tiles) stage(tile + 2);
+      if (tile + 3 < n_tiles) prefetch(tile + 3);
+      if (tile + 1 < n_tiles) widen_v(tile + 1);
+      __syncthreads();
+    }
+    return;
+  }
 
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int t0 = tile * BN;
@@ -517,6 +531,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
         }
 
       // ---- S^T = K Q^T for this 32-key block, K widened in registers -------------------
+      __builtin_amdgcn_s_setprio(1);
       floatx16_t sacc[NSK];
       const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
@@ -538,6 +553,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
             __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[ch / (GK / 16)], 0, 0, 0);
       }
 
+      __builtin_amdgcn_s_setprio(0);
       // requested now, used after the softmax arithmetic: V scales and the V^T operands
       // of the first 16-key chunk
       float svv[NSV][16];
@@ -641,6 +657,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
       // ---- O^T += V^T P'^T for the 32 keys of this block; one more MFMA per chunk and
       //      V group feeds the extra block: its row s collects the zero-point sum of group
       //      s and rows 4..6 (group 0 only) the softmax denominator ------------------------
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         u32x4_t av[NDB], aw[NSV];
@@ -669,6 +686,7 @@ __global__ __launch_bounds__(256, 2) void fused_attn_kernel(AttnParams p) {
         }
       }
 
+      __builtin_amdgcn_s_setprio(0);
       // between the two key blocks, with the first block's PV MFMAs in flight: widen
       // the next tile's V into the other V^T slot
       if (kb == 0 && tile + 1 < n_tiles) widen_v(tile + 1);
@@ -715,7 +733,7 @@ void launch(const AttnParams &p, hipStream_t st) {
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV>), grid, dim3(256), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV>), grid, dim3(NT), lds_bytes, st, p);
 }
 
 template <int D, int BITS>
