@@ -224,13 +224,13 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
 template <int D, int BITS, int GK, int GV> struct AttnLds {
   static constexpr int WPR = D * BITS / 32;
-  static constexpr int RSK = WPR + 4;       // packed K row stride (words): 16-byte rows
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
   static constexpr bool kFoldSv = (D / GV == 1);   // one V group: its scale rides inside the logits
   static constexpr int kParFloats = ((D / GK) + (kFoldSv ? 1 : 2) * (D / GV)) * 64;
   static constexpr int RSR = 64 + 8;        // stride (bf16) of the rows feeding the extra PV MFMA
-  static constexpr int kKp = 0;
-  static constexpr int kVp = kKp + 3 * 64 * RSK * 4;
+  static constexpr int KXS = D + 8;         // stride (bf16) of a widened K row: 16-byte rows, bank spread
+  static constexpr int kKx = 0;             // widened K, two tiles
+  static constexpr int kVp = kKx + 2 * 64 * KXS * 2;
   static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
   static constexpr int kKz = kVt + 2 * D * (64 + 8) * 2;          // rank-1 operands of S^T, 2 x 16 bytes per key and group
   static constexpr int kWz = kKz + 3 * (D / GK) * 64 * 32;        // 8 rows per slot for the extra PV MFMA
@@ -249,12 +249,14 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   using L = AttnLds<D, BITS, GK, GV>;
 
   // Pipelined LDS buffers (one workgroup barrier per tile):
-  //   packed K, packed V and the per-key parameters of tile t live in slot t % 3,
-  //   the widened V^T of tile t in slot t % 2.
-  // While tile t is being attended, V of tile t+1 is widened and tile t+2 is
-  // written from the registers it was loaded into one iteration earlier.
+  //   packed V and the per-key parameters of tile t live in slot t % 3, the
+  //   widened K and the widened V^T of tile t in slot t % 2.
+  // While tile t is being attended, K and V of tile t+1 are widened (K straight
+  // from the registers it was loaded into one iteration earlier, once per
+  // workgroup, so the eight wavefronts share the work) and packed V of tile t+2 is
+  // written from its registers.
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  u32 *const lds_kp = reinterpret_cast<u32 *>(lds_raw + L::kKp);          // [3][BN][RSK]
+  uint16_t *const lds_kx = reinterpret_cast<uint16_t *>(lds_raw + L::kKx);  // [2][BN][KXS] widened K codes (MFMA A operands)
   u32 *const lds_vp = reinterpret_cast<u32 *>(lds_raw + L::kVp);          // [3][BN][RSV]
   uint16_t *const lds_vt = reinterpret_cast<uint16_t *>(lds_raw + L::kVt);  // [2][D][VTS]  raw V codes, transposed
   u32x4_t *const lds_kz = reinterpret_cast<u32x4_t *>(lds_raw + L::kKz);  // [3][NSK][BN][2] rank-1 A operands (per lane half)
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   uint16_t *const lds_wz = reinterpret_cast<uint16_t *>(lds_raw + L::kWz);
   float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
   int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
-  constexpr int RSK = L::RSK, RSV = L::RSV;
+  constexpr int KXS = L::KXS, RSV = L::RSV;
   // parameter block of one tile: ck [NSK][BN]; vr [NSV][BN]; sv [NSV][BN] unless folded
   constexpr bool FOLD_SV = L::kFoldSv;
   constexpr int RSR = L::RSR;
@@ -365,6 +367,17 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   u32x4_t kreg[LPT], vreg[LPT];
   float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
 
+  auto prefetch_k = [&](int tile) {
+    const int t0 = tile * BN;
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int piece = tid + i * NT;
+      if (LPT * NT == QUADS || piece < QUADS) {
+        const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
+        kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + (int64_t)key * WPR + (piece % (WPR / 4)) * 4);
+      }
+    }
+  };
   auto prefetch = [&](int tile) {
     const int t0 = tile * BN;
 #pragma unroll
@@ -372,9 +385,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       const int piece = tid + i * NT;
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
-        const int64_t off = (int64_t)key * WPR + (piece % (WPR / 4)) * 4;
-        kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + off);
-        vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + off);
+        vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + (int64_t)key * WPR + (piece % (WPR / 4)) * 4);
       }
     }
     // scales: thread t handles key t % 64; wavefront w takes K group w and V group
@@ -399,15 +410,13 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // registers -> LDS slot of `tile` (packed words as they are, parameters precombined)
   auto stage = [&](int tile) {
     const int sl = tile % 3;
-    u32 *kp = lds_kp + sl * BN * RSK, *vp = lds_vp + sl * BN * RSV;
+    u32 *vp = lds_vp + sl * BN * RSV;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = piece / (WPR / 4), w4 = (piece % (WPR / 4)) * 4;
-        constexpr u32 KX = KCodec<BITS>::kStageXor, VX = VCodec<BITS>::kStageXor;
-        const u32x4_t kx = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
-        *reinterpret_cast<u32x4_t *>(&kp[key * RSK + w4]) = kx;
+        constexpr u32 VX = VCodec<BITS>::kStageXor;
         // V rows use an odd stride (bank spread for the column reads of the widening step)
 #pragma unroll
         for (int j = 0; j < 4; ++j) vp[key * RSV + w4 + j] = vreg[i][j] ^ VX;
@@ -477,12 +486,35 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     }
   };
 
-  // ---- prologue: tiles 0 and 1 staged, V of tile 0 widened, tile 2 in registers ------
+  // packed K of `tile` (in kreg) -> widened bf16 rows: each 16-byte piece holds OPQ octets
+  // of one key, every octet becomes one 16-byte MFMA A operand
+  auto widen_k = [&](int tile) {
+    uint16_t *kx = lds_kx + (tile & 1) * BN * KXS;
+    constexpr int OPQ = 16 / BITS;            // octets per 16-byte piece
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int piece = tid + i * NT;
+      if (LPT * NT == QUADS || piece < QUADS) {
+        const int key = piece / (WPR / 4), oct0 = (piece % (WPR / 4)) * OPQ;
+        constexpr u32 KX = KCodec<BITS>::kStageXor;
+        const u32 q4[4] = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
+#pragma unroll
+        for (int j = 0; j < OPQ; ++j) {
+          u32 a[4];
+          KCodec<BITS>::expand(q4, j, kmask, a);
+          *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
+        }
+      }
+    }
+  };
+
+  // ---- prologue: V tiles 0 and 1 staged, K and V of tile 0 widened, K of tile 1 and V
+  //      of tile 2 in registers ------------------------------------------------------------
   if (tid < 3) lds_flag[tid] = 0;
   if (tid < 3 * RSR) lds_wz[((tid / RSR) * 8 + 7) * RSR + tid % RSR] = 0;   // the all-zero row of each slot
   __syncthreads();
-  if (n_tiles > 0) { prefetch(0); stage(0); }
-  if (n_tiles > 1) { prefetch(1); stage(1); }
+  if (n_tiles > 0) { prefetch_k(0); prefetch(0); stage(0); widen_k(0); }
+  if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
   if (n_tiles > 0) widen_v(0);
   if (n_tiles > 2) prefetch(2);
@@ -494,202 +526,221 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     for (int tile = 0; tile < n_tiles; ++tile) {
       if (tile + 2 < n_tiles) stage(tile + 2);
       if (tile + 3 < n_tiles) prefetch(tile + 3);
-      if (tile + 1 < n_tiles) widen_v(tile + 1);
+      if (tile + 1 < n_tiles) { widen_v(tile + 1); widen_k(tile + 1); }
+      if (tile + 2 < n_tiles) prefetch_k(tile + 2);
       __syncthreads();
     }
     return;
   }
 
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const int t0 = tile * BN;
-    const u32 *kp = lds_kp + (tile % 3) * BN * RSK;
-    const float *par = lds_par + (tile % 3) * L::kParFloats;
-    const uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
-    const u32x4_t *kz = lds_kz + (tile % 3) * NSK * BN * 2;
-    const uint16_t *wz = lds_wz + (tile % 3) * 8 * RSR;
-    const bool tile_rem = lds_flag[tile % 3] == tile + 1;   // tagged with the tile, so stale tags never match
+  // ---- the three phases of one 32-key block, as lambdas over per-tile state --------
+  // LDS operands are requested ahead of their use where the registers allow it (the
+  // scheduling fences keep the requests where they are written).
+  constexpr bool HOIST = (NSK == 1 && NSV == 1);
+  int t0 = 0;
+  const uint16_t *kx = nullptr, *vt = nullptr, *wz = nullptr;
+  const float *par = nullptr;
+  const u32x4_t *kz = nullptr;
+  bool tile_rem = false, first = true;
+  // register i of this lane <-> key kb*32 + 16*(i/8) + 8*half + i%8 of the tile
+  floatx16_t sacc[2][NSK];
+  u32 pop[2][NSV][2][4];          // P'^T operands: p * vs as bf16, [block][V group][16-key chunk][dword]
+  float ckv[2][NSK][16], svv[2][NSV][16];
+  u32x4_t vta[NDB], wza[NSV];
 
+  auto begin_tile = [&](int tile) {
+    t0 = tile * BN;
+    kx = lds_kx + (tile & 1) * BN * KXS;
+    par = lds_par + (tile % 3) * L::kParFloats;
+    vt = lds_vt + (tile & 1) * D * VTS;
+    kz = lds_kz + (tile % 3) * NSK * BN * 2;
+    wz = lds_wz + (tile % 3) * 8 * RSR;
+    tile_rem = lds_flag[tile % 3] == tile + 1;   // tagged with the tile, so stale tags never match
     // slot (tile+2)%3 was last read during tile-1 (before the barrier): refill it
     if (tile + 2 < n_tiles) stage(tile + 2);
     if (tile + 3 < n_tiles) prefetch(tile + 3);
+  };
+  // with the PV MFMAs of a block in flight: widen the next tile's K and V into the other slots
+  auto widen_next = [&](int tile) {
+    if (tile + 1 < n_tiles) {
+      widen_v(tile + 1);
+      widen_k(tile + 1);
+      if (tile + 2 < n_tiles) prefetch_k(tile + 2);
+    }
+  };
+  auto load_scales = [&](int kb) {
+#pragma unroll
+    for (int s = 0; s < (HOIST ? NSK : 0); ++s)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
+        const float4 t = *reinterpret_cast<const float4 *>(&par[P_CK + s * BN + key]);
+        ckv[kb][s][4 * i4] = t.x; ckv[kb][s][4 * i4 + 1] = t.y; ckv[kb][s][4 * i4 + 2] = t.z; ckv[kb][s][4 * i4 + 3] = t.w;
+      }
+#pragma unroll
+    for (int s = 0; s < ((HOIST && !FOLD_SV) ? NSV : 0); ++s)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
+        const float4 t = *reinterpret_cast<const float4 *>(&par[P_SV + s * BN + key]);
+        svv[kb][s][4 * i4] = t.x; svv[kb][s][4 * i4 + 1] = t.y; svv[kb][s][4 * i4 + 2] = t.z; svv[kb][s][4 * i4 + 3] = t.w;
+      }
+  };
+  auto load_v_operands = [&](int kb, int c) {
+#pragma unroll
+    for (int d = 0; d < NDB; ++d)
+      vta[d] = *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
+#pragma unroll
+    for (int s = 0; s < NSV; ++s)
+      wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
+  };
 
+  // S^T = K Q^T for one 32-key block; the A operands are the widened K rows in LDS
+  auto qk = [&](int kb) {
+    __builtin_amdgcn_s_setprio(1);
+    const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      // LDS operands are requested well ahead of their use (the scheduling fences keep
-      // the requests where they are written): with two wavefronts per SIMD there is
-      // little else to cover the LDS latency.  Only where the registers allow it.
-      constexpr bool HOIST = (NSK == 1 && NSV == 1);
-      // register i of this lane <-> key kb*32 + 16*(i/8) + 8*half + i%8 of the tile
-      float ckv[NSK][16];
+    for (int s = 0; s < NSK; ++s) {
+      // starts the accumulator with the zero-point term (see bq above)
+      floatx16_t zero;
 #pragma unroll
-      for (int s = 0; s < (HOIST ? NSK : 0); ++s)
+      for (int j = 0; j < 16; ++j) zero[j] = 0.f;
+      sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
+                                                            __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+    }
+    const uint16_t *krow = &kx[krow_i * KXS];
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
-          const float4 t = *reinterpret_cast<const float4 *>(&par[P_CK + s * BN + key]);
-          ckv[s][4 * i4] = t.x; ckv[s][4 * i4 + 1] = t.y; ckv[s][4 * i4 + 2] = t.z; ckv[s][4 * i4 + 3] = t.w;
-        }
+    for (int ch = 0; ch < NCH; ++ch) {
+      const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[k_octet<GK>(ch, half) * 8]);
+      sacc[kb][ch / (GK / 16)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][ch / (GK / 16)], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+  };
 
-      // ---- S^T = K Q^T for this 32-key block, K widened in registers -------------------
-      __builtin_amdgcn_s_setprio(1);
-      floatx16_t sacc[NSK];
-      const int krow_i = kb * 32 + kperm(col);
+  // logits -> P'^T operands of one block: online softmax against a lazily moved reference
+  auto softmax = [&](int kb) {
+    float z[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float v = -m_ref;
 #pragma unroll
       for (int s = 0; s < NSK; ++s) {
-        // starts the accumulator with the zero-point term (see bq above)
-        floatx16_t zero;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) zero[j] = 0.f;
-        sacc[s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
-                                                          __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+        const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+        v = __builtin_fmaf(HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key], sacc[kb][s][i], v);
       }
-      const u32 *krow = &kp[krow_i * RSK];
-#pragma unroll
-      for (int ch = 0; ch < NCH; ++ch) {
-        u32 a[4];
-        KCodec<BITS>::expand(krow, k_octet<GK>(ch, half), kmask, a);
-        const u32x4_t av = {a[0], a[1], a[2], a[3]};
-        sacc[ch / (GK / 16)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[ch / (GK / 16)], 0, 0, 0);
-      }
-
-      __builtin_amdgcn_s_setprio(0);
-      // requested now, used after the softmax arithmetic: V scales and the V^T operands
-      // of the first 16-key chunk
-      float svv[NSV][16];
-#pragma unroll
-      for (int s = 0; s < ((HOIST && !FOLD_SV) ? NSV : 0); ++s)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
-          const float4 t = *reinterpret_cast<const float4 *>(&par[P_SV + s * BN + key]);
-          svv[s][4 * i4] = t.x; svv[s][4 * i4 + 1] = t.y; svv[s][4 * i4 + 2] = t.z; svv[s][4 * i4 + 3] = t.w;
-        }
-      u32x4_t vta[NDB], wza[NSV];
-      auto load_v_operands = [&](int c) {
-#pragma unroll
-        for (int d = 0; d < NDB; ++d)
-          vta[d] = *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
-#pragma unroll
-        for (int s = 0; s < NSV; ++s) {
-          wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
-        }
-      };
-      if constexpr (HOIST) load_v_operands(0);
-      if constexpr (HOIST) __builtin_amdgcn_sched_barrier(0);
-
-      // ---- logits of this block in the log2 domain, relative to the reference --------
-      float z[16];
+      z[i] = v;
+    }
+    // mask: block-causal key limit, and the ragged last tile
+    if (t0 + BN > wave_minlim) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float v = -m_ref;
-#pragma unroll
-        for (int s = 0; s < NSK; ++s) {
-          const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          v = __builtin_fmaf(HOIST ? ckv[s][i] : par[P_CK + s * BN + key], sacc[s][i], v);
-        }
-        z[i] = v;
+        const int key = t0 + kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+        if (key >= limit) z[i] = -INFINITY;
       }
-      // mask: block-causal key limit, and the ragged last tile
-      if (t0 + BN > wave_minlim) {
+    }
+    float zmax = z[0];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = t0 + kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          if (key >= limit) z[i] = -INFINITY;
-        }
+    for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
+    zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+    if (first || __any(zmax > kRescaleAt)) {
+      // Move the reference to the row's current maximum: up only (never down) once
+      // something has been accumulated; the very first block takes its maximum as it
+      // is, negative or not (the accumulators are still zero, so alpha = 1 is exact).
+      const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      m_ref += delta;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] -= delta;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) racc[j] *= alpha;
+#pragma unroll
+      for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
+    }
+    first = false;
+    float pv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
+#pragma unroll
+    for (int s = 0; s < NSV; ++s)
+#pragma unroll
+      for (int i2 = 0; i2 < 8; ++i2) {
+        const int i = 2 * i2;
+        const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+        if constexpr (FOLD_SV) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
+        else if constexpr (HOIST)
+          pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[kb][s][i], pv[i + 1] * svv[kb][s][i + 1]);
+        else
+          pop[kb][s][i >> 3][(i & 7) >> 1] =
+              pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
       }
-
-      // ---- online softmax against a lazily moved reference --------------------------
-      float zmax = z[0];
-#pragma unroll
-      for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
-      zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-      const bool first = (tile == 0 && kb == 0);
-      if (first || __any(zmax > kRescaleAt)) {
-        // Move the reference to the row's current maximum: up only (never down) once
-        // something has been accumulated; the very first block takes its maximum as it
-        // is, negative or not (the accumulators are still zero, so alpha = 1 is exact).
-        const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
-        const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
-        m_ref += delta;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) z[i] -= delta;
-#pragma unroll
-        for (int d = 0; d < NDB; ++d)
-#pragma unroll
-          for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) racc[j] *= alpha;
-#pragma unroll
-        for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
-      }
-
-      // P'^T operands: for each V scale group, p * vs as bf16; 16 registers -> 2 chunks of 4 dwords
-      float pv[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
-      u32 pop[NSV][2][4];
+    if (tile_rem) {
+      // the remainder term must see the same bf16-rounded weights as the MFMA
 #pragma unroll
       for (int s = 0; s < NSV; ++s)
 #pragma unroll
         for (int i2 = 0; i2 < 8; ++i2) {
           const int i = 2 * i2;
           const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          if constexpr (FOLD_SV) pop[s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
-          else if constexpr (HOIST) pop[s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[s][i], pv[i + 1] * svv[s][i + 1]);
-          else pop[s][i >> 3][(i & 7) >> 1] =
-              pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
+          const u32 pk = pop[kb][s][i >> 3][(i & 7) >> 1];
+          r_run[s] = __builtin_fmaf(u2f(pk << 16), par[P_VR + s * BN + key], r_run[s]);
+          r_run[s] = __builtin_fmaf(u2f(pk & 0xffff0000u), par[P_VR + s * BN + key + 1], r_run[s]);
         }
-      if (tile_rem) {
-        // the remainder term must see the same bf16-rounded weights as the MFMA
-#pragma unroll
-        for (int s = 0; s < NSV; ++s)
-#pragma unroll
-          for (int i2 = 0; i2 < 8; ++i2) {
-            const int i = 2 * i2;
-            const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-            const u32 pk = pop[s][i >> 3][(i & 7) >> 1];
-            r_run[s] = __builtin_fmaf(u2f(pk << 16), par[P_VR + s * BN + key], r_run[s]);
-            r_run[s] = __builtin_fmaf(u2f(pk & 0xffff0000u), par[P_VR + s * BN + key + 1], r_run[s]);
-          }
-      }
+    }
+  };
 
-      // ---- O^T += V^T P'^T for the 32 keys of this block; one more MFMA per chunk and
-      //      V group feeds the extra block: its row s collects the zero-point sum of group
-      //      s and rows 4..6 (group 0 only) the softmax denominator ------------------------
-      __builtin_amdgcn_s_setprio(1);
+  // O^T += V^T P'^T for the 32 keys of one block; one more MFMA per chunk and V group
+  // feeds the extra block: its row s collects the zero-point sum of group s and rows
+  // 4..6 (group 0 only) the softmax denominator
+  auto pv_mfma = [&](int kb, bool preloaded) {
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        u32x4_t av[NDB], aw[NSV];
-        if constexpr (!HOIST) load_v_operands(c);
+    for (int c = 0; c < 2; ++c) {
+      u32x4_t av[NDB], aw[NSV];
+      if (!(preloaded && c == 0) && !(HOIST && c == 1)) load_v_operands(kb, c);
 #pragma unroll
-        for (int d = 0; d < NDB; ++d) av[d] = vta[d];
+      for (int d = 0; d < NDB; ++d) av[d] = vta[d];
 #pragma unroll
-        for (int s = 0; s < NSV; ++s) aw[s] = wza[s];
-        if (HOIST && c == 0) {
-          load_v_operands(1);   // in flight under this chunk's MFMAs
-          if constexpr (HOIST) __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int d = 0; d < NDB; ++d) {
-          constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
-          const int s = d / DBS;
-          u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
-          oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[d]),
-                                                            __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
-        }
-#pragma unroll
-        for (int s = 0; s < NSV; ++s) {
-          u32x4_t bv = {pop[s][c][0], pop[s][c][1], pop[s][c][2], pop[s][c][3]};
-          racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
-                                                         __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
-        }
+      for (int s = 0; s < NSV; ++s) aw[s] = wza[s];
+      if (HOIST && c == 0) {
+        load_v_operands(kb, 1);   // in flight under this chunk's MFMAs
+        __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int d = 0; d < NDB; ++d) {
+        constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
+        const int s = d / DBS;
+        u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
+        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[d]),
+                                                          __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
+      }
+#pragma unroll
+      for (int s = 0; s < NSV; ++s) {
+        u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
+        racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
+                                                       __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+  };
 
-      __builtin_amdgcn_s_setprio(0);
-      // between the two key blocks, with the first block's PV MFMAs in flight: widen
-      // the next tile's V into the other V^T slot
-      if (kb == 0 && tile + 1 < n_tiles) widen_v(tile + 1);
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    begin_tile(tile);
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      load_scales(kb);
+      qk(kb);
+      if constexpr (HOIST) {
+        load_v_operands(kb, 0);   // used after the softmax arithmetic
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      softmax(kb);
+      pv_mfma(kb, HOIST);
+      if (kb == 0) widen_next(tile);
     }
     __syncthreads();   // the one barrier per tile
   }
