@@ -100,3 +100,58 @@ def test_var_d16_per_head_int8_fp32(dev):
 def test_empty(dev):
     q, s, z = ops.quant_pack(torch.empty(2, 0, 3, 8, device=dev), (0, 1), 8)
     assert q.shape == (2, 0, 3, 2)
+
+
+@pytest.mark.parametrize('mask', range(1, 16))
+def test_every_reduce_set_on_tiled_shapes(dev, mask):
+    """All 15 non-empty reduce sets over the four dims, on shapes that exercise the
+    tiled path's cases: inner dim shorter and longer than a workgroup's row lanes,
+    several chunks of partials per group, 3 and 64 column lanes."""
+    dims = tuple(d for d in range(4) if (mask >> d) & 1)
+    g = torch.Generator().manual_seed(100 + mask)
+    for shape, dtype in [((3, 5, 70, 32), torch.bfloat16), ((2, 40, 7, 128), torch.float32),
+                         ((5, 3, 33, 512), torch.bfloat16), ((2, 3, 100, 24), torch.float16),
+                         ((64, 2, 300, 64), torch.bfloat16)]:
+        x = (torch.randn(*shape, generator=g) * 3 + 0.25).to(dtype)
+        x[..., 1] *= 9
+        for bits, asym in ((8, False), (4, True)):
+            note('general tiled', mask, shape, dtype, bits, asym)
+            _check(x, dims, bits, asym, True, dev)
+
+
+def test_all_ones_scale_significand_in_general_path(dev):
+    """A group whose scale is (2 - 2^-23) * 2^e must take the exact division (see
+    test_gpu_quant_rows.py::test_scale_with_all_ones_significand)."""
+    import numpy as np
+    s_star = np.float32((2 - 2.0 ** -23) * 0.25)
+    top = None
+    a = np.float32(np.float64(s_star) * 127.0)
+    for cand in [a] + [np.nextafter(a, np.float32(np.inf))] * 0:
+        if np.float32(cand) / np.float32(127.0) == s_star:
+            top = float(cand)
+    c = a
+    for _ in range(16):
+        if top is not None:
+            break
+        c = np.nextafter(c, np.float32(np.inf))
+        if np.float32(c) / np.float32(127.0) == s_star:
+            top = float(c)
+    c = a
+    for _ in range(16):
+        if top is not None:
+            break
+        c = np.nextafter(c, np.float32(-np.inf))
+        if np.float32(c) / np.float32(127.0) == s_star:
+            top = float(c)
+    assert top is not None
+    half = np.float32(np.float64(s_star) * 0.5)
+    x = torch.zeros(2, 3, 40, 64)
+    x[0, 1, 5, :] = top                                            # per-channel groups of head 1: scale = s_star
+    x[1, 1, 7, :] = float(np.nextafter(half, np.float32(np.inf)))  # rounds to 1 under IEEE division, 0 under the shortcut
+    x[1, 1, 8, :] = float(half)
+    x[0, 0, :, :] = torch.randn(40, 64, generator=torch.Generator().manual_seed(5))
+    q, s, _ = O.quant_reduce(x, (0, 2), 8, False)
+    assert bool(((s[0, 1, 0].view(torch.int32) & 0x7fffff) == 0x7fffff).all())
+    assert int(q[1, 1, 7, 0]) == 1
+    note('general all-ones scale')
+    _check(x, (0, 2), 8, False, True, dev)

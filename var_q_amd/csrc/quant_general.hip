@@ -1,13 +1,15 @@
 // General two-phase quantizer: groups that span rows (the six grouping methods
 // of VAR_Q/quant.py:75-95, which all reduce over the batch dim, plus any other
 // reduce set).  A single HBM read cannot serve such groups, so:
-//   phase A  group min/max (or max-abs) -> workspace, via ordered-integer atomics
-//   finalize workspace -> scale / zero-point           (VAR_Q/quant.py:112-116)
+//   phase A  group min/max (or max-abs): one partial per (chunk, group) in the
+//            workspace, no atomics (tiled path below)
+//   finalize fold the partials -> scale / zero-point      (VAR_Q/quant.py:112-116)
 //   phase B  re-read input (L2 / Infinity-Cache resident for KV-sized tensors),
 //            divide, round half-to-even, clamp, pack    (VAR_Q/quant.py:118-121,
 //            VAR_Q/pack_unpack.py:177-196)
 // min/max are exactly associative, so the result does not depend on the order
-// in which partial results meet.
+// in which partial results meet.  Channel counts that are not a multiple of 8 and
+// rows wider than 512 channels take scalar kernels with ordered-integer atomics.
 #include "varq_common.h"
 
 namespace {
@@ -56,131 +58,246 @@ __device__ __forceinline__ void row_to_idx(const GenParams &p, int64_t r, int64_
   i0 = t / p.n1;
 }
 
-// ---- phase A, c % 8 == 0 ---------------------------------------------------
-// Lane layout: c8p lanes per row (lanes >= c8 idle), 256/c8p rows per pass.
-// Each thread walks rows r0 + k*rowlanes and keeps a running min/max for its
-// current group, flushing with atomics when the group changes.  When the whole
-// block stayed in one group the flush first goes through LDS so that only one
-// thread per column issues atomics.
+// ---- fast path (c % 8 == 0, at most 512 channels): tiled, atomic-free -------------
+// The leading dims are brought to a canonical form on the host (Plan): a linear
+// index `ko` over kept outer dims, a linear index `ro` over reduced outer dims,
+// and along contiguous rows either a kept extent Q (d2 kept) or a reduced extent
+// RI (d2 reduced):
+//     row   = ko*ko_rs + ro*ro_rs + (q | ri)
+//     group = ko*ko_gs + q*q_gs  (+ channel when the channel dim is kept)
+// A workgroup is 256 threads = R row lanes x c8p column lanes (8 channels each) and
+// owns one (ko, tile of Q, chunk z of the reduced steps).  Every thread sees a
+// single group (per channel) for its whole life: no group lookups and no integer
+// divisions in the loop.  Phase A leaves one partial min/max per (z, group) in the
+// workspace (plain stores, each written exactly once), the finalize kernel folds
+// the Z partials, phase B walks the same decomposition with the group's scale,
+// reciprocal and zero-point in registers.
+struct Plan {
+  int64_t ko_rs, ro_rs, ko_gs, q_gs;
+  int nko, nro, Q, RI;
+  int lanesQ, sub, tilesQ;     // row lanes spent on q; positions folded into the rest; tiles over Q
+  int fold_ro;                 // 1: the spare row lanes fold consecutive ro (RI == 1), 0: consecutive rows of RI
+  int T;                       // steps per ro along RI (inner reduced), 1 when d2 is kept
+  int steps, Z, steps_per_chunk;
+  int R, c8, c8p, shift;
+};
+
+// decode the workgroup and lane; returns false for an idle lane
+struct Lane {
+  int ko, q, f, col, z;
+  bool live;
+};
+__device__ __forceinline__ Lane decode(const Plan &pl) {
+  Lane l;
+  const int bid = blockIdx.x;
+  l.z = bid % pl.Z;
+  const int kb = bid / pl.Z;
+  const int tq = kb % pl.tilesQ;
+  l.ko = kb / pl.tilesQ;
+  l.col = threadIdx.x & (pl.c8p - 1);
+  const int rowlane = threadIdx.x >> pl.shift;
+  const int lq = rowlane % pl.lanesQ;
+  l.f = rowlane / pl.lanesQ;
+  l.q = tq * pl.lanesQ + lq;
+  l.live = l.col < pl.c8 && l.f < pl.sub && l.q < pl.Q;
+  return l;
+}
+
+// Calls body(row) for every row of this thread, in step order.
+template <typename F>
+__device__ __forceinline__ void for_rows(const Plan &pl, const Lane &l, F body) {
+  const int s0 = l.z * pl.steps_per_chunk, s1 = min(s0 + pl.steps_per_chunk, pl.steps);
+  const int64_t base = (int64_t)l.ko * pl.ko_rs + l.q;
+  if (pl.fold_ro) {
+    // d2 kept: a step is `sub` consecutive reduced positions
+    for (int s = s0; s < s1; ++s) {
+      const int ro = s * pl.sub + l.f;
+      if (ro < pl.nro) body(base + (int64_t)ro * pl.ro_rs);
+    }
+  } else {
+    // d2 reduced: a step is `sub` (= R) consecutive rows of one ro
+    int ro = s0 / pl.T, t = s0 - ro * pl.T;
+    for (int s = s0; s < s1; ++s) {
+      const int ri = t * pl.sub + l.f;
+      if (ri < pl.RI) body(base + (int64_t)ro * pl.ro_rs + ri);
+      if (++t == pl.T) { t = 0; ++ro; }
+    }
+  }
+}
+
 template <int DT, bool ASYM, bool KEEPC>
-__global__ __launch_bounds__(256) void minmax_kernel(GenParams p) {
+__global__ __launch_bounds__(256) void minmax_tiled_kernel(GenParams p, Plan pl, float *part_max, float *part_min) {
   constexpr int NV = KEEPC ? 8 : 1;
   __shared__ float lds_mx[256 * NV];
   __shared__ float lds_mn[ASYM ? 256 * NV : 1];
-
-  const int lane_col = threadIdx.x & (p.c8p - 1);
-  const int rowlane = threadIdx.x >> p.c8p_shift;
-  const int rowlanes = 256 >> p.c8p_shift;
-  const bool col_live = lane_col < p.c8;
-  const int64_t r_begin = (int64_t)blockIdx.x * p.rows_per_block;
-  const int64_t r_end = min(r_begin + p.rows_per_block, p.rows);
-
+  const Lane l = decode(pl);
   float mx[NV], mn[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) { mx[j] = ASYM ? -INFINITY : 0.f; mn[j] = INFINITY; }
-  int64_t cur = -1;
-  bool flushed_midway = false;
-
-  auto flush = [&](int64_t g) {
-    if (KEEPC) {
-      if (!col_live) return;
+  if (l.live) {
+    for_rows(pl, l, [&](int64_t row) {
+      float v[8];
+      In8<DT>::load(p.x, row * p.c + l.col * 8, v);
+      if (KEEPC) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        atomicMax(&p.ws_max[g + lane_col * 8 + j], ASYM ? enc_ord(mx[j]) : f2u(mx[j]));
-        if (ASYM) atomicMin(&p.ws_min[g + lane_col * 8 + j], enc_ord(mn[j]));
-      }
-    } else if (lane_col == 0) {
-      atomicMax(&p.ws_max[g], ASYM ? enc_ord(mx[0]) : f2u(mx[0]));
-      if (ASYM) atomicMin(&p.ws_min[g], enc_ord(mn[0]));
-    }
-  };
-
-  for (int64_t r = r_begin + rowlane; r < r_end; r += rowlanes) {
-    int64_t i0, i1, i2;
-    row_to_idx(p, r, i0, i1, i2);
-    const int64_t g = i0 * p.gs0 + i1 * p.gs1 + i2 * p.gs2;
-    if (g != cur) {
-      if (cur >= 0) { flush(cur); flushed_midway = true; }
-      cur = g;
-#pragma unroll
-      for (int j = 0; j < NV; ++j) { mx[j] = ASYM ? -INFINITY : 0.f; mn[j] = INFINITY; }
-    }
-    float v[8];
-    if (col_live) In8<DT>::load(p.x, r * p.c + lane_col * 8, v);
-    else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = ASYM ? NAN : 0.f;  // fmin/fmax ignore NaN
-    }
-    if (KEEPC) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (ASYM) { mx[j] = fmaxf(mx[j], v[j]); mn[j] = fminf(mn[j], v[j]); }
-        else mx[j] = fmaxf(mx[j], fabsf(v[j]));
-      }
-    } else {
-      float a, b = INFINITY;
-      if (ASYM) {
-        a = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
-        b = fminf(fminf(fminf(v[0], v[1]), fminf(v[2], v[3])), fminf(fminf(v[4], v[5]), fminf(v[6], v[7])));
-      } else {
-        a = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
-                  fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
-      }
-      // reduce over the lanes of this row (c8p <= 64: a row never spans wavefronts)
-      for (int off = 1; off < p.c8p; off <<= 1) {
-        a = fmaxf(a, __shfl_xor(a, off, 64));
-        if (ASYM) b = fminf(b, __shfl_xor(b, off, 64));
-      }
-      mx[0] = fmaxf(mx[0], a);
-      if (ASYM) mn[0] = fminf(mn[0], b);
-    }
-  }
-
-  // Was the whole block one group?  (cur is -1 for threads that saw no row.)
-  __shared__ long long first_g;
-  if (threadIdx.x == 0) first_g = cur;
-  __syncthreads();
-  const bool uniform = __syncthreads_and(!flushed_midway && (cur == first_g || cur < 0)) && first_g >= 0;
-
-  if (!uniform) {
-    if (cur >= 0) flush(cur);
-    return;
-  }
-
-  // block-uniform: tree through LDS, then one set of atomics
-#pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    lds_mx[j * 256 + threadIdx.x] = (cur >= 0) ? mx[j] : (ASYM ? -INFINITY : 0.f);
-    if (ASYM) lds_mn[j * 256 + threadIdx.x] = (cur >= 0) ? mn[j] : INFINITY;
-  }
-  __syncthreads();
-  if (KEEPC) {
-    // combine the rowlanes that share a column octet
-    if (rowlane == 0 && col_live) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float a = lds_mx[j * 256 + lane_col], b = ASYM ? lds_mn[j * 256 + lane_col] : 0.f;
-        for (int rl = 1; rl < rowlanes; ++rl) {
-          a = fmaxf(a, lds_mx[j * 256 + rl * p.c8p + lane_col]);
-          if (ASYM) b = fminf(b, lds_mn[j * 256 + rl * p.c8p + lane_col]);
+        for (int j = 0; j < 8; ++j) {
+          if (ASYM) { mx[j] = fmaxf(mx[j], v[j]); mn[j] = fminf(mn[j], v[j]); }
+          else mx[j] = fmaxf(mx[j], fabsf(v[j]));
         }
-        atomicMax(&p.ws_max[first_g + lane_col * 8 + j], ASYM ? enc_ord(a) : f2u(a));
-        if (ASYM) atomicMin(&p.ws_min[first_g + lane_col * 8 + j], enc_ord(b));
+      } else if (ASYM) {
+        mx[0] = fmaxf(mx[0], fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7]))));
+        mn[0] = fminf(mn[0], fminf(fminf(fminf(v[0], v[1]), fminf(v[2], v[3])), fminf(fminf(v[4], v[5]), fminf(v[6], v[7]))));
+      } else {
+        mx[0] = fmaxf(mx[0], fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                                   fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7])))));
       }
+    });
+  }
+  if (!KEEPC) {
+    // fold the column lanes of a row (c8p <= 64: a row never spans wavefronts; idle lanes hold the identity)
+    for (int off = 1; off < pl.c8p; off <<= 1) {
+      mx[0] = fmaxf(mx[0], __shfl_xor(mx[0], off, 64));
+      if (ASYM) mn[0] = fminf(mn[0], __shfl_xor(mn[0], off, 64));
+    }
+  }
+  // fold the `sub` row lanes that share q (lane index = (f*lanesQ + lq)*c8p + col)
+  if (pl.sub > 1) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      lds_mx[j * 256 + threadIdx.x] = mx[j];
+      if (ASYM) lds_mn[j * 256 + threadIdx.x] = mn[j];
+    }
+    __syncthreads();
+    if (l.f == 0) {
+      const int stride = pl.lanesQ * pl.c8p;
+      for (int f = 1; f < pl.sub; ++f)
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+          mx[j] = fmaxf(mx[j], lds_mx[j * 256 + threadIdx.x + f * stride]);
+          if (ASYM) mn[j] = fminf(mn[j], lds_mn[j * 256 + threadIdx.x + f * stride]);
+        }
+    }
+  }
+  if (l.f != 0 || l.q >= pl.Q || l.col >= pl.c8 || (!KEEPC && l.col != 0)) return;
+  const int64_t g = (int64_t)l.ko * pl.ko_gs + (int64_t)l.q * pl.q_gs + (KEEPC ? l.col * 8 : 0);
+  float *dmx = part_max + (int64_t)l.z * p.n_groups + g;
+  float *dmn = part_min + (int64_t)l.z * p.n_groups + g;
+  if (KEEPC) {
+    reinterpret_cast<float4 *>(dmx)[0] = make_float4(mx[0], mx[1], mx[2], mx[3]);
+    reinterpret_cast<float4 *>(dmx)[1] = make_float4(mx[4 % NV], mx[5 % NV], mx[6 % NV], mx[7 % NV]);
+    if (ASYM) {
+      reinterpret_cast<float4 *>(dmn)[0] = make_float4(mn[0], mn[1], mn[2], mn[3]);
+      reinterpret_cast<float4 *>(dmn)[1] = make_float4(mn[4 % NV], mn[5 % NV], mn[6 % NV], mn[7 % NV]);
     }
   } else {
-    for (int s = 128; s > 0; s >>= 1) {
-      if (threadIdx.x < s) {
-        lds_mx[threadIdx.x] = fmaxf(lds_mx[threadIdx.x], lds_mx[threadIdx.x + s]);
-        if (ASYM) lds_mn[threadIdx.x] = fminf(lds_mn[threadIdx.x], lds_mn[threadIdx.x + s]);
-      }
-      __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-      atomicMax(&p.ws_max[first_g], ASYM ? enc_ord(lds_mx[0]) : f2u(lds_mx[0]));
-      if (ASYM) atomicMin(&p.ws_min[first_g], enc_ord(lds_mn[0]));
+    dmx[0] = mx[0];
+    if (ASYM) dmn[0] = mn[0];
+  }
+}
+
+// partials -> scale, zero-point, reciprocal and the flag of the exact-quotient shortcut.
+// 256 threads = ZL z-lanes x 256/ZL adjacent groups; the z-lanes of a group meet in LDS.
+template <bool ASYM>
+__global__ __launch_bounds__(256) void finalize_tiled_kernel(GenParams p, int Z, int ZL, const float *part_max,
+                                                             const float *part_min, float *rinv, u32 *plain) {
+  __shared__ float lds_mx[256];
+  __shared__ float lds_mn[256];
+  const int gpb = 256 / ZL;                       // groups per block
+  const int gl = threadIdx.x % gpb, zl = threadIdx.x / gpb;
+  const int64_t g = (int64_t)blockIdx.x * gpb + gl;
+  float mx = ASYM ? -INFINITY : 0.f, mn = INFINITY;
+  if (g < p.n_groups) {
+    for (int z = zl; z < Z; z += ZL) {
+      mx = fmaxf(mx, part_max[(int64_t)z * p.n_groups + g]);
+      if (ASYM) mn = fminf(mn, part_min[(int64_t)z * p.n_groups + g]);
     }
   }
+  lds_mx[threadIdx.x] = mx;
+  lds_mn[threadIdx.x] = mn;
+  __syncthreads();
+  for (int h = ZL >> 1; h > 0; h >>= 1) {
+    if (zl < h) {
+      lds_mx[threadIdx.x] = fmaxf(lds_mx[threadIdx.x], lds_mx[threadIdx.x + h * gpb]);
+      lds_mn[threadIdx.x] = fminf(lds_mn[threadIdx.x], lds_mn[threadIdx.x + h * gpb]);
+    }
+    __syncthreads();
+  }
+  if (zl != 0 || g >= p.n_groups) return;
+  mx = lds_mx[threadIdx.x];
+  mn = lds_mn[threadIdx.x];
+  float s;
+  if (ASYM) {
+    s = fmaxf((mx - mn) / (float)((1 << p.bits) - 1), p.eps);
+    p.zp[g] = (float)p.qmin - rintf(mn / s);
+  } else {
+    s = fmaxf(mx / (float)p.qmax, p.eps);
+  }
+  p.scale[g] = s;
+  rinv[g] = 1.0f / s;
+  // x/s == RN(q0 + (x - q0*s)*r) with q0 = RN(x*r), r = RN(1/s), for every finite x unless the
+  // significand of s is all ones or the residual can underflow
+  plain[g] = (s > 0x1p-96f && s < 0x1p96f && (f2u(s) & 0x7fffffu) != 0x7fffffu) ? 1u : 0u;
+}
+
+template <int DT, bool KEEPC>
+__global__ __launch_bounds__(256) void quant_tiled_kernel(GenParams p, Plan pl, const float *rinv, const u32 *plain) {
+  constexpr int NV = KEEPC ? 8 : 1;
+  const Lane l = decode(pl);
+  // 2-bit words are assembled from two adjacent column lanes: idle lanes must still reach the shuffle
+  const bool live = l.live;
+  const int64_t g = (int64_t)l.ko * pl.ko_gs + (int64_t)(live ? l.q : 0) * pl.q_gs + (KEEPC ? (live ? l.col : 0) * 8 : 0);
+  float s[NV], r[NV], z[NV];
+  bool all_plain = true;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    s[j] = p.scale[g + j];
+    r[j] = rinv[g + j];
+    z[j] = p.asym ? p.zp[g + j] : 0.f;
+    all_plain = all_plain && plain[g + j] != 0u;
+  }
+  const float qmin = (float)p.qmin, qmax = (float)p.qmax;
+  const u32 mask = (1u << p.bits) - 1u;
+  if (!live) return;   // (only the 2-bit path shuffles, and there c8 is even: partners are live together)
+  for_rows(pl, l, [&](int64_t row) {
+    float v[8];
+    In8<DT>::load(p.x, row * p.c + l.col * 8, v);
+    int q[8];
+    if (all_plain) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sj = s[j % NV], rj = r[j % NV];
+        const float q0 = v[j] * rj;
+        const float t = __builtin_fmaf(__builtin_fmaf(-q0, sj, v[j]), rj, q0);
+        q[j] = (int)__builtin_amdgcn_fmed3f(rintf(t) + z[j % NV], qmin, qmax);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = (int)__builtin_amdgcn_fmed3f(rintf(v[j] / s[j % NV]) + z[j % NV], qmin, qmax);
+    }
+    const int64_t o = row * p.c8 + l.col;
+    if (p.codes) {
+      u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
+      u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
+      *reinterpret_cast<uint2 *>(p.codes + o * 8) = make_uint2(lo, hi);
+    }
+    if (p.words) {
+      if (p.bits == 8) {
+        u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
+        u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
+        *reinterpret_cast<uint2 *>(p.words + row * p.wpr + l.col * 2) = make_uint2(lo, hi);
+      } else {
+        u32 w = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w |= ((u32)q[j] & mask) << (j * p.bits);
+        if (p.bits == 4) {
+          p.words[row * p.wpr + l.col] = (int32_t)w;
+        } else {  // 2 bits: 16 codes per word = two adjacent octets (c % 16 == 0 on this path)
+          u32 other = __shfl_xor(w, 1, 64);
+          if ((l.col & 1) == 0) p.words[row * p.wpr + (l.col >> 1)] = (int32_t)(w | (other << 16));
+        }
+      }
+    }
+  });
 }
 
 // ---- phase A, any c: one thread per element --------------------------------
@@ -223,65 +340,6 @@ __device__ __forceinline__ int quant_one(float v, float s, float zp, bool asym, 
   return (int)__builtin_amdgcn_fmed3f(n, qmin, qmax);
 }
 
-// ---- phase B, c % 8 == 0: one thread per octet -----------------------------
-template <int DT, bool KEEPC>
-__global__ __launch_bounds__(256) void quant_general_kernel(GenParams p) {
-  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (o >= p.rows * p.c8) return;
-  const int64_t r = o / p.c8;
-  const int col = (int)(o - r * p.c8);
-  int64_t i0, i1, i2;
-  row_to_idx(p, r, i0, i1, i2);
-  const int64_t g = i0 * p.gs0 + i1 * p.gs1 + i2 * p.gs2 + (KEEPC ? col * 8 : 0);
-
-  float v[8];
-  In8<DT>::load(p.x, o * 8, v);
-  const float qmin = (float)p.qmin, qmax = (float)p.qmax;
-  int q[8];
-  if (KEEPC) {
-    const float4 *sp = reinterpret_cast<const float4 *>(p.scale + g);  // g % 8 == 0 when c % 8 == 0
-    float4 sa = sp[0], sb = sp[1];
-    const float s[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
-    float z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (p.asym) {
-      const float4 *zp = reinterpret_cast<const float4 *>(p.zp + g);
-      float4 za = zp[0], zb = zp[1];
-      z[0] = za.x; z[1] = za.y; z[2] = za.z; z[3] = za.w; z[4] = zb.x; z[5] = zb.y; z[6] = zb.z; z[7] = zb.w;
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] = quant_one(v[j], s[j], z[j], p.asym, qmin, qmax);
-  } else {
-    const float s = p.scale[g];
-    const float z = p.asym ? p.zp[g] : 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] = quant_one(v[j], s, z, p.asym, qmin, qmax);
-  }
-
-  if (p.codes) {
-    u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
-    u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
-    *reinterpret_cast<uint2 *>(p.codes + o * 8) = make_uint2(lo, hi);
-  }
-  if (p.words) {
-    const u32 mask = (1u << p.bits) - 1u;
-    if (p.bits == 8) {
-      u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
-      u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
-      *reinterpret_cast<uint2 *>(p.words + r * p.wpr + col * 2) = make_uint2(lo, hi);
-    } else {
-      u32 w = 0;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) w |= ((u32)q[j] & mask) << (j * p.bits);
-      if (p.bits == 4) {
-        p.words[r * p.wpr + col] = (int32_t)w;
-      } else {  // 2 bits: 16 codes per word = two adjacent octets (c % 16 == 0 on this path)
-        u32 other = __shfl_xor(w, 1, 64);
-        if ((col & 1) == 0) p.words[r * p.wpr + (col >> 1)] = (int32_t)(w | (other << 16));
-      }
-    }
-  }
-}
-
 // ---- phase B, any c: one thread per output word (or per code group) ---------
 template <int DT>
 __global__ void quant_scalar_kernel(GenParams p) {
@@ -308,28 +366,109 @@ __global__ void quant_scalar_kernel(GenParams p) {
   if (p.words) p.words[r * wpr + wi] = (int32_t)w;
 }
 
+// Host side of the tiled path: canonical form of the leading dims and the launch shape.
+// Returns false when the shape needs the scalar kernels.
+bool make_plan(const int64_t *sh, int reduce_mask, int64_t n_groups, Plan &pl) {
+  const int64_t n0 = sh[0], n1 = sh[1], n2 = sh[2], c = sh[3];
+  const int64_t rows = n0 * n1 * n2;
+  if (c % 8 != 0 || rows <= 0 || rows >= (1ll << 31) - 512) return false;
+  pl.c8 = (int)(c / 8);
+  int c8p = 1, shl = 0;
+  while (c8p < pl.c8) { c8p <<= 1; ++shl; }
+  if (c8p > 64) return false;
+  pl.c8p = c8p; pl.shift = shl; pl.R = 256 / c8p;
+  const bool k0 = !(reduce_mask & 1), k1 = !(reduce_mask & 2), k2 = !(reduce_mask & 4), kc = !(reduce_mask & 8);
+  int64_t stride = kc ? c : 1;
+  const int64_t gs2 = k2 ? stride : 0; if (k2) stride *= n2;
+  const int64_t gs1 = k1 ? stride : 0; if (k1) stride *= n1;
+  const int64_t gs0 = k0 ? stride : 0;
+  int64_t nko = 1, nro = 1, Q = 1, RI = 1;
+  pl.ko_rs = pl.ro_rs = pl.ko_gs = pl.q_gs = 0;
+  if (k2) {
+    Q = n2; pl.q_gs = gs2;
+    if (k1) {
+      Q = n1 * n2;                                   // gs1 == gs2 * n2: q runs over (i1, i2)
+      if (k0) Q = rows;                              // every row its own group
+      else { nro = n0; pl.ro_rs = n1 * n2; }
+    } else if (k0) { nko = n0; pl.ko_rs = n1 * n2; pl.ko_gs = gs0; nro = n1; pl.ro_rs = n2; }
+    else { nro = n0 * n1; pl.ro_rs = n2; }
+  } else {
+    RI = n2;
+    if (!k1) {
+      RI = n1 * n2;
+      if (!k0) RI = rows;
+      else { nko = n0; pl.ko_rs = n1 * n2; pl.ko_gs = gs0; }
+    } else if (k0) { nko = n0 * n1; pl.ko_rs = n2; pl.ko_gs = gs1; }     // gs0 == gs1 * n1
+    else { nko = n1; pl.ko_rs = n2; pl.ko_gs = gs1; nro = n0; pl.ro_rs = n1 * n2; }
+  }
+  pl.nko = (int)nko; pl.nro = (int)nro; pl.Q = (int)Q; pl.RI = (int)RI;
+  pl.lanesQ = (int)(Q < pl.R ? Q : pl.R);
+  pl.sub = pl.R / pl.lanesQ;
+  pl.tilesQ = (int)((Q + pl.lanesQ - 1) / pl.lanesQ);
+  pl.fold_ro = (RI == 1);
+  int64_t steps;
+  if (pl.fold_ro) { pl.T = 1; steps = (nro + pl.sub - 1) / pl.sub; }
+  else { pl.T = (int)((RI + pl.sub - 1) / pl.sub); steps = nro * pl.T; }
+  const int64_t kept_blocks = nko * pl.tilesQ;
+  int64_t Z = (4096 + kept_blocks - 1) / kept_blocks;
+  const int64_t zcap = (8ll << 20) / (n_groups > 0 ? n_groups : 1);   // partials stay below 64 MiB
+  if (Z > zcap) Z = zcap;
+  if (Z > steps) Z = steps;
+  if (Z < 1) Z = 1;
+  const int64_t spc = (steps + Z - 1) / Z;
+  Z = (steps + spc - 1) / spc;                     // no empty chunk: every (z, group) partial gets written
+  if (steps >= (1ll << 31) || kept_blocks * Z >= (1ll << 31)) return false;
+  pl.steps = (int)steps; pl.Z = (int)Z; pl.steps_per_chunk = (int)spc;
+  return true;
+}
+
+size_t plan_workspace_bytes(const Plan &pl, int64_t n_groups) {
+  return (size_t)n_groups * (2 + 2 * (size_t)pl.Z) * sizeof(float);
+}
+
+template <int DT>
+int run_tiled(GenParams &p, const Plan &pl, void *workspace, hipStream_t st) {
+  const int64_t ng = p.n_groups;
+  float *rinv = reinterpret_cast<float *>(workspace);
+  u32 *plain = reinterpret_cast<u32 *>(rinv + ng);
+  float *part_max = rinv + 2 * ng;
+  float *part_min = part_max + (int64_t)pl.Z * ng;
+  dim3 grid((unsigned)((int64_t)pl.nko * pl.tilesQ * pl.Z));
+  if (p.asym) {
+    if (p.keepc) hipLaunchKernelGGL((minmax_tiled_kernel<DT, true, true>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
+    else hipLaunchKernelGGL((minmax_tiled_kernel<DT, true, false>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
+  } else {
+    if (p.keepc) hipLaunchKernelGGL((minmax_tiled_kernel<DT, false, true>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
+    else hipLaunchKernelGGL((minmax_tiled_kernel<DT, false, false>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
+  }
+  // z-lanes per group in the finalize kernel: enough threads in total, no more lanes than partials
+  int ZL = 1;
+  while (ZL < 256 && ZL < pl.Z && ng * ZL < 65536) ZL <<= 1;
+  dim3 fgrid((unsigned)((ng + 256 / ZL - 1) / (256 / ZL)));
+  if (p.asym)
+    hipLaunchKernelGGL((finalize_tiled_kernel<true>), fgrid, dim3(256), 0, st, p, pl.Z, ZL, part_max, part_min, rinv, plain);
+  else
+    hipLaunchKernelGGL((finalize_tiled_kernel<false>), fgrid, dim3(256), 0, st, p, pl.Z, ZL, part_max, part_min, rinv, plain);
+  // phase B has no partials to keep apart: longer chunks amortize the per-thread parameter loads
+  Plan pb = pl;
+  constexpr int min_spc = 16;   // measured on [32,30,680,64] and [2,16,10521,128]: 12..24 steps per thread are best
+  if (pb.steps_per_chunk < min_spc) {
+    pb.steps_per_chunk = min_spc < pb.steps ? min_spc : pb.steps;
+    pb.Z = (pb.steps + pb.steps_per_chunk - 1) / pb.steps_per_chunk;
+  }
+  dim3 bgrid((unsigned)((int64_t)pb.nko * pb.tilesQ * pb.Z));
+  if (p.keepc) hipLaunchKernelGGL((quant_tiled_kernel<DT, true>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
+  else hipLaunchKernelGGL((quant_tiled_kernel<DT, false>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
+  return 0;
+}
+
+// any shape: one thread per element / per output word, group min/max by ordered-integer atomics
 template <int DT>
 int run_general(GenParams &p, hipStream_t st) {
   const int64_t ng = p.n_groups;
   hipLaunchKernelGGL(init_ws_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, st, p.ws_max,
                      p.asym ? p.ws_min : (u32 *)nullptr, ng);
-  const bool fast = (p.c % 8 == 0) && p.c8p <= 64;
-  if (fast) {
-    const int rowlanes = 256 / p.c8p;
-    // aim for a few thousand blocks, at least 8 passes each
-    int64_t rpb = (p.rows + 4095) / 4096;
-    rpb = ((rpb + rowlanes - 1) / rowlanes) * rowlanes;
-    if (rpb < 8 * rowlanes) rpb = 8 * rowlanes;
-    p.rows_per_block = (int)rpb;
-    dim3 grid((unsigned)((p.rows + rpb - 1) / rpb));
-    if (p.asym) {
-      if (p.keepc) hipLaunchKernelGGL((minmax_kernel<DT, true, true>), grid, dim3(256), 0, st, p);
-      else hipLaunchKernelGGL((minmax_kernel<DT, true, false>), grid, dim3(256), 0, st, p);
-    } else {
-      if (p.keepc) hipLaunchKernelGGL((minmax_kernel<DT, false, true>), grid, dim3(256), 0, st, p);
-      else hipLaunchKernelGGL((minmax_kernel<DT, false, false>), grid, dim3(256), 0, st, p);
-    }
-  } else {
+  {
     const int64_t n = p.rows * p.c;
     dim3 grid((unsigned)((n + 255) / 256));
     if (p.asym) hipLaunchKernelGGL((minmax_scalar_kernel<DT, true>), grid, dim3(256), 0, st, p);
@@ -340,13 +479,7 @@ int run_general(GenParams &p, hipStream_t st) {
     if (p.asym) hipLaunchKernelGGL((finalize_kernel<true>), grid, dim3(256), 0, st, p);
     else hipLaunchKernelGGL((finalize_kernel<false>), grid, dim3(256), 0, st, p);
   }
-  const bool fast_b = (p.c % 8 == 0) && (!p.words || (p.c * p.bits) % 32 == 0);
-  if (fast_b) {
-    const int64_t n = p.rows * p.c8;
-    dim3 grid((unsigned)((n + 255) / 256));
-    if (p.keepc) hipLaunchKernelGGL((quant_general_kernel<DT, true>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((quant_general_kernel<DT, false>), grid, dim3(256), 0, st, p);
-  } else {
+  {
     const int vals = p.words ? 32 / p.bits : 4;
     const int64_t n = p.rows * ((p.c + vals - 1) / vals);
     dim3 grid((unsigned)((n + 255) / 256));
@@ -366,7 +499,10 @@ int64_t count_groups(const int64_t *s, int reduce_mask) {
 
 extern "C" size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask) {
   if (!host_shape4) return 0;
-  return (size_t)count_groups(host_shape4, reduce_mask) * 2 * sizeof(u32);
+  const int64_t ng = count_groups(host_shape4, reduce_mask);
+  Plan pl;
+  if (make_plan(host_shape4, reduce_mask, ng, pl)) return plan_workspace_bytes(pl, ng);
+  return (size_t)ng * 2 * sizeof(u32);
 }
 
 extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
@@ -385,9 +521,12 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   VARQ_CHECK_ARG(scale && (!asym || zp), "quant_pack: scale/zp output missing");
   VARQ_CHECK_ARG(x && workspace, "quant_pack: null pointer");
   const int64_t ng = count_groups(s, reduce_mask);
-  if (workspace_bytes < (size_t)ng * 2 * sizeof(u32))
-    return varq_set_error(VARQ_ERR_WORKSPACE, "quant_pack: workspace %zu < %zu bytes", workspace_bytes,
-                          (size_t)ng * 2 * sizeof(u32));
+  Plan pl;
+  // the tiled kernels pack whole words per octet: c*bits must fill words (always true for 4 and 8 bits)
+  const bool tiled = make_plan(s, reduce_mask, ng, pl) && (!words || (s[3] * bits) % 32 == 0);
+  const size_t need = tiled ? plan_workspace_bytes(pl, ng) : (size_t)ng * 2 * sizeof(u32);
+  if (workspace_bytes < need)
+    return varq_set_error(VARQ_ERR_WORKSPACE, "quant_pack: workspace %zu < %zu bytes", workspace_bytes, need);
   VARQ_CHECK_ARG(rows * s[3] < (1ll << 40), "quant_pack: tensor too large");
 
   GenParams p;
@@ -415,7 +554,11 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   p.asym = asym ? 1 : 0;
   p.eps = eps;
   hipStream_t st = (hipStream_t)stream;
-  if (x_dtype == VARQ_F32) run_general<VARQ_F32>(p, st);
+  if (tiled) {
+    if (x_dtype == VARQ_F32) run_tiled<VARQ_F32>(p, pl, workspace, st);
+    else if (x_dtype == VARQ_BF16) run_tiled<VARQ_BF16>(p, pl, workspace, st);
+    else run_tiled<VARQ_F16>(p, pl, workspace, st);
+  } else if (x_dtype == VARQ_F32) run_general<VARQ_F32>(p, st);
   else if (x_dtype == VARQ_BF16) run_general<VARQ_BF16>(p, st);
   else run_general<VARQ_F16>(p, st);
   VARQ_CHECK_LAUNCH("quant_pack");
