@@ -19,8 +19,9 @@ struct DeqParams {
   RowMap in_map;           // (i0,i1,i2) -> input row
   int64_t n1, n2;
   int64_t ss0, ss1, ss2, ss3;
-  int64_t octets_per_pair, blocks_per_pair;
+  int64_t octets_per_pair;
   int c, c8, wpr, bits, group;
+  int c8_shift;            // log2(c8) when c8 is a power of two, else -1
 };
 
 template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t elem, const float (&f)[8], int n_valid) {
@@ -48,13 +49,13 @@ template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t ele
 
 template <int ODT>
 __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
-  const int64_t pair = blockIdx.x / p.blocks_per_pair;
-  const int64_t tile = blockIdx.x - pair * p.blocks_per_pair;
-  const int64_t o = tile * 256 + threadIdx.x;
+  // grid = (tiles of 256 octets, i1, i0): no division to find the block's place
+  const int64_t i0 = blockIdx.z, i1 = blockIdx.y;
+  const int o = blockIdx.x * 256 + threadIdx.x;          // octet inside the (i0, i1) pair, < 2^31
   if (o >= p.octets_per_pair) return;
-  const int64_t i0 = pair / p.n1, i1 = pair - i0 * p.n1;
-  const int64_t i2 = o / p.c8;
-  const int col = (int)(o - i2 * p.c8);
+  int i2, col;
+  if (p.c8_shift >= 0) { i2 = o >> p.c8_shift; col = o & (p.c8 - 1); }
+  else { i2 = o / p.c8; col = o - i2 * p.c8; }
   const int ch0 = col * 8;
   const int n_valid = min(8, p.c - ch0);
   const int64_t in_row = i0 * p.in_map.os0 + i1 * p.in_map.os1 + i2 * p.in_map.os2 + p.in_map.off;
@@ -100,6 +101,21 @@ __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[j] = (float)q[j] * s;
+    }
+  } else if (p.group == 1 && p.ss3 == 1 && n_valid == 8 && ((sbase + ch0) & 3) == 0) {
+    // one scale per channel, contiguous: two 16-byte loads
+    const float4 *sp = reinterpret_cast<const float4 *>(p.scale + sbase + ch0);
+    const float4 sa = sp[0], sb = sp[1];
+    const float sv[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
+    if (p.zp) {
+      const float4 *zq = reinterpret_cast<const float4 *>(p.zp + sbase + ch0);
+      const float4 za = zq[0], zb = zq[1];
+      const float zv[8] = {za.x, za.y, za.z, za.w, zb.x, zb.y, zb.z, zb.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = ((float)q[j] - zv[j]) * sv[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = (float)q[j] * sv[j];
     }
   } else {
 #pragma unroll
@@ -147,10 +163,13 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
     p.in_map.os0 = s[1] * s[2]; p.in_map.os1 = s[2]; p.in_map.os2 = 1; p.in_map.off = 0; p.in_map.slot_dim = -1;
   }
   p.octets_per_pair = s[2] * p.c8;
-  p.blocks_per_pair = (p.octets_per_pair + 255) / 256;
-  const int64_t blocks = p.blocks_per_pair * s[0] * s[1];
-  VARQ_CHECK_ARG(blocks < (1ll << 31), "dequant: too many blocks");
-  dim3 grid((unsigned)blocks);
+  p.c8_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == p.c8) p.c8_shift = sh;
+  const int64_t tiles = (p.octets_per_pair + 255) / 256;
+  // a pair with few rows wastes lanes of its last block only; pairs map to grid.y/z (limit 65535 each)
+  VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 256 && s[1] <= 65535 && s[0] <= 65535, "dequant: shape exceeds the grid limits");
+  dim3 grid((unsigned)tiles, (unsigned)s[1], (unsigned)s[0]);
   hipStream_t st = (hipStream_t)stream;
   if (out_dtype == VARQ_F32) hipLaunchKernelGGL(dequant_kernel<VARQ_F32>, grid, dim3(256), 0, st, p);
   else if (out_dtype == VARQ_BF16) hipLaunchKernelGGL(dequant_kernel<VARQ_BF16>, grid, dim3(256), 0, st, p);
