@@ -146,6 +146,28 @@ int varq_fused_attn(const void *q, void *out,
                     int Lq, int Lk, int Lk_stride, int D,
                     const int32_t *kv_limit, float softmax_scale, void *stream);
 
+/*
+ * Producer side of the quantized cache in one pass (an extension: the reference does
+ * this as separate tensor expressions before calling its quantizer,
+ * Infinity/infinity/models/basic.py:316-330 with apply_rotary_emb at :103-123, and
+ * VAR/models/basic_var.py:137-147).  Reads the qkv projection output
+ * [B, L, 3, H, c] once and
+ *   - writes q: optionally l2-normalised (x / max(|x|_2, norm_eps)) and multiplied by
+ *     q_scale_mul[h], optionally rotated (pairs (2i, 2i+1) by the angle whose cos/sin
+ *     are rope_cos/sin[token_start + l][i]), as bf16 [B, H, L, c];
+ *   - quantizes k (normalised, rotated) and v group-wise (as varq_quant_pack_rows) into
+ *     their cache rows: input row (b, l, h) goes to the row the map gives for
+ *     (n0, n1, n2) = (B, L, H).
+ * c in {32, 64, 128}; group a power of two in [8, c] (>= 16 for 2-bit codes).
+ */
+int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int L, int H, int c,
+                            const float *q_scale_mul, int l2norm, float norm_eps,
+                            const float *rope_cos, const float *rope_sin, int token_start,
+                            void *q_out, int group, int bits, int asym, float eps,
+                            const int64_t *host_rowmap, const int32_t *slot,
+                            int32_t *k_words, float *k_scale, float *k_zp,
+                            int32_t *v_words, float *v_scale, float *v_zp, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -336,3 +336,52 @@ def synth_kv(shape: Sequence[int], seed: int, dist: str = 'normal', outlier_frac
     ch = torch.randperm(d, generator=go)[:n_out]
     x[..., ch] *= outlier_mul
     return x.to(dtype)
+
+
+def prepare_qkv(qkv: torch.Tensor, scale_mul: Optional[torch.Tensor] = None, l2norm: bool = False,
+                norm_eps: float = 1e-12, rope=None, token_start: int = 0):
+    """EXTENSION (parity unpinned by reference: the reference leaves the summation order of
+    the norm to the backend).  The producer side of Infinity/infinity/models/basic.py:316-330
+    (F.normalize, .mul(scale_mul), apply_rotary_emb at :103-123) and
+    VAR/models/basic_var.py:137-141 restated for a qkv projection output [B,L,3,H,c]:
+    returns q [B,H,L,c] bf16, k [B,H,L,c] fp32, v [B,H,L,c] in the input dtype.
+
+    All arithmetic fp32, each operation rounded on its own.  Sum of squares: the 8
+    channels of an octet left to right, then octets pairwise ((o0+o1)+(o2+o3))+...;
+    y = x / max(sqrt(ss), norm_eps) with correctly rounded sqrt and true division; q times scale_mul[h]; rotation
+    of the pairs (2i, 2i+1): even = cos*y0 - sin*y1, odd = sin*y0 + cos*y1."""
+    B, L, three, H, c = qkv.shape
+    assert three == 3 and c % 8 == 0 and (c // 8) & (c // 8 - 1) == 0
+    q, k, v = (qkv[:, :, t].permute(0, 2, 1, 3).contiguous() for t in range(3))      # [B,H,L,c]
+    qf, kf = q.float(), k.float()
+
+    def normalize(x):
+        sq = x * x
+        o = sq.reshape(*sq.shape[:-1], c // 8, 8)
+        acc = o[..., 0]
+        for j in range(1, 8):
+            acc = acc + o[..., j]
+        while acc.shape[-1] > 1:
+            acc = acc[..., 0::2] + acc[..., 1::2]
+        # correctly rounded fp32 square root: through fp64 (53 >= 2*24+2 bits, so the second rounding
+        # cannot change the result); torch's vectorized fp32 sqrt on CPU is off by an ulp now and then
+        denom = torch.sqrt(acc.double()).float().clamp_min(norm_eps)                  # [..., 1]
+        return x / denom
+
+    if l2norm:
+        qf, kf = normalize(qf), normalize(kf)
+        if scale_mul is not None:
+            qf = qf * scale_mul.float().view(1, H, 1, 1)
+    if rope is not None:
+        cos, sin = rope
+        cs = cos[token_start:token_start + L].float().view(1, 1, L, c // 2)
+        sn = sin[token_start:token_start + L].float().view(1, 1, L, c // 2)
+
+        def rotate(x):
+            x2 = x.reshape(*x.shape[:-1], c // 2, 2)
+            even = cs * x2[..., 0] - sn * x2[..., 1]
+            odd = sn * x2[..., 0] + cs * x2[..., 1]
+            return torch.stack([even, odd], dim=-1).reshape(x.shape)
+
+        qf, kf = rotate(qf), rotate(kf)
+    return qf.to(torch.bfloat16), kf, v

@@ -119,3 +119,56 @@ def test_unquantized_cache_path_matches_full_sequence_attention(dev):
     bias = O.block_causal_bias(pn).to(dev).view(1, 1, L, L)
     full = m(torch.cat(xs, dim=1), attn_bias=bias)
     assert torch.allclose(steps, full, atol=2e-5)
+
+
+def test_infinity_fused_producer_vs_unfused(dev):
+    """The one-kernel producer (normalise + scale + rotate + quantize into the cache) inside
+    the module: same outputs as the unfused drop-in within the attention tolerance, and a
+    cache that dequantizes to the unfused one within one quantization step (torch's own
+    normalisation on the GPU rounds differently, so a code can move by one)."""
+    torch.manual_seed(7)
+    C, H = 1024, 8
+    hw = [(p, p) for p in (1, 2, 4, 6, 8, 12)]
+    total = sum(h * w for h, w in hw)
+    rope = hooks.rope2d_tables(C // H, hw)
+    kw = dict(embed_dim=C, num_heads=H, layout='BHLc', q_bits=4, quant_method='G_GROUP', group_size=128,
+              symmetric=False, enable_quantization=True, max_tokens=total)
+    a_mod = hooks.InfinitySelfAttention(fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.InfinitySelfAttention(fused=True, fused_producer=True, **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    start = 0
+    for h, w in hw:
+        note('hooks infinity fused producer', h, w)
+        x = torch.randn(2, h * w, C, device=dev, dtype=torch.bfloat16)
+        a = a_mod(x, rope=rope, token_start=start).float()
+        b = b_mod(x, rope=rope, token_start=start).float()
+        start += h * w
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), ((h, w), (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995
+    ka, kb = a_mod.k_quant.dequant_all(), b_mod.packed_cache.dequant('k')
+    step = a_mod.k_quant.cached_scale.max().item()
+    assert (ka - kb).abs().max().item() <= 1.01 * step
+    assert (ka != kb).float().mean().item() < 0.02
+
+
+@pytest.mark.parametrize('layout', ['BLHc', 'BHLc'])
+def test_var_fused_producer_vs_unfused(dev, layout):
+    torch.manual_seed(8)
+    C, H = 512, 8
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, q_bits=8, quant_method='G_GROUP', group_size=64,
+              symmetric=True, enable_quantization=True, max_tokens=100)
+    a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.VarSelfAttention(0, fused=True, fused_producer=True, **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    for p in (1, 2, 3, 4, 5, 6):
+        note('hooks var fused producer', layout, p)
+        x = torch.randn(4, p * p, C, device=dev, dtype=torch.bfloat16)
+        a, b = a_mod(x).float(), b_mod(x).float()
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0)
+        assert _cos(a, b) >= 0.9995

@@ -1,0 +1,108 @@
+"""Producer-side fusion (normalise + scale + rotate + quantize into the cache in one
+kernel) against the CPU oracle: the prepared q (bf16), the packed words, scales and
+zero-points of k and v are bit-exact, because the oracle fixes the one thing the
+reference's tensor expressions leave open, the summation order of the norm."""
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import note
+from var_q_amd import PackedKVCache, hooks, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(dev, B, L, H, c, dtype, bits, group, asym, l2norm, with_mul, with_rope, start=0, Lmax=None, off=0):
+    g = torch.Generator().manual_seed(B * 131 + L * 17 + c + bits)
+    qkv = (torch.randn(B, L, 3, H, c, generator=g) * 1.7).to(dtype)
+    qkv[..., 3] *= 9
+    mul = (torch.rand(H, generator=g) * 5 + 0.5) if with_mul else None
+    rope = None
+    if with_rope:
+        hw = [(3, 4), (5, 5), (8, 8)]
+        rope = hooks.rope2d_tables(c, hw)
+        assert rope[0].shape[0] >= start + L
+    qo, ko, vo = O.prepare_qkv(qkv, mul, l2norm, 1e-12, rope, start)
+    Lmax = Lmax or (L + off)
+    W, ns = c * bits // 32, c // group
+    mk = lambda last, dt: torch.full((B, H, Lmax, last), 7, dtype=dt, device=dev)
+    kw, vw = mk(W, torch.int32), mk(W, torch.int32)
+    ks, kz, vs, vz = (mk(ns, torch.float32) for _ in range(4))
+    q_out = torch.empty(B, H, L, c, dtype=torch.bfloat16, device=dev)
+    rowmap = [B, L, H, H * Lmax, 1, Lmax, off, -1]
+    ops.qkv_prepare_append(qkv.to(dev), q_out, group, bits, asym, 1e-12, kw, ks, kz if asym else None,
+                           vw, vs, vz if asym else None, rowmap, None,
+                           None if mul is None else mul.to(dev), l2norm, 1e-12,
+                           None if rope is None else (rope[0].to(dev), rope[1].to(dev)), start)
+    torch.cuda.synchronize()
+    assert torch.equal(q_out.cpu().view(torch.int16), qo.view(torch.int16)), 'prepared q differs'
+    for name, x, w, s, z in (('k', ko, kw, ks, kz), ('v', vo, vw, vs, vz)):
+        cq, cs, cz = O.quant_groupwise(x, group, bits, asym)
+        want, _ = O.pack_last_dim(cq, bits)
+        sl = slice(off, off + L)
+        assert torch.equal(s[:, :, sl].cpu(), cs), f'{name} scale differs'
+        if asym:
+            assert torch.equal(z[:, :, sl].cpu(), cz), f'{name} zero-point differs'
+        assert torch.equal(w[:, :, sl].cpu(), want), f'{name} packed words differ'
+        if off:
+            assert bool((w[:, :, :off] == 7).all()) and bool((s[:, :, :off] == 7).all()), 'rows outside the step touched'
+
+
+@pytest.mark.parametrize('c,group', [(64, 64), (64, 32), (128, 128), (128, 64), (128, 16), (32, 32)])
+@pytest.mark.parametrize('bits,asym', [(4, True), (8, False), (2, True)])
+def test_infinity_style_norm_scale_rope(dev, c, group, bits, asym):
+    for dtype in (torch.bfloat16, torch.float32):
+        note('qkv_prepare infinity', c, group, bits, asym, dtype)
+        _run(dev, 2, 9, 3, c, dtype, bits, group, asym, True, True, True, start=5, Lmax=20, off=4)
+
+
+@pytest.mark.parametrize('l2norm,with_mul,with_rope', [(False, False, False), (True, False, False), (True, True, False),
+                                                       (False, False, True)])
+def test_var_style_and_partial_pipelines(dev, l2norm, with_mul, with_rope):
+    note('qkv_prepare var', l2norm, with_mul, with_rope)
+    _run(dev, 3, 16, 5, 64, torch.float16, 4, 64, True, l2norm, with_mul, with_rope)
+    _run(dev, 1, 1, 1, 128, torch.bfloat16, 8, 128, False, l2norm, with_mul, with_rope)
+
+
+def test_zero_rows_and_tiny_norms(dev):
+    """An all-zero token (norm clamps to eps) and denormal-sized rows."""
+    B, L, H, c = 1, 4, 2, 64
+    qkv = torch.randn(B, L, 3, H, c, generator=torch.Generator().manual_seed(9))
+    qkv[0, 1] = 0.0
+    qkv[0, 2] *= 1e-30
+    q_ref, k_ref, _ = O.prepare_qkv(qkv, None, True)
+    kw = torch.zeros(B, H, L, c // 8, dtype=torch.int32, device=dev)
+    vw = torch.zeros_like(kw)
+    ks, kz, vs, vz = (torch.zeros(B, H, L, 1, device=dev) for _ in range(4))
+    q_out = torch.empty(B, H, L, c, dtype=torch.bfloat16, device=dev)
+    note('qkv_prepare zero rows')
+    ops.qkv_prepare_append(qkv.to(dev), q_out, 64, 4, True, 1e-12, kw, ks, kz, vw, vs, vz, [B, L, H, H * L, 1, L, 0, -1],
+                           l2norm=True)
+    assert torch.equal(q_out.cpu().view(torch.int16), q_ref.view(torch.int16))
+    cq, cs, cz = O.quant_groupwise(k_ref, 64, 4, True)
+    assert torch.equal(ks.cpu(), cs) and torch.equal(kz.cpu(), cz) and torch.equal(kw.cpu(), O.pack_last_dim(cq, 4)[0])
+
+
+def test_cache_append_from_qkv_mixed_bits(dev):
+    """Through the cache class, heads of different widths: equals preparing on the CPU
+    and appending k, v the ordinary way."""
+    B, H, D = 2, 6, 128
+    bits = [4, 8, 2, 4, 8, 2]
+    hw = [(1, 1), (2, 2), (4, 4)]
+    rope = hooks.rope2d_tables(D, hw)
+    rope_d = (rope[0].to(dev), rope[1].to(dev))
+    mul = torch.rand(H, generator=torch.Generator().manual_seed(2)) * 3 + 1
+    a = PackedKVCache(B, H, 21, D, bits, 64, dev)
+    b = PackedKVCache(B, H, 21, D, bits, 64, dev)
+    g = torch.Generator().manual_seed(3)
+    for h_, w_ in hw:
+        n = h_ * w_
+        qkv = torch.randn(B, n, 3, H, D, generator=g).bfloat16()
+        start = a.len
+        note('qkv_prepare cache', n)
+        q_gpu = a.append_from_qkv(qkv.to(dev), mul.to(dev), True, 1e-12, rope_d)
+        q_ref, k_ref, v_ref = O.prepare_qkv(qkv, mul, True, 1e-12, rope, start)
+        b.append(k_ref.to(dev), v_ref.to(dev))
+        assert torch.equal(q_gpu.cpu().view(torch.int16), q_ref.view(torch.int16))
+    assert a.len == b.len == 21
+    assert torch.equal(a.dequant('k'), b.dequant('k')) and torch.equal(a.dequant('v'), b.dequant('v'))

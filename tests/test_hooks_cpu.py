@@ -109,3 +109,26 @@ def test_infinity_module_rope_offsets_and_cache():
     assert plain.cached_k.shape == (2, H, 21, C // H)
     # the cached keys are unit vectors: normalisation and rotation both preserve that
     assert torch.allclose(plain.cached_k.norm(dim=-1), torch.ones(2, H, 21), atol=1e-5)
+
+
+def test_oracle_prepare_qkv_follows_the_reference_expressions():
+    """The oracle of the fused producer fixes a summation order for the norm; against
+    torch's own F.normalize / scale / rotation (the reference's expressions,
+    Infinity basic.py:316-330 and :103-123) it may differ by rounding only."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(8)
+    B, L, H, c = 2, 9, 3, 64
+    qkv = torch.randn(B, L, 3, H, c, generator=g)
+    mul = torch.rand(H, generator=g) * 4 + 1
+    rope = hooks.rope2d_tables(c, [(2, 2), (3, 3)])
+    q, k, v = O.prepare_qkv(qkv, mul, True, 1e-12, rope, 4)
+    qr, kr, vr = (qkv[:, :, t].permute(0, 2, 1, 3) for t in range(3))
+    qn = F.normalize(qr, dim=-1, eps=1e-12).mul(mul.view(1, H, 1, 1))
+    kn = F.normalize(kr, dim=-1, eps=1e-12)
+    qn, kn = hooks.apply_rope2d(qn, rope[0], rope[1], 4, 2), hooks.apply_rope2d(kn, rope[0], rope[1], 4, 2)
+    assert torch.allclose(k, kn, atol=2e-7, rtol=1e-6)
+    assert torch.allclose(q.float(), qn, atol=0, rtol=2 ** -7)          # bf16 result
+    assert torch.equal(v, vr)
+    # without normalisation and rotation the data passes through
+    q2, k2, _ = O.prepare_qkv(qkv.bfloat16())
+    assert torch.equal(k2, kr.bfloat16().float()) and torch.equal(q2, qr.bfloat16())

@@ -27,6 +27,12 @@ SYMBOLS = {
                                 c_int, c_int, c_int, c_void_p,
                                 c_int, c_int, c_int, c_int,
                                 c_void_p, c_float, c_void_p]),
+    'varq_qkv_prepare_append': (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                        c_void_p, c_int, c_float,
+                                        c_void_p, c_void_p, c_int,
+                                        c_void_p, c_int, c_int, c_int, c_float,
+                                        POINTER(c_int64), c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
 
 _lib = None

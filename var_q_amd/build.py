@@ -28,6 +28,7 @@ FLAGS = {
     'quant_general.hip': ['-ffp-contract=off'],
     'pack_unpack.hip': ['-ffp-contract=off'],
     'dequant.hip': ['-ffp-contract=off'],
+    'qkv_prepare.hip': ['-ffp-contract=off'],
     'fused_attn.hip': [],
 }
 

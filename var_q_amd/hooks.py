@@ -18,7 +18,9 @@ cached.  Two backends behind the same interface:
   * `fused=True`: `PackedKVCache.append` + `PackedKVCache.attend`: the step is
     quantized in place into a pre-allocated packed cache and attention reads the
     packed codes; no dequantized K/V exists.  Needs a row-local quantizer
-    (`quant_method='G_GROUP'`).
+    (`quant_method='G_GROUP'`).  With `fused_producer=True` the normalisation,
+    the per-head scale of q, the rotation and the quantization of k and v run as
+    one kernel on the qkv projection output (`PackedKVCache.append_from_qkv`).
 
 The transformer blocks around the attention (AdaLN, FFN, cross-attention) are
 outside this package.
@@ -83,13 +85,15 @@ class _QuantizedSelfAttention(nn.Module):
 
     def __init__(self, embed_dim: int, num_heads: int, layout: str, q_bits, quant_method: str, enable_quantization: bool,
                  fused: bool, group_size: Optional[int], symmetric: bool, max_tokens: int, block_idx: int,
-                 quantizer_factory: Optional[Callable] = None):
+                 quantizer_factory: Optional[Callable] = None, fused_producer: bool = False):
         super().__init__()
         assert embed_dim % num_heads == 0 and layout in ('BLHc', 'BHLc')
         self.num_heads, self.head_dim = num_heads, embed_dim // num_heads
         self.layout, self.block_idx = layout, block_idx
         self.q_bits, self.quant_method, self.enable_quantization = q_bits, quant_method, enable_quantization
         self.fused, self.group_size, self.symmetric, self.max_tokens = fused, group_size, symmetric, max_tokens
+        self.fused_producer = fused_producer
+        assert fused or not fused_producer, 'fused_producer needs the fused backend'
         self._quantizer_factory = quantizer_factory or VAR_Q
         if fused:
             assert enable_quantization and quant_method == 'G_GROUP' and group_size, \
@@ -114,10 +118,13 @@ class _QuantizedSelfAttention(nn.Module):
             self.k_quant = self._quantizer_factory(**kw)
             self.v_quant = self._quantizer_factory(**kw)
 
-    def _project(self, x):
+    def _qkv(self, x):
         B, L, _ = x.shape
         bias = torch.cat((self.q_bias, self.zero_k_bias, self.v_bias))
-        qkv = F.linear(x, self.mat_qkv.weight.to(x.dtype), bias.to(x.dtype)).view(B, L, 3, self.num_heads, self.head_dim)
+        return F.linear(x, self.mat_qkv.weight.to(x.dtype), bias.to(x.dtype)).view(B, L, 3, self.num_heads, self.head_dim)
+
+    def _project(self, x):
+        qkv = self._qkv(x)
         if self.layout == 'BLHc':
             return qkv.unbind(dim=2)                       # each [B,L,H,c]
         return qkv.permute(2, 0, 3, 1, 4).unbind(dim=0)     # each [B,H,L,c]
@@ -131,6 +138,21 @@ class _QuantizedSelfAttention(nn.Module):
         o = F.scaled_dot_product_attention(q.to(out_dtype), k.to(out_dtype), v.to(out_dtype), scale=scale,
                                            attn_mask=None if attn_bias is None else attn_bias.to(out_dtype))
         return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim)
+
+    def _fused_from_qkv(self, x, scale: float, scale_mul, l2norm: bool, rope, token_start, attn_bias):
+        """qkv projection -> one producer kernel (normalise, scale, rotate, quantize into the
+        cache) -> fused attention; returns [B,L,C]."""
+        if attn_bias is not None:
+            raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')
+        qkv = self._qkv(x)
+        B, L = qkv.shape[:2]
+        if self.packed_cache is None:
+            self.packed_cache = PackedKVCache(B, self.num_heads, self.max_tokens, self.head_dim, self.q_bits,
+                                              self.group_size, qkv.device, symmetric=self.symmetric)
+        mul = None if scale_mul is None else scale_mul.detach().float().reshape(-1).contiguous()
+        q = self.packed_cache.append_from_qkv(qkv, mul, l2norm, 1e-12, rope, token_start)
+        o = self.packed_cache.attend(q, scale)                                          # [B,H,L,c]
+        return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(x.dtype)
 
     def _cache_and_attend(self, q, k, v, scale: float, attn_bias, out_dtype):
         B = q.shape[0]
@@ -166,9 +188,9 @@ class VarSelfAttention(_QuantizedSelfAttention):
     def __init__(self, block_idx: int, embed_dim: int = 1024, num_heads: int = 16, attn_l2_norm: bool = True,
                  layout: str = 'BLHc', q_bits=8, quant_method: str = 'G_SCALE_HEAD_DIM', enable_quantization: bool = False,
                  fused: bool = False, group_size: Optional[int] = None, symmetric: bool = True, max_tokens: int = 680,
-                 quantizer_factory: Optional[Callable] = None):
+                 quantizer_factory: Optional[Callable] = None, fused_producer: bool = False):
         super().__init__(embed_dim, num_heads, layout, q_bits, quant_method, enable_quantization, fused, group_size,
-                         symmetric, max_tokens, block_idx, quantizer_factory)
+                         symmetric, max_tokens, block_idx, quantizer_factory, fused_producer)
         self.attn_l2_norm = attn_l2_norm
         if attn_l2_norm:
             self.scale = 1.0
@@ -178,6 +200,10 @@ class VarSelfAttention(_QuantizedSelfAttention):
             self.scale = 0.25 / math.sqrt(self.head_dim)
 
     def forward(self, x: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if self.caching and self.fused_producer:
+            mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp() if self.attn_l2_norm else None
+            o = self._fused_from_qkv(x, self.scale, mul, self.attn_l2_norm, None, None, attn_bias)
+            return self.proj(o.to(self.proj.weight.dtype))
         q, k, v = self._project(x)
         main_type = x.dtype
         if self.attn_l2_norm:
@@ -199,9 +225,9 @@ class InfinitySelfAttention(_QuantizedSelfAttention):
     def __init__(self, embed_dim: int = 2048, num_heads: int = 16, tau: float = 1.0, cos_attn: bool = True,
                  layout: str = 'BHLc', q_bits=8, quant_method: str = 'G_SCALE_HEAD_DIM', enable_quantization: bool = False,
                  fused: bool = False, group_size: Optional[int] = None, symmetric: bool = True, max_tokens: int = 10521,
-                 block_idx: int = 0, quantizer_factory: Optional[Callable] = None):
+                 block_idx: int = 0, quantizer_factory: Optional[Callable] = None, fused_producer: bool = False):
         super().__init__(embed_dim, num_heads, layout, q_bits, quant_method, enable_quantization, fused, group_size,
-                         symmetric, max_tokens, block_idx, quantizer_factory)
+                         symmetric, max_tokens, block_idx, quantizer_factory, fused_producer)
         self.tau, self.cos_attn = tau, cos_attn
         if cos_attn:
             self.scale = 1.0
@@ -215,6 +241,13 @@ class InfinitySelfAttention(_QuantizedSelfAttention):
                 rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, token_start: int = 0) -> torch.Tensor:
         """rope = (cos, sin) from rope2d_tables for the whole schedule; token_start =
         number of tokens of the scales before this one."""
+        if self.caching and self.fused_producer:
+            mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp() if self.cos_attn else None
+            rope_dev = None
+            if rope is not None:
+                rope_dev = tuple(t.to(x.device, torch.float32).contiguous() for t in rope)
+            o = self._fused_from_qkv(x, self.scale, mul, self.cos_attn, rope_dev, token_start, attn_bias)
+            return self.proj(o.to(self.proj.weight.dtype))
         q, k, v = self._project(x)
         main_type = x.dtype
         if self.cos_attn:

@@ -137,6 +137,28 @@ class PackedKVCache:
                                      c.v_zp if asym else None, rowmap, c.slot)
         self.len += n
 
+    def append_from_qkv(self, qkv: torch.Tensor, q_scale_mul: Optional[torch.Tensor] = None, l2norm: bool = False,
+                        norm_eps: float = 1e-12, rope=None, token_start: Optional[int] = None) -> torch.Tensor:
+        """One pass from the qkv projection output [B,n,3,H,D] to the cache: k (l2-normalised and
+        rotated if asked) and v are quantized into tokens len..len+n, the prepared q comes back
+        as bf16 [B,H,n,D] (Infinity/infinity/models/basic.py:316-330 in one kernel).
+        token_start (default: the cache length) selects the rotary table rows."""
+        B, n, three, H, D = qkv.shape
+        assert three == 3 and (B, H, D) == (self.B, self.H, self.D)
+        assert self.len + n <= self.Lmax, 'cache overflow'
+        qkv = qkv.contiguous()
+        q_out = torch.empty((B, H, n, D), dtype=torch.bfloat16, device=qkv.device)
+        asym = not self.symmetric
+        start = self.len if token_start is None else token_start
+        for c in self.classes:
+            hc = len(c.heads)
+            rowmap = [B, n, H, hc * self.Lmax, 1, self.Lmax, self.len, 2]
+            ops.qkv_prepare_append(qkv, q_out, self.group, c.bits, asym, self.eps, c.k_words, c.k_scale,
+                                   c.k_zp if asym else None, c.v_words, c.v_scale, c.v_zp if asym else None,
+                                   rowmap, c.slot, q_scale_mul, l2norm, norm_eps, rope, start)
+        self.len += n
+        return q_out
+
     def attend(self, q: torch.Tensor, softmax_scale: float, kv_limit: Optional[torch.Tensor] = None,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fused dequant attention of q [B,H,Lq,D] (bf16) over the cached tokens."""

@@ -201,6 +201,41 @@ def dequant_window(words: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.
 
 
 # ---------------------------------------------------------------------------
+# producer side: normalise + rotate + quantize straight into the cache
+# ---------------------------------------------------------------------------
+def qkv_prepare_append(qkv: torch.Tensor, q_out: torch.Tensor, group: int, bits: int, asym: bool, eps: float,
+                       k_words: torch.Tensor, k_scale: torch.Tensor, k_zp: Optional[torch.Tensor],
+                       v_words: torch.Tensor, v_scale: torch.Tensor, v_zp: Optional[torch.Tensor],
+                       rowmap: Sequence[int], slot: Optional[torch.Tensor] = None,
+                       q_scale_mul: Optional[torch.Tensor] = None, l2norm: bool = False, norm_eps: float = 1e-12,
+                       rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, token_start: int = 0) -> None:
+    """qkv [B,L,3,H,c] (output of the qkv projection) -> q_out [B,H,L,c] bf16 (normalised,
+    scaled per head, rotated) and k, v quantized into the cache buffers through a row map
+    over (B, L, H) (see include/varq.h)."""
+    _gpu(qkv, 'qkv'); _gpu(q_out, 'q_out')
+    assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous()
+    B, L, _, H, c = qkv.shape
+    assert q_out.shape == (B, H, L, c) and q_out.dtype == torch.bfloat16 and q_out.is_contiguous()
+    assert list(rowmap[:3]) == [B, L, H]
+    cos = sin = None
+    if rope is not None:
+        cos, sin = rope
+        _gpu(cos, 'rope cos'); _gpu(sin, 'rope sin')
+        assert cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+        assert cos.shape == sin.shape and cos.shape[1] == c // 2 and cos.shape[0] >= token_start + L
+    if q_scale_mul is not None:
+        _gpu(q_scale_mul, 'q_scale_mul')
+        assert q_scale_mul.dtype == torch.float32 and q_scale_mul.numel() == H and q_scale_mul.is_contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(qkv.device):
+        check(lib.varq_qkv_prepare_append(qkv.data_ptr(), _dt(qkv), B, L, H, c, _ptr(q_scale_mul), int(l2norm), norm_eps,
+                                          _ptr(cos), _ptr(sin), token_start, q_out.data_ptr(), group, bits, int(asym), eps,
+                                          i64arr(rowmap), _ptr(slot), k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp),
+                                          v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), _stream(qkv)),
+              'varq_qkv_prepare_append')
+
+
+# ---------------------------------------------------------------------------
 # fused dequant flash-attention
 # ---------------------------------------------------------------------------
 def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_zp: Optional[torch.Tensor],
