@@ -48,9 +48,9 @@ template <int LANES> __device__ __forceinline__ float group_allsum(float v) {
   return v;
 }
 
-// x / d as IEEE division rounds it (see quant_rows.hip for the argument)
-__device__ __forceinline__ float exact_div(float x, float d, float r, bool plain) {
-  if (!plain) return x / d;
+// x / d as IEEE division rounds it, for a divisor that passed plain_divisor (see
+// quant_rows.hip for the argument); r = RN(1/d)
+__device__ __forceinline__ float exact_div(float x, float d, float r) {
   const float q0 = x * r;
   return __builtin_fmaf(__builtin_fmaf(-q0, d, x), r, q0);
 }
@@ -78,12 +78,22 @@ __device__ __forceinline__ void quant_octet(const float (&v)[8], float eps, floa
   const float s = ASYM ? fmaxf((mx - mn) / (float)QRange<BITS>::kLevels, eps) : fmaxf(mx / kMax, eps);
   const float r = 1.0f / s;
   const bool plain = plain_divisor(s);
-  const float zp = ASYM ? kMin - rintf(mn / s) : 0.f;
+  // the shortcut or the division for the whole wavefront: no per-element branches
+  const bool wave_plain = __builtin_amdgcn_ballot_w64(!plain) == 0;
+  const float zp = ASYM ? kMin - rintf(wave_plain ? exact_div(mn, s, r) : mn / s) : 0.f;
+  float t[8];
+  if (wave_plain) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = exact_div(v[j], s, r);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = v[j] / s;
+  }
   u32 acc = 0;
   w0 = 0; w1 = 0;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const float n = rintf(exact_div(v[j], s, r, plain));
+    const float n = rintf(t[j]);
     const int q = (int)__builtin_amdgcn_fmed3f(ASYM ? n + zp : n, kMin, kMax);
     acc = __builtin_amdgcn_alignbit((u32)q, acc, BITS);
     if (BITS == 8 && j == 3) { w0 = acc; acc = 0; }
@@ -97,16 +107,19 @@ __device__ __forceinline__ void quant_octet(const float (&v)[8], float eps, floa
 // One lane = 8 channels of one (b, l, h); LR = c/8 lanes form the row, LG = group/8 a group.
 template <int DT, int BITS, bool ASYM, int LR, int LG>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
-  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t r = o / LR;
+  // Lanes walk the (b, h, l) order of the outputs, so the prepared q, the packed words and
+  // the scales of a wavefront are contiguous; the reads are whole 16*LR-byte rows either way.
+  const u32 o = blockIdx.x * 256u + threadIdx.x;      // < 2^31 (checked on the host)
+  const u32 r = o / LR;
   const int col = (int)(o - r * LR);
-  const bool live = r < p.rows;
-  const int64_t rc = live ? r : p.rows - 1;          // idle lanes recompute the last row, never store
-  const int h = (int)(rc % p.H);
-  const int64_t bl = rc / p.H;
-  const int l = (int)(bl % p.L);
-  const int b = (int)(bl / p.L);
+  const bool live = r < (u32)p.rows;
+  const u32 rc = live ? r : (u32)p.rows - 1u;         // idle lanes recompute the last row, never store
+  const int l = (int)(rc % (u32)p.L);
+  const u32 bh = rc / (u32)p.L;
+  const int h = (int)(bh % (u32)p.H);
+  const int b = (int)(bh / (u32)p.H);
   const int c = p.c;
+  const int64_t bl = (int64_t)b * p.L + l;
   const int64_t base = (bl * 3) * (int64_t)p.H * c + (int64_t)h * c + col * 8;
   const int64_t tstride = (int64_t)p.H * c;
 
@@ -125,11 +138,16 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     const float rq = 1.0f / dq, rk = 1.0f / dk;
     const bool pq = plain_divisor(dq), pk = plain_divisor(dk);
     const float mul = p.scale_mul ? p.scale_mul[h] : 1.f;
+    if (__builtin_amdgcn_ballot_w64(!(pq && pk)) == 0) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      q[j] = exact_div(q[j], dq, rq, pq);
-      if (p.scale_mul) q[j] = q[j] * mul;
-      k[j] = exact_div(k[j], dk, rk, pk);
+      for (int j = 0; j < 8; ++j) { q[j] = exact_div(q[j], dq, rq); k[j] = exact_div(k[j], dk, rk); }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { q[j] = q[j] / dq; k[j] = k[j] / dk; }
+    }
+    if (p.scale_mul) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q[j] = q[j] * mul;
     }
   }
   if (p.cos) {
@@ -246,7 +264,7 @@ extern "C" int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int 
   VARQ_CHECK_ARG(qkv && q_out && k_words && v_words && k_scale && v_scale && (!asym || (k_zp && v_zp)) && host_rowmap,
                  "qkv_prepare: null pointer");
   VARQ_CHECK_ARG(((uintptr_t)qkv & 15) == 0 && ((uintptr_t)q_out & 15) == 0, "qkv_prepare: qkv and q_out must be 16-byte aligned");
-  VARQ_CHECK_ARG(rows * (c / 8) < (1ll << 40), "qkv_prepare: tensor too large");
+  VARQ_CHECK_ARG(rows * (c / 8) < (1ll << 31) - 256, "qkv_prepare: tensor too large");
 
   PrepParams p;
   p.qkv = qkv; p.scale_mul = q_scale_mul; p.cos = rope_cos; p.sin = rope_sin; p.q_out = q_out;
