@@ -34,10 +34,23 @@ template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t ele
       for (int j = 0; j < n_valid; ++j) o[j] = f[j];
     }
   } else {
+    uint16_t *o = reinterpret_cast<uint16_t *>(out) + elem;
+    if (ODT == VARQ_BF16 && n_valid == 8) {
+      // hardware round-to-nearest-even conversion, two values per instruction
+      typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+      typedef float f2 __attribute__((ext_vector_type(2)));
+      u32 w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f2 v = {f[2 * j], f[2 * j + 1]};
+        w[j] = __builtin_bit_cast(u32, __builtin_convertvector(v, bf2));
+      }
+      *reinterpret_cast<uint4 *>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+      return;
+    }
     uint16_t h[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) h[j] = (ODT == VARQ_BF16) ? f32_to_bf16_rne(f[j]) : f32_to_f16_rne(f[j]);
-    uint16_t *o = reinterpret_cast<uint16_t *>(out) + elem;
     if (n_valid == 8) {
       *reinterpret_cast<uint4 *>(o) = make_uint4(h[0] | ((u32)h[1] << 16), h[2] | ((u32)h[3] << 16),
                                                  h[4] | ((u32)h[5] << 16), h[6] | ((u32)h[7] << 16));
