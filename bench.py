@@ -1,12 +1,12 @@
 #!/usr/bin/env python3
 """Benchmark of the VAR-Q hot path on one MI355X.
 
-One step = one pass over BASELINE config 4 (Infinity-2B shape): quantize+pack K
+One step = one pass over benchmark configuration 4 (Infinity-2B shape): quantize+pack K
 and V [2,16,10521,128] bf16 to INT4 group-128 asymmetric, then fused dequant
 attention of the final scale's 4096 queries over all 10521 packed keys.  Inputs
 are resident in HBM before the timed region.  Prints ONE JSON line.
 
-After the timed region (and outside `value`) it also replays BASELINE config 5,
+After the timed region (and outside `value`) it also replays benchmark configuration 5,
 one image batch of the Infinity schedule through the pre-allocated mixed-bit
 cache (append + attend per scale), and reports its latency per image.
 
@@ -221,7 +221,7 @@ def main():
         'value': round(kv_gbps, 3), 'unit': 'GB/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'bf16 MFMA over int4 codes, fp32 scales', 'data': 'synthetic',
+        'dtype': 'bf16', 'dtype_detail': 'bf16 MFMA operands holding exact int4 codes, fp32 scales and accumulation', 'data': 'synthetic',
         'config': {'workload': 'config 4: Infinity-2B KV [B=2,H=16,L=10521,D=128] bf16 -> INT4 group-128 asymmetric '
                                'quantize+pack of K and V, then fused dequant attention of the final 4096 queries',
                    'B': B, 'H': H, 'L': L, 'D': D, 'Lq': LQ, 'bits': BITS, 'group': GROUP, 'input_sets_cycled': NBUF},

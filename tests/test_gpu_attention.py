@@ -7,7 +7,7 @@ How the tolerance is applied, and why.  The kernel multiplies the integer codes
 exactly and applies scales/zero-points in fp32; the oracle first rounds the
 dequantized K and V to bf16 (as the reference's attention backends do).  On
 unit-range data the two agree to well inside 2e-2.  On the heavy-tailed
-BASELINE config-4 data (outputs up to ~95, where one bf16 ulp is 0.5) the
+the Infinity-2B benchmark data (configuration 4) (outputs up to ~95, where one bf16 ulp is 0.5) the
 oracle's operand rounding alone moves ITS output by up to ~4 from the fp64
 value, while the kernel stays within ~0.3 of it.  So the checks are:
     cosine(out, oracle) >= 0.9995                                   (literal)
@@ -117,13 +117,13 @@ def test_block_causal_mask_multi_scale_queries(dev):
 
 
 def test_config2_var_d16_batch(dev):
-    """BASELINE config 2 (batch cut to 4 for the CPU oracle): K g=32, V g=64,
+    """benchmark configuration 2 (batch cut to 4 for the CPU oracle): K g=32, V g=64,
     INT4, final-scale 256 queries over 680 keys, all visible."""
     _run(dev, 4, 16, 256, 680, 64, 4, 32, 64, seed=2002, what='c2')
 
 
 def test_config4_infinity2b_subset(dev):
-    """BASELINE config 4 at full sequence length for a subset of heads:
+    """benchmark configuration 4 at full sequence length for a subset of heads:
     Student-t data with x20 outlier channels, INT4 g=128, final 4096 queries."""
     _run(dev, 1, 2, 4096, 10521, 128, 4, 128, 128, seed=4004, dist='student4', what='c4 subset')
 

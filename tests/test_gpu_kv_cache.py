@@ -1,5 +1,5 @@
 """Incremental generation over a scale schedule with the pre-allocated packed
-cache: append a step, attend with that step's queries (BASELINE config 5 in
+cache: append a step, attend with that step's queries (benchmark configuration 5 in
 miniature, mixed per-head bit-widths)."""
 import math
 

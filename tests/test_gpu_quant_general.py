@@ -81,7 +81,7 @@ def test_adversarial_values(dev):
 
 
 def test_var_d30_shapes(dev):
-    """BASELINE config 3 (batch reduced for the CPU oracle): INT2 asymmetric
+    """benchmark configuration 3 (batch reduced for the CPU oracle): INT2 asymmetric
     per-head-per-dim and INT8 symmetric per-channel on [B,30,680,64] bf16."""
     x = O.synth_kv((4, 30, 680, 64), seed=1003, dtype=torch.bfloat16)
     note('general c3 int2 asym per-head-per-dim')
@@ -91,7 +91,7 @@ def test_var_d30_shapes(dev):
 
 
 def test_var_d16_per_head_int8_fp32(dev):
-    """BASELINE config 1: fp32 [2,16,680,64], INT8 symmetric per-head."""
+    """benchmark configuration 1: fp32 [2,16,680,64], INT8 symmetric per-head."""
     note('general c1')
     x = O.synth_kv((2, 16, 680, 64), seed=1001)
     _check(x, (0, 2, 3), 8, False, True, dev)

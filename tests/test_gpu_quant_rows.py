@@ -98,7 +98,7 @@ def test_empty_and_single_row(dev):
 
 
 def test_infinity2b_full_shape_int4_g128(dev):
-    """BASELINE config 4 at full size: [2,16,10521,128] bf16, INT4 asym g=128."""
+    """benchmark configuration 4 at full size: [2,16,10521,128] bf16, INT4 asym g=128."""
     note('quant_rows c4 full')
     x = O.synth_kv((2, 16, 10521, 128), seed=1004, dist='student4', outlier_frac=0.01, outlier_mul=20.0,
                    dtype=torch.bfloat16)
@@ -106,7 +106,7 @@ def test_infinity2b_full_shape_int4_g128(dev):
 
 
 def test_var_d16_batch_shape_int4(dev):
-    """BASELINE config 2 shapes (B reduced to 8 to keep the CPU oracle quick):
+    """benchmark configuration 2 shapes (B reduced to 8 to keep the CPU oracle quick):
     K group 32, V group 64."""
     note('quant_rows c2')
     k = O.synth_kv((8, 16, 680, 64), seed=1002, dtype=torch.bfloat16)
