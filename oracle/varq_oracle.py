@@ -25,6 +25,10 @@ Pinning status
                                       constant group, error bound scale/2)
   attention_ref (EXTENSION)           torch SDPA (library) on bf16 operands;
                                       checked against an fp64 softmax formula
+  prepare_qkv (EXTENSION)             parity unpinned by reference (its norm's
+                                      summation order is the backend's); checked
+                                      against torch's F.normalize / scale /
+                                      rotation to rounding, norm-preservation
 """
 from __future__ import annotations
 
