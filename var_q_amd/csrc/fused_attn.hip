@@ -642,7 +642,11 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     float zmax = z[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
-    zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+    {
+      // the other lane half of the same query, without a trip through LDS
+      const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
+      zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
+    }
     if (first || __any(zmax > kRescaleAt)) {
       // Move the reference to the row's current maximum: up only (never down) once
       // something has been accumulated; the very first block takes its maximum as it
