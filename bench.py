@@ -10,7 +10,7 @@ After the timed region (and outside `value`) it also replays benchmark configura
 one image batch of the Infinity schedule through the pre-allocated mixed-bit
 cache (append + attend per scale), and reports its latency per image.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5] [--no-c3]
 """
 import argparse
 import json
@@ -101,6 +101,48 @@ def c5_latency(torch, dev, passes=10, warm=3):
             'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes}
 
 
+def c3_rates(torch, dev, reps=20, warm=5):
+    """Config 3: VAR-d30 shape, K/V bf16 [32,30,680,64], quantized per (head, channel) over
+    batch and tokens: (i) INT2 asymmetric, (ii) INT8 symmetric (the reference's
+    G_SCALE_HEAD_DIM).  Times quantize+pack, unpack+dequant (bf16 out) and the fused
+    attention of the final 256 queries, with CUDA events around `reps` launches each."""
+    from var_q_amd import ops
+    B3, H3, L3, D3, LQ3 = 32, 30, 680, 64, 256
+    gd = torch.Generator(device=dev).manual_seed(3003)
+    k, v = (torch.randn(B3, H3, L3, D3, device=dev, generator=gd).bfloat16() for _ in range(2))
+    q = torch.randn(B3, H3, LQ3, D3, device=dev, generator=gd).bfloat16()
+
+    def timed(fn):
+        for _ in range(warm):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    out = {'workload': 'config 3: VAR-d30 K/V bf16 [32,30,680,64], one (scale, zp) per (head, channel); '
+                       'final-scale 256 queries'}
+    n_el = B3 * H3 * L3 * D3
+    for name, bits, asym in (('int2_asym', 2, True), ('int8_sym', 8, False)):
+        kw, ks, kz = ops.quant_pack(k, (0, 2), bits, asym)
+        vw, vs, vz = ops.quant_pack(v, (0, 2), bits, asym)
+        t_q = timed(lambda: ops.quant_pack(k, (0, 2), bits, asym))
+        t_d = timed(lambda: ops.dequant(kw, ks, kz, D3, bits, torch.bfloat16))
+        tab = lambda t: None if t is None else t.reshape(H3, D3).contiguous()
+        o = torch.empty_like(q)
+        t_a = timed(lambda: ops.fused_attn_channel(q, kw, tab(ks), tab(kz), vw, tab(vs), tab(vz), bits, L3,
+                                                   1.0 / math.sqrt(D3), out=o))
+        packed = n_el * bits // 8
+        out[name] = {'quant_pack_us': round(t_q * 1e6, 1), 'quant_pack_GBps': round((n_el * 2 + packed) / t_q / 1e9, 1),
+                     'unpack_dequant_us': round(t_d * 1e6, 1), 'unpack_dequant_GBps': round((packed + n_el * 2) / t_d / 1e9, 1),
+                     'fused_attn_us': round(t_a * 1e6, 1),
+                     'fused_attn_TFLOPs': round(4 * B3 * H3 * LQ3 * L3 * D3 / t_a / 1e12, 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -108,6 +150,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
     ap.add_argument('--no-c5', action='store_true', help='skip the config-5 latency leg (profiling runs)')
+    ap.add_argument('--no-c3', action='store_true', help='skip the config-3 rates leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -238,6 +281,7 @@ def main():
                           'traffic': None if not traffic else traffic.get('quant_pack_rows')},
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
+        'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
     }
     print(json.dumps(line), flush=True)
 

@@ -147,6 +147,32 @@ int varq_fused_attn(const void *q, void *out,
                     const int32_t *kv_limit, float softmax_scale, void *stream);
 
 /*
+ * The same attention over a cache quantized per (head, channel), the layout of the
+ * reference's G_SCALE_HEAD_DIM and G_HEAD_DIM methods (scale of shape [1,H,1,c],
+ * VAR_Q/quant.py:84-88,112-116; G_SCALE_HEAD_DIM is the method of the shipped JSON rules)
+ * and of their affine per-head-per-dim extension:
+ *   K[b,h,j,d] = k_chan_scale[h,d] * (k_codes[b,h,j,d] - k_chan_zp[h,d]),  V likewise.
+ * A scalar scale (G_TENSOR, G_SCALE) is the table filled with it.
+ * A cache that the reference's append methods filled step by step
+ * (VAR_Q/quant.py:196-201: every step is quantized with its own scale, expanded over the
+ * step's tokens and concatenated) has one table per step: keys
+ * [host_seg_end[s-1], host_seg_end[s]) use table s, the last segment ends at Lk.
+ *   k_chan_scale, k_chan_zp, v_chan_scale, v_chan_zp
+ *                        fp32 [nseg, Hkv, D]; zero-points NULL = symmetric.  With one
+ *                        segment k_chan_zp may be NULL for an affine K as well: it shifts
+ *                        every logit of a query by the same amount, which the softmax cancels
+ *   nseg, host_seg_end   1..16 segments; host int32 [nseg] (may be NULL when nseg == 1)
+ *   everything else as in varq_fused_attn; one bit-width for K and V.
+ */
+int varq_fused_attn_channel(const void *q, void *out,
+                            const int32_t *k_words, const float *k_chan_scale, const float *k_chan_zp,
+                            const int32_t *v_words, const float *v_chan_scale, const float *v_chan_zp,
+                            int nseg, const int32_t *host_seg_end,
+                            int bits, int B, int Hq, int Hkv, const int32_t *head_map,
+                            int Lq, int Lk, int Lk_stride, int D,
+                            const int32_t *kv_limit, float softmax_scale, void *stream);
+
+/*
  * Producer side of the quantized cache in one pass (an extension: the reference does
  * this as separate tensor expressions before calling its quantizer,
  * Infinity/infinity/models/basic.py:316-330 with apply_rotary_emb at :103-123, and

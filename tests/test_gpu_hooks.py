@@ -172,3 +172,57 @@ def test_var_fused_producer_vs_unfused(dev, layout):
         rng = a.abs().max().item()
         assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0)
         assert _cos(a, b) >= 0.9995
+
+
+@pytest.mark.parametrize('method,bits,sym', [('G_SCALE_HEAD_DIM', 8, True), ('G_HEAD_DIM', 8, True), ('G_TENSOR', 8, True),
+                                             ('G_SCALE', 8, True), ('G_TOKEN', 8, True), ('G_TOKEN_HEAD', 4, True),
+                                             ('G_SCALE_HEAD_DIM', 4, False), ('G_HEAD', 8, True)])
+def test_quantizer_backend_vs_dropin(dev, method, bits, sym):
+    """fused='quantizer': the reference's own rules (quantizer + per-step cache as in the
+    drop-in) with the attention reading the packed caches, A/B against the drop-in that
+    dequantizes the whole cache and calls SDPA.  Both hold the same caches; the outputs
+    differ by the attention arithmetic only."""
+    torch.manual_seed(6)
+    C, H = 512, 8
+    pn = (1, 2, 3, 4, 5, 6, 8, 10, 13, 16)
+    kw = dict(embed_dim=C, num_heads=H, layout='BHLc', q_bits=bits, quant_method=method, symmetric=sym,
+              enable_quantization=True, max_tokens=680)
+    a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.VarSelfAttention(0, fused='quantizer', **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    for p in pn:
+        note('hooks quantizer backend', method, bits, sym, p)
+        x = torch.randn(2, p * p, C, device=dev, dtype=torch.bfloat16)
+        a, b = a_mod(x).float(), b_mod(x).float()
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995
+    assert torch.equal(a_mod.k_quant.dequant_all(), b_mod.k_quant.dequant_all())
+    assert torch.equal(a_mod.v_quant.dequant_all(), b_mod.v_quant.dequant_all())
+
+
+def test_quantizer_backend_infinity_shipped_rule(dev):
+    """The Infinity hook with the shipped rule (G_SCALE_HEAD_DIM, 8 bits, BHLc,
+    Infinity-VAR_Q-8.json) over the first scales of its schedule, head dim 128."""
+    torch.manual_seed(7)
+    C, H = 512, 4
+    pn = (1, 2, 4, 6, 8, 12, 16)
+    kw = dict(embed_dim=C, num_heads=H, layout='BHLc', q_bits=8, quant_method='G_SCALE_HEAD_DIM',
+              enable_quantization=True, max_tokens=sum(p * p for p in pn))
+    a_mod = hooks.InfinitySelfAttention(fused=False, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.InfinitySelfAttention(fused='quantizer', **kw).to(dev).to(torch.bfloat16)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    rope = hooks.rope2d_tables(C // H, [(p, p) for p in pn])
+    start = 0
+    for p in pn:
+        note('hooks quantizer backend infinity', p)
+        x = torch.randn(2, p * p, C, device=dev, dtype=torch.bfloat16)
+        a, b = a_mod(x, rope=rope, token_start=start).float(), b_mod(x, rope=rope, token_start=start).float()
+        start += p * p
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995

@@ -84,3 +84,59 @@ def test_per_head_extension_single_call(dev):
     s = O.scale_sym(x, (0, 2, 3), 8)
     assert torch.equal(got.cpu(), O.dequant_sym(O.codes_sym(x, s, 8), s))
     assert gpu.scale.shape == (1, 16, 1, 1)
+
+
+@pytest.mark.parametrize('method', list(O.METHODS))
+@pytest.mark.parametrize('bits', [4, 8])
+def test_fused_attention_over_quantizer_caches(dev, method, bits):
+    """`fused_attention` over the packed caches of two drop-in quantizers, all six methods of
+    the reference, four steps, against the oracle class's dequant_all -> bf16 SDPA on the CPU
+    (the path the reference runs: VAR_Q/quant.py:216-230 into the attention backend).
+    Tolerance: cosine >= 0.9995, max-abs 2e-2 in units of the output range."""
+    from var_q_amd.quant import fused_attention
+    note('fused_attention', method, bits)
+    ks, vs = _steps('BHLc', torch.bfloat16, seed=20 + bits), _steps('BHLc', torch.bfloat16, seed=30 + bits)
+    rk, rv = O.OracleVARQ(bits, 'BHLc', method, pack_to_int32=False), O.OracleVARQ(bits, 'BHLc', method, pack_to_int32=False)
+    gk, gv = VAR_Q(bits, 'BHLc', method), VAR_Q(bits, 'BHLc', method)
+    g = torch.Generator().manual_seed(5)
+    for k, v in zip(ks, vs):
+        kd, vd = rk.use_var_q(k), rv.use_var_q(v)
+        for qz, item in ((gk, k), (gv, v)):
+            qz.quant(item.to(dev))
+            qz.cache()
+        q = torch.randn(k.shape[0], k.shape[1], k.shape[2], k.shape[3], generator=g).bfloat16()
+        out = fused_attention(q.to(dev), gk, gv, 0.125).float().cpu()
+        ref = O.attention_ref(q, kd, vd, 0.125).float()
+        span = max(1.0, float(ref.abs().max()))
+        err = float((out - ref).abs().max())
+        cos = float(torch.nn.functional.cosine_similarity(out.flatten().double(), ref.flatten().double(), dim=0))
+        assert cos >= 0.9995 and err <= 2e-2 * span, (method, bits, k.shape[2], err, span, cos)
+
+
+def test_fused_attention_refuses_what_it_cannot_serve(dev):
+    from var_q_amd.quant import fused_attention
+    x = torch.randn(1, 2, 4, 64, device=dev)
+    q = torch.randn(1, 2, 4, 64, device=dev)
+    a, b = VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM'), VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM')
+    with pytest.raises(ValueError, match='packed cache'):
+        fused_attention(q, a, b, 1.0)                       # nothing cached yet
+    for qz in (a, b):
+        qz.use_var_q(x)
+    fused_attention(q, a, b, 1.0)
+    with pytest.raises(ValueError, match='BHLc'):
+        c = VAR_Q(8, 'BLHc', 'G_SCALE_HEAD_DIM')
+        c.use_var_q(x.transpose(1, 2).contiguous())
+        fused_attention(q, c, c, 1.0)
+    with pytest.raises(ValueError, match='bit-width'):
+        d = VAR_Q(4, 'BHLc', 'G_SCALE_HEAD_DIM')
+        d.use_var_q(x)
+        fused_attention(q, a, d, 1.0)
+    with pytest.raises(ValueError, match='cannot be combined'):
+        e = VAR_Q(8, 'BHLc', 'G_TOKEN')
+        e.use_var_q(x)
+        fused_attention(q, a, e, 1.0)
+    with pytest.raises(ValueError, match='steps'):
+        for _ in range(16):                                   # 17 cached steps
+            for qz in (a, b):
+                qz.use_var_q(x)
+        fused_attention(q, a, b, 1.0)

@@ -27,6 +27,13 @@ SYMBOLS = {
                                 c_int, c_int, c_int, c_void_p,
                                 c_int, c_int, c_int, c_int,
                                 c_void_p, c_float, c_void_p]),
+    'varq_fused_attn_channel': (c_int, [c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p,
+                                        c_int, POINTER(c_int32),
+                                        c_int, c_int, c_int, c_int, c_void_p,
+                                        c_int, c_int, c_int, c_int,
+                                        c_void_p, c_float, c_void_p]),
     'varq_qkv_prepare_append': (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_int, c_float,
                                         c_void_p, c_void_p, c_int,

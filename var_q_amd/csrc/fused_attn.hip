@@ -58,11 +58,20 @@ constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
 
+constexpr int kMaxSegments = 16;
+
 struct AttnParams {
   const __bf16 *q;
   __bf16 *out;
   const u32 *k_words, *v_words;
   const float *k_scale, *k_zp, *v_scale, *v_zp;
+  // per-(head, channel) quantization (CHAN kernels): fp32 [Hkv, D] tables shared by all
+  // tokens and batch entries; the per-key pointers above are unused then
+  const float *k_chan_scale, *k_chan_zp, *v_chan_scale, *v_chan_zp;
+  // the tables may change along the keys: keys [seg_end[s-1], seg_end[s]) use table s
+  // (fp32 [nseg, Hkv, D]); this is a cache that was quantized step by step
+  int nseg;
+  int seg_end[kMaxSegments];
   const int32_t *head_map;
   const int32_t *kv_limit;
   int B, Hq, Hkv, Lq, Lk, Lstride;
@@ -239,8 +248,20 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
   static constexpr int kBytes = kFlag + 16;
 };
 
-template <int D, int BITS, int GK, int GV>
+// CHAN: scales and zero-points per (head, channel) instead of per (key, channel group).
+// Then K[l,d] = sk[d] * (code[l,d] - zk[d]) and q.K[l] = sum_d (q[d] sk[d]) code[l,d] minus
+// a term that does not depend on the key, which the softmax cancels: the kernel attends
+// the raw codes with q scaled per channel.  With one table that term can be left out; when
+// the tables change along the keys it differs from segment to segment and is added to the
+// logits as a per-query constant of the segment.
+// Likewise out[d] = sv[d] * (sum_l p[l] code[l,d] - zv[d]) because the weights sum to one:
+// V runs with unit scale and the affine map is applied to the normalized output.
+// When the tables change along the keys (segments), key tiles never straddle a segment:
+// at a boundary the Q operands are rebuilt with the new K table and the output
+// accumulators are re-expressed in units of the new V table.
+template <int D, int BITS, int GK, int GV, bool CHAN>
 __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
+  static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NSK = D / GK, NSV = D / GV;
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
@@ -297,23 +318,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 
   // Q^T operands, gathered in the slot order of the K codec
   u32x4_t qb[NCH];
-  float qsum[NSK];
-#pragma unroll
-  for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
-#pragma unroll
-  for (int ch = 0; ch < NCH; ++ch) {
-    const int oct = k_octet<GK>(ch, half);
-    uint16_t e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      e[j] = reinterpret_cast<const uint16_t *>(qptr)[oct * 8 + KCodec<BITS>::slot_d(j)];
-      qsum[ch / (GK / 16)] += u2f((u32)e[j] << 16);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) qb[ch][j] = (u32)e[2 * j] | ((u32)e[2 * j + 1] << 16);
-  }
-#pragma unroll
-  for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
+  u32x4_t bq[NSK];
   // The K zero-point term -(kzp+kOff)/kMul * sum(q) is a rank-1 update of S^T and
   // rides on one more MFMA per key block and group.  Both factors are split into
   // three bf16 pieces (a0+a1+a2, b0+b1+b2, exact) and the 9 products are laid on
@@ -322,15 +327,44 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // the term, is dropped).  With a single V group, slots 0..2 of the upper half add
   // log2(vs)/ck (three pieces against 1.0), which makes exp2(logit) come out as
   // p * vs without a multiplication; the other upper slots are zero.
-  u32x4_t bq[NSK];
+  float qbias = 0.f;   // CHAN: -softmax_scale*log2(e) * sum_d q'[d] zk[d] of the current segment
+  auto load_q = [&](int seg) {
+    float qsum[NSK], zb = 0.f;
 #pragma unroll
-  for (int s = 0; s < NSK; ++s) {
-    u32 b0, b1, b2;
-    split3_bf16(qsum[s], b0, b1, b2);
-    if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
-    else if (FOLD_SV && s == 0) bq[s] = u32x4_t{0x3f803f80u, 0x00003f80u, 0u, 0u};
-    else bq[s] = u32x4_t{0u, 0u, 0u, 0u};
-  }
+    for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+      const int oct = k_octet<GK>(ch, half);
+      uint16_t e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int d = oct * 8 + KCodec<BITS>::slot_d(j);
+        e[j] = reinterpret_cast<const uint16_t *>(qptr)[d];
+        if constexpr (CHAN) {
+          // q[d] * sk[d], rounded to bf16 like any MFMA operand
+          const int64_t ti = ((int64_t)seg * p.Hkv + hs) * D + d;
+          const float qs = u2f((u32)e[j] << 16) * p.k_chan_scale[ti];
+          e[j] = (uint16_t)(pack_bf16_rne(qs, 0.f) & 0xffffu);
+          if (p.k_chan_zp) zb = __builtin_fmaf(u2f((u32)e[j] << 16), p.k_chan_zp[ti], zb);
+        }
+        qsum[ch / (GK / 16)] += u2f((u32)e[j] << 16);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qb[ch][j] = (u32)e[2 * j] | ((u32)e[2 * j + 1] << 16);
+    }
+#pragma unroll
+    for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
+    if constexpr (CHAN) qbias = -p.scale_log2e * (zb + __shfl_xor(zb, 32, 64));
+#pragma unroll
+    for (int s = 0; s < NSK; ++s) {
+      u32 b0, b1, b2;
+      split3_bf16(qsum[s], b0, b1, b2);
+      if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
+      else if (FOLD_SV && s == 0) bq[s] = u32x4_t{0x3f803f80u, 0x00003f80u, 0u, 0u};
+      else bq[s] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  };
+  load_q(0);
 
   // ---- tile range: every lane of the workgroup runs the same number of tiles ----
   __shared__ int lds_maxlim;
@@ -339,7 +373,26 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   atomicMax(&lds_maxlim, q_live ? limit : 0);
   __syncthreads();
   const int kv_end = lds_maxlim;
-  const int n_tiles = (kv_end + BN - 1) / BN;
+  int n_tiles = (kv_end + BN - 1) / BN;
+  if constexpr (CHAN) {
+    // key tiles never straddle a segment of the tables: count them segment by segment
+    n_tiles = 0;
+    for (int s = 0, beg = 0; s < p.nseg && beg < kv_end; beg = p.seg_end[s], ++s)
+      n_tiles += (min(p.seg_end[s], kv_end) - beg + BN - 1) / BN;
+  }
+  // Position of a stream of consecutive tiles (the K prefetch, the V prefetch and the
+  // attention itself each walk the tiles in order).  Without segments tile t starts at
+  // key t * BN; with segments a tile ends where its segment ends.
+  struct TileCursor { int seg, start; };
+  auto cursor_advance = [&](TileCursor &c) {
+    if constexpr (CHAN) {
+      c.start += BN;
+      if (c.start >= p.seg_end[c.seg] && c.seg + 1 < p.nseg) { c.start = p.seg_end[c.seg]; ++c.seg; }
+    } else {
+      c.start += BN;
+    }
+  };
+  TileCursor cur_k{0, 0}, cur_v{0, 0}, cur_a{0, 0};
   int wave_minlim = q_live ? limit : p.Lk;
   for (int off = 1; off < 64; off <<= 1) wave_minlim = min(wave_minlim, __shfl_xor(wave_minlim, off, 64));
 
@@ -367,8 +420,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   u32x4_t kreg[LPT], vreg[LPT];
   float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
 
-  auto prefetch_k = [&](int tile) {
-    const int t0 = tile * BN;
+  auto prefetch_k = [&](int) {   // the next tile of the K stream
+    const int t0 = cur_k.start;
+    cursor_advance(cur_k);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
@@ -378,8 +432,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       }
     }
   };
-  auto prefetch = [&](int tile) {
-    const int t0 = tile * BN;
+  auto prefetch = [&](int) {   // the next tile of the V stream
+    const int t0 = cur_v.start;
+    cursor_advance(cur_v);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
@@ -391,7 +446,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     // scales: thread t handles key t % 64; wavefront w takes K group w and V group
     // 3 - w, which puts the K and the V arithmetic of the single-group case on
     // different wavefronts
-    {
+    if constexpr (CHAN) {
+      ksc = 1.f; kzp = 0.f; vsc = 1.f; vzp = 0.f; ksc0 = 1.f;   // unit per-key parameters
+    } else {
       const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = NW - 1 - seg;
       if (seg < NSK) {
         const int64_t g = (kv_row0 + key) * NSK + seg;
@@ -548,8 +605,53 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   float ckv[2][NSK][16], svv[2][NSV][16];
   u32x4_t vta[NDB], wza[NSV];
 
+  // per-channel tables: segment of the tile being attended, end of the tile's keys, and the
+  // softmax denominator as it was when the current segment began
+  int seg_a = 0, tile_end = 0;
+  float l_prev = 0.f;
+  // A new segment begins.  The true (unnormalized) output is, per channel,
+  //   sv * (kMul * oacc - rq - zv * (l_sum - l_prev))
+  // with rq, l_sum the readings of the extra block; the accumulators are re-expressed so that
+  // the same formula holds with the new tables and l_prev = l_sum, and the Q operands are
+  // rebuilt with the new K table.
+  auto segment_boundary = [&](int seg_new) {
+    if constexpr (CHAN) {
+      const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
+      const float rq = __shfl(racc[0], col, 64) + r_run[0];
+      const float dl = l_sum - l_prev;
+      constexpr float VM = VCodec<BITS>::kMul;
+      const float *sv_old = p.v_chan_scale + ((int64_t)seg_a * p.Hkv + hs) * D;
+      const float *sv_new = p.v_chan_scale + ((int64_t)seg_new * p.Hkv + hs) * D;
+      const float *zv_old = p.v_chan_zp ? p.v_chan_zp + ((int64_t)seg_a * p.Hkv + hs) * D : nullptr;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int c0 = d * 32 + 8 * g4 + 4 * half;
+          const float4 so = *reinterpret_cast<const float4 *>(sv_old + c0), sn = *reinterpret_cast<const float4 *>(sv_new + c0);
+          float4 zo = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (zv_old) zo = *reinterpret_cast<const float4 *>(zv_old + c0);
+          const float ro[4] = {so.x / sn.x, so.y / sn.y, so.z / sn.z, so.w / sn.w};
+          const float zz[4] = {zo.x, zo.y, zo.z, zo.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            oacc[d][4 * g4 + j] = (ro[j] * (VM * oacc[d][4 * g4 + j] - rq - zz[j] * dl) + rq) * (1.f / VM);
+        }
+      l_prev = l_sum;
+      seg_a = seg_new;
+      load_q(seg_new);
+    }
+  };
+
   auto begin_tile = [&](int tile) {
-    t0 = tile * BN;
+    if constexpr (CHAN) {
+      t0 = cur_a.start;
+      tile_end = min(t0 + BN, p.seg_end[cur_a.seg]);
+      if (cur_a.seg != seg_a) segment_boundary(cur_a.seg);
+      cursor_advance(cur_a);
+    } else {
+      t0 = tile * BN;
+    }
     kx = lds_kx + (tile & 1) * BN * KXS;
     par = lds_par + (tile % 3) * L::kParFloats;
     vt = lds_vt + (tile & 1) * D * VTS;
@@ -623,7 +725,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     float z[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      float v = -m_ref;
+      float v = CHAN ? qbias - m_ref : -m_ref;
 #pragma unroll
       for (int s = 0; s < NSK; ++s) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
@@ -631,12 +733,14 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       }
       z[i] = v;
     }
-    // mask: block-causal key limit, and the ragged last tile
-    if (t0 + BN > wave_minlim) {
+    // mask: block-causal key limit, the ragged last tile, and (per-channel tables) the
+    // keys of the next segment behind a short tile
+    const int lim_t = CHAN ? min(limit, tile_end) : limit;
+    if (t0 + BN > (CHAN ? min(wave_minlim, tile_end) : wave_minlim)) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = t0 + kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        if (key >= limit) z[i] = -INFINITY;
+        if (key >= lim_t) z[i] = -INFINITY;
       }
     }
     float zmax = z[0];
@@ -664,6 +768,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       for (int j = 0; j < 16; ++j) racc[j] *= alpha;
 #pragma unroll
       for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
+      if constexpr (CHAN) l_prev *= alpha;
     }
     first = false;
     float pv[16];
@@ -768,8 +873,19 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
-        const float o0 = (VM * oacc[d][4 * g4 + 0] - r) * inv, o1 = (VM * oacc[d][4 * g4 + 1] - r) * inv;
-        const float o2 = (VM * oacc[d][4 * g4 + 2] - r) * inv, o3 = (VM * oacc[d][4 * g4 + 3] - r) * inv;
+        float o0 = (VM * oacc[d][4 * g4 + 0] - r) * inv, o1 = (VM * oacc[d][4 * g4 + 1] - r) * inv;
+        float o2 = (VM * oacc[d][4 * g4 + 2] - r) * inv, o3 = (VM * oacc[d][4 * g4 + 3] - r) * inv;
+        if constexpr (CHAN) {
+          // weighted mean of the codes -> values: sv * (mean - zv * share) per channel, share
+          // = the part of the weights that belongs to the current segment (1 without segments)
+          const int64_t c0 = ((int64_t)seg_a * p.Hkv + hs) * D + d * 32 + 8 * g4 + 4 * half;
+          const float4 sv = *reinterpret_cast<const float4 *>(p.v_chan_scale + c0);
+          float4 zv = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (p.v_chan_zp) zv = *reinterpret_cast<const float4 *>(p.v_chan_zp + c0);
+          const float share = (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
+          o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
+          o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
+        }
         uint2 v = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
         *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = v;
       }
@@ -777,18 +893,18 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   }
 }
 
-template <int D, int BITS, int GK, int GV>
+template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
   constexpr int lds_bytes = AttnLds<D, BITS, GK, GV>::kBytes;
   static bool configured = false;   // above 64 KiB the limit has to be raised once per process
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     configured = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV>), grid, dim3(NT), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN>), grid, dim3(NT), lds_bytes, st, p);
 }
 
 template <int D, int BITS>
@@ -834,6 +950,9 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.k_words = reinterpret_cast<const u32 *>(k_words);
   p.v_words = reinterpret_cast<const u32 *>(v_words);
   p.k_scale = k_scale; p.k_zp = k_zp; p.v_scale = v_scale; p.v_zp = v_zp;
+  p.k_chan_scale = nullptr; p.k_chan_zp = nullptr; p.v_chan_scale = nullptr; p.v_chan_zp = nullptr;
+  p.nseg = 1;
+  for (int s = 0; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
   p.head_map = head_map; p.kv_limit = kv_limit;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
   p.q_tiles = (Lq + BM - 1) / BM;
@@ -854,5 +973,65 @@ extern "C" int varq_fused_attn(const void *q, void *out,
     return varq_set_error(VARQ_ERR_UNSUPPORTED, "fused_attn: no kernel for D=%d bits=%d k_group=%d v_group=%d", D, k_bits,
                           k_group, v_group);
   VARQ_CHECK_LAUNCH("fused_attn");
+  return VARQ_OK;
+}
+
+extern "C" int varq_fused_attn_channel(const void *q, void *out,
+                                       const int32_t *k_words, const float *k_chan_scale, const float *k_chan_zp,
+                                       const int32_t *v_words, const float *v_chan_scale, const float *v_chan_zp,
+                                       int nseg, const int32_t *host_seg_end,
+                                       int bits, int B, int Hq, int Hkv, const int32_t *head_map,
+                                       int Lq, int Lk, int Lk_stride, int D,
+                                       const int32_t *kv_limit, float softmax_scale, void *stream) {
+  VARQ_CHECK_ARG(q && out && k_words && v_words && k_chan_scale && v_chan_scale, "fused_attn_channel: null pointer");
+  VARQ_CHECK_ARG(nseg >= 1 && nseg <= kMaxSegments, "fused_attn_channel: nseg must be 1..%d (got %d)", kMaxSegments, nseg);
+  VARQ_CHECK_ARG(nseg == 1 || host_seg_end, "fused_attn_channel: segment ends missing");
+  VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn_channel: bad sizes");
+  VARQ_CHECK_ARG(head_map || Hkv == Hq, "fused_attn_channel: Hkv != Hq needs a head map");
+  VARQ_CHECK_ARG(D == 64 || D == 128, "fused_attn_channel: D must be 64 or 128 (got %d)", D);
+  VARQ_CHECK_ARG(bits == 2 || bits == 4 || bits == 8, "fused_attn_channel: bits must be 2, 4 or 8 (got %d)", bits);
+  if (Lq == 0 || Lk == 0) {
+    if (Lq > 0) return varq_set_error(VARQ_ERR_INVALID, "fused_attn_channel: no keys to attend");
+    return VARQ_OK;
+  }
+  VARQ_CHECK_ARG((int64_t)B * Hkv * Lk_stride * D < (1ll << 40), "fused_attn_channel: cache too large");
+  VARQ_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
+                 "fused_attn_channel: q must be 16-byte and out 8-byte aligned");
+  VARQ_CHECK_ARG(((uintptr_t)v_chan_scale & 15) == 0 && ((uintptr_t)v_chan_zp & 15) == 0,
+                 "fused_attn_channel: the V tables must be 16-byte aligned");
+
+  AttnParams p;
+  p.q = reinterpret_cast<const __bf16 *>(q);
+  p.out = reinterpret_cast<__bf16 *>(out);
+  p.k_words = reinterpret_cast<const u32 *>(k_words);
+  p.v_words = reinterpret_cast<const u32 *>(v_words);
+  p.k_scale = nullptr; p.k_zp = nullptr; p.v_scale = nullptr; p.v_zp = nullptr;
+  p.k_chan_scale = k_chan_scale; p.k_chan_zp = k_chan_zp; p.v_chan_scale = v_chan_scale; p.v_chan_zp = v_chan_zp;
+  p.nseg = nseg;
+  for (int s = 0, prev = 0; s < nseg; ++s) {
+    // the last segment runs to the end of the keys whatever the caller's table says
+    const int e = (s == nseg - 1 || !host_seg_end) ? Lk : host_seg_end[s];
+    VARQ_CHECK_ARG(e > prev || (s == nseg - 1 && e >= prev), "fused_attn_channel: segment ends must increase");
+    VARQ_CHECK_ARG(e <= Lk, "fused_attn_channel: segment end %d beyond Lk=%d", e, Lk);
+    p.seg_end[s] = e;
+    prev = e;
+  }
+  for (int s = nseg; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
+  p.head_map = head_map; p.kv_limit = kv_limit;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
+  p.q_tiles = (Lq + BM - 1) / BM;
+  p.bh_total = B * Hkv;
+  p.scale_log2e = softmax_scale * kLog2e;
+  hipStream_t st = (hipStream_t)stream;
+  if (D == 128) {
+    if (bits == 4) launch<128, 4, 128, 128, true>(p, st);
+    else if (bits == 8) launch<128, 8, 128, 128, true>(p, st);
+    else launch<128, 2, 128, 128, true>(p, st);
+  } else {
+    if (bits == 4) launch<64, 4, 64, 64, true>(p, st);
+    else if (bits == 8) launch<64, 8, 64, 64, true>(p, st);
+    else launch<64, 2, 64, 64, true>(p, st);
+  }
+  VARQ_CHECK_LAUNCH("fused_attn_channel");
   return VARQ_OK;
 }

@@ -10,7 +10,7 @@ reference quantizer,
 i.e. `kv_caching(True)` creates one K and one V quantizer, `forward` projects
 x to q/k/v, normalises (and rotates) q and k, pushes k and v through the
 quantized cache and attends with the current scale's queries over everything
-cached.  Two backends behind the same interface:
+cached.  Three backends behind the same interface:
 
   * `fused=False`: the drop-in `VAR_Q.use_var_q` (dequantized full-length K/V
     out) followed by scaled-dot-product attention, which is what the reference
@@ -20,7 +20,11 @@ cached.  Two backends behind the same interface:
     packed codes; no dequantized K/V exists.  Needs a row-local quantizer
     (`quant_method='G_GROUP'`).  With `fused_producer=True` the normalisation,
     the per-head scale of q, the rotation and the quantization of k and v run as
-    one kernel on the qkv projection output (`PackedKVCache.append_from_qkv`).
+    one kernel on the qkv projection output (`PackedKVCache.append_from_qkv`);
+  * `fused='quantizer'`: the drop-in quantizers of any rule of the JSON files (the shipped
+    G_SCALE_HEAD_DIM rule included) do `quant` + `cache` as in the first backend, and
+    `var_q_amd.quant.fused_attention` attends over their packed caches, so the
+    dequantized full-length K/V of `dequant_all` is never built.  Layout BHLc.
 
 The transformer blocks around the attention (AdaLN, FFN, cross-attention) are
 outside this package.
@@ -33,7 +37,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .kv_cache import PackedKVCache
-from .quant import VAR_Q
+from .quant import VAR_Q, fused_attention
 
 
 def rope2d_tables(head_dim: int, scale_hw: Sequence[Tuple[int, int]], normalized_by_hw: int = 2,
@@ -93,11 +97,14 @@ class _QuantizedSelfAttention(nn.Module):
         self.q_bits, self.quant_method, self.enable_quantization = q_bits, quant_method, enable_quantization
         self.fused, self.group_size, self.symmetric, self.max_tokens = fused, group_size, symmetric, max_tokens
         self.fused_producer = fused_producer
-        assert fused or not fused_producer, 'fused_producer needs the fused backend'
+        assert fused is True or not fused_producer, 'fused_producer needs the packed-cache backend (fused=True)'
         self._quantizer_factory = quantizer_factory or VAR_Q
-        if fused:
+        assert fused in (False, True, 'quantizer'), "fused: False, True or 'quantizer'"
+        if fused is True:
             assert enable_quantization and quant_method == 'G_GROUP' and group_size, \
                 'the fused backend needs the row-local group-wise quantizer (quant_method="G_GROUP", group_size=g)'
+        if fused == 'quantizer':
+            assert enable_quantization and layout == 'BHLc', "fused='quantizer' needs quantization and layout BHLc"
         self.mat_qkv = nn.Linear(embed_dim, embed_dim * 3, bias=False)
         self.q_bias, self.v_bias = nn.Parameter(torch.zeros(embed_dim)), nn.Parameter(torch.zeros(embed_dim))
         self.register_buffer('zero_k_bias', torch.zeros(embed_dim))
@@ -111,7 +118,7 @@ class _QuantizedSelfAttention(nn.Module):
         self.caching, self.cached_k, self.cached_v = enable, None, None
         self.k_quant = self.v_quant = None
         self.packed_cache = None
-        if enable and self.enable_quantization and not self.fused:
+        if enable and self.enable_quantization and self.fused is not True:
             kw = dict(quant_bits=self.q_bits, qkv_format=self.layout, quant_method=self.quant_method, blk_idx=self.block_idx)
             if self.quant_method == 'G_GROUP' or not self.symmetric:
                 kw.update(group_size=self.group_size, symmetric=self.symmetric)
@@ -158,6 +165,14 @@ class _QuantizedSelfAttention(nn.Module):
         B = q.shape[0]
         l_dim = 1 if self.layout == 'BLHc' else 2
         L = q.shape[l_dim]
+        if self.caching and self.fused == 'quantizer':
+            if attn_bias is not None:
+                raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')
+            for quantizer, item in ((self.k_quant, k), (self.v_quant, v)):
+                quantizer.quant(item)
+                quantizer.cache()
+            o = fused_attention(q, self.k_quant, self.v_quant, scale)                     # [B,H,L,c]
+            return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
         if self.caching and self.fused:
             if attn_bias is not None:
                 raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')

@@ -8,6 +8,8 @@ from __future__ import annotations
 
 from typing import Optional, Sequence, Tuple
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -273,4 +275,59 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
                                   v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), v_bits, v_group,
                                   B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
                                   _ptr(kv_limit), float(softmax_scale), _stream(q)), 'varq_fused_attn')
+    return out
+
+
+def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: torch.Tensor,
+                       k_chan_zp: Optional[torch.Tensor],
+                       v_words: torch.Tensor, v_chan_scale: torch.Tensor, v_chan_zp: Optional[torch.Tensor],
+                       bits: int, Lk: int, softmax_scale: float,
+                       kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
+                       out: Optional[torch.Tensor] = None, seg_ends: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Attention over a cache quantized per (head, channel): the scale layout of the
+    reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
+    (G_TENSOR, G_SCALE) expanded to the table, and the affine per-head-per-dim variant.
+    q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32; k_chan_scale,
+    v_chan_scale, v_chan_zp fp32 with nseg*Hkv*D elements (any shape that flattens to
+    [nseg, Hkv, D]).  seg_ends (at most 16 increasing key counts, the last one = Lk) says
+    where the tables change along the keys: a cache filled step by step by the reference's
+    append methods has one table per step (VAR_Q/quant.py:196-201).
+    With a single table the zero-point of K may be None even for an affine K: it shifts all
+    logits of a query alike."""
+    for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_chan_scale, 'k_chan_scale'),
+                 (v_chan_scale, 'v_chan_scale')):
+        _gpu(t, n)
+        assert t.is_contiguous(), f'{n} must be contiguous'
+    assert q.dtype == torch.bfloat16 and q.dim() == 4
+    B, Hq, Lq, D = q.shape
+    Bk, Hkv, Lstride, W = k_words.shape
+    assert Bk == B and v_words.shape == k_words.shape and W * 32 == D * bits
+    nseg = 1 if seg_ends is None else len(seg_ends)
+    ends = None
+    if seg_ends is not None:
+        assert 1 <= nseg <= 16 and int(seg_ends[-1]) == Lk, 'seg_ends: 1..16 entries, the last one equal to Lk'
+        ends = (ctypes.c_int32 * nseg)(*[int(e) for e in seg_ends])
+    for t, n in ((k_chan_scale, 'k_chan_scale'), (k_chan_zp, 'k_chan_zp'), (v_chan_scale, 'v_chan_scale'),
+                 (v_chan_zp, 'v_chan_zp')):
+        if t is not None:
+            _gpu(t, n)
+            assert t.dtype == torch.float32 and t.numel() == nseg * Hkv * D and t.is_contiguous(), \
+                f'{n} must be fp32 [nseg, Hkv, D]'
+    if out is None:
+        out = torch.empty_like(q)
+    if kv_limit is not None:
+        _gpu(kv_limit, 'kv_limit')
+        assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
+    if head_map is not None:
+        _gpu(head_map, 'head_map')
+        assert head_map.dtype == torch.int32 and head_map.numel() == Hkv
+    else:
+        assert Hkv == Hq
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        check(lib.varq_fused_attn_channel(q.data_ptr(), out.data_ptr(),
+                                          k_words.data_ptr(), k_chan_scale.data_ptr(), _ptr(k_chan_zp),
+                                          v_words.data_ptr(), v_chan_scale.data_ptr(), _ptr(v_chan_zp),
+                                          nseg, ends, bits, B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
+                                          _ptr(kv_limit), float(softmax_scale), _stream(q)), 'varq_fused_attn_channel')
     return out

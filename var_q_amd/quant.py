@@ -23,10 +23,12 @@ Behaviour kept on purpose, because callers can observe it:
 Extensions (absent from the reference): `symmetric=False` selects the min/max
 affine quantizer (attributes `zp`, `cached_zp`); quant_method 'G_GROUP' with
 `group_size=g` quantizes g contiguous channels of each token independently
-(batch and tokens not reduced); 'G_HEAD' keeps one scale per head.
+(batch and tokens not reduced); 'G_HEAD' keeps one scale per head;
+`fused_attention(q, k_quant, v_quant, scale)` attends over two packed caches
+without dequantizing them.
 GPU tensors only.
 """
-from typing import Dict, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -115,6 +117,8 @@ class VAR_Q:
 
     # ---------------- cache views ----------------
     def _reset_cache(self):
+        # (tokens, scale, zp) of every cached step, for the fused attention
+        self._segments: List[Tuple[int, torch.Tensor, Optional[torch.Tensor]]] = []
         self._c_item = _Growable(self.dim_cat)
         self._c_scale = _Growable(self.dim_cat)
         self._c_zp = _Growable(self.dim_cat)
@@ -184,11 +188,13 @@ class VAR_Q:
             self._c_scale.append(s_cur)
             if z_cur is not None:
                 self._c_zp.append(z_cur)
+            self._segments.append((q_cur.size(self.dim_cat), self.scale, self.zp))
         elif m == 'G_HEAD_DIM':
             self._c_item.replace(q_cur)
             self._c_scale.replace(s_cur)
             if z_cur is not None:
                 self._c_zp.replace(z_cur)
+            self._segments = [(q_cur.size(self.dim_cat), self.scale, self.zp)]
         else:
             raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
 
@@ -232,3 +238,73 @@ def _dequant_views(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tens
     for d in range(3):
         assert scale.shape[d] in (1, q.shape[d]), f'scale dim {d}: {scale.shape[d]} vs {q.shape[d]}'
     return ops.dequant_window(q, scale, zp, (n0, n1, n2, c), strides, group, bits, rowmap, out_dtype)
+
+
+# methods whose scale does not depend on the token: one table per cached step
+_TABLE_METHODS = ('G_SCALE_HEAD_DIM', 'G_HEAD_DIM', 'G_TENSOR', 'G_SCALE', 'G_HEAD')
+# methods with one scale (per channel group) per token
+_TOKEN_METHODS = ('G_TOKEN', 'G_TOKEN_HEAD', 'G_GROUP')
+MAX_TABLE_STEPS = 16
+
+
+def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_scale: float,
+                    kv_limit: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(scale * q K^T) V over the packed caches of two quantizers, without the
+    dequantized full-length K/V that `dequant_all` would produce (the reference computes
+    exactly that and hands it to its attention backend: VAR_Q/quant.py:216-230,
+    Infinity/infinity/models/basic.py:339-351).
+
+    q [B,H,Lq,c] (cast to bf16); both quantizers in layout 'BHLc', packed, same bit-width,
+    c in {64, 128}, after at least one `cache()`.  Methods whose scale is shared by the
+    tokens of a step (G_SCALE_HEAD_DIM -- the shipped rule --, G_HEAD_DIM, G_TENSOR, G_SCALE,
+    G_HEAD) go through one table per cached step, at most MAX_TABLE_STEPS steps; per-token
+    methods (G_TOKEN, G_TOKEN_HEAD, G_GROUP) through per-token scales.  kv_limit: int32
+    [Lq], query i sees keys j < kv_limit[i].  Returns bf16 [B,H,Lq,c]."""
+    for qz, n in ((k_quant, 'k_quant'), (v_quant, 'v_quant')):
+        if qz.qkv_format != 'BHLc':
+            raise ValueError(f'fused_attention: {n} must use layout BHLc')
+        if not qz.pack_to_int32 or qz.cached_item is None:
+            raise ValueError(f'fused_attention: {n} needs a packed cache (pack_to_int32=True, after cache())')
+    bits = k_quant.quant_bits
+    if v_quant.quant_bits != bits:
+        raise ValueError('fused_attention: K and V must use the same bit-width')
+    kbuf, vbuf = k_quant._c_item.buf, v_quant._c_item.buf
+    Lk = k_quant._c_item.len
+    if v_quant._c_item.len != Lk or kbuf.shape != vbuf.shape:
+        raise ValueError('fused_attention: the K and V caches differ in length or capacity')
+    B, H, cap, _ = kbuf.shape
+    c = k_quant._pack_meta['orig_c']
+    if c not in (64, 128):
+        raise ValueError(f'fused_attention: head dim {c} not supported (64 or 128)')
+    q = q.to(torch.bfloat16).contiguous()
+    assert q.dim() == 4 and q.shape[0] == B and q.shape[1] == H and q.shape[3] == c, 'q must be [B,H,Lq,c]'
+    km, vm = k_quant.quant_method, v_quant.quant_method
+    if km in _TABLE_METHODS and vm in _TABLE_METHODS:
+        ends, acc = [], 0
+        for (n, _, _), (nv, _, _) in zip(k_quant._segments, v_quant._segments):
+            if n != nv:
+                raise ValueError('fused_attention: K and V were cached in different steps')
+            acc += n
+            ends.append(acc)
+        if len(ends) > MAX_TABLE_STEPS or len(v_quant._segments) != len(ends) or acc != Lk:
+            raise ValueError(f'fused_attention: at most {MAX_TABLE_STEPS} cached steps, the same for K and V')
+
+        def table(segs, idx):
+            rows = [None if seg[idx] is None else seg[idx].expand(1, H, 1, c).reshape(H, c) for seg in segs]
+            return None if rows[0] is None else torch.stack(rows).float().contiguous()
+        return ops.fused_attn_channel(q, kbuf, table(k_quant._segments, 1), table(k_quant._segments, 2),
+                                      vbuf, table(v_quant._segments, 1), table(v_quant._segments, 2),
+                                      bits, Lk, softmax_scale, kv_limit=kv_limit, out=out, seg_ends=ends)
+    if km in _TOKEN_METHODS and vm in _TOKEN_METHODS:
+        def per_token(qz):
+            s, z = qz.cached_scale, qz.cached_zp
+            full = torch.empty((B, H, cap, s.shape[3]), dtype=torch.float32, device=q.device)
+            full[:, :, :Lk] = s
+            fz = None
+            if z is not None:
+                fz = torch.zeros_like(full)
+                fz[:, :, :Lk] = z
+            return full, fz
+        (ks, kz), (vs, vz) = per_token(k_quant), per_token(v_quant)
+        return ops.fused_attn(q, kbuf, ks, kz, vbuf, vs, vz, bits, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out)
+    raise ValueError(f'fused_attention: methods {km} / {vm} cannot be combined')
