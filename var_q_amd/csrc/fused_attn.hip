@@ -286,6 +286,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   uint16_t *const lds_wz = reinterpret_cast<uint16_t *>(lds_raw + L::kWz);
   float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
   int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
+  // CHAN: the tables of this head for every segment, [nseg][4][D] fp32: K scale, K zero-point,
+  // V scale, V zero-point (zeros where a table is absent); filled once in the prologue
+  float *const lds_tab = reinterpret_cast<float *>(lds_raw + (L::kBytes + 15) / 16 * 16);
   constexpr int KXS = L::KXS, RSV = L::RSV;
   // parameter block of one tile: ck [NSK][BN]; vr [NSV][BN]; sv [NSV][BN] unless folded
   constexpr bool FOLD_SV = L::kFoldSv;
@@ -328,29 +331,40 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // log2(vs)/ck (three pieces against 1.0), which makes exp2(logit) come out as
   // p * vs without a multiplication; the other upper slots are zero.
   float qbias = 0.f;   // CHAN: -softmax_scale*log2(e) * sum_d q'[d] zk[d] of the current segment
-  auto load_q = [&](int seg) {
+  // (called from two places: force the inlining, or its captures would live in memory)
+  auto load_q = [&](int seg) __attribute__((always_inline)) {
     float qsum[NSK], zb = 0.f;
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
       const int oct = k_octet<GK>(ch, half);
-      uint16_t e[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int d = oct * 8 + KCodec<BITS>::slot_d(j);
-        e[j] = reinterpret_cast<const uint16_t *>(qptr)[d];
-        if constexpr (CHAN) {
-          // q[d] * sk[d], rounded to bf16 like any MFMA operand
-          const int64_t ti = ((int64_t)seg * p.Hkv + hs) * D + d;
-          const float qs = u2f((u32)e[j] << 16) * p.k_chan_scale[ti];
-          e[j] = (uint16_t)(pack_bf16_rne(qs, 0.f) & 0xffffu);
-          if (p.k_chan_zp) zb = __builtin_fmaf(u2f((u32)e[j] << 16), p.k_chan_zp[ti], zb);
-        }
-        qsum[ch / (GK / 16)] += u2f((u32)e[j] << 16);
+      // the octet's eight channels in one 16-byte load, then into the codec's slot order
+      const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
+      float sk[8], zk[8];
+      if constexpr (CHAN) {
+        const float *tk = lds_tab + (seg * 4 + 0) * D + oct * 8, *tz = lds_tab + (seg * 4 + 1) * D + oct * 8;
+        const float4 s0 = *reinterpret_cast<const float4 *>(tk), s1 = *reinterpret_cast<const float4 *>(tk + 4);
+        const float4 z0 = *reinterpret_cast<const float4 *>(tz), z1 = *reinterpret_cast<const float4 *>(tz + 4);
+        sk[0] = s0.x; sk[1] = s0.y; sk[2] = s0.z; sk[3] = s0.w; sk[4] = s1.x; sk[5] = s1.y; sk[6] = s1.z; sk[7] = s1.w;
+        zk[0] = z0.x; zk[1] = z0.y; zk[2] = z0.z; zk[3] = z0.w; zk[4] = z1.x; zk[5] = z1.y; zk[6] = z1.z; zk[7] = z1.w;
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) qb[ch][j] = (u32)e[2 * j] | ((u32)e[2 * j + 1] << 16);
+      for (int j2 = 0; j2 < 4; ++j2) {
+        // operand slots 2*j2 and 2*j2+1, one dword
+        const int d0 = KCodec<BITS>::slot_d(2 * j2), d1 = KCodec<BITS>::slot_d(2 * j2 + 1);   // channels within the octet
+        const u32 lo = (raw[d0 >> 1] >> (16 * (d0 & 1))) << 16, hi = (raw[d1 >> 1] >> (16 * (d1 & 1))) << 16;
+        u32 pair = (lo >> 16) | hi;
+        if constexpr (CHAN) {
+          // q[d] * sk[d], rounded to bf16 like any MFMA operand
+          pair = pack_bf16_rne(u2f(lo) * sk[d0], u2f(hi) * sk[d1]);
+          zb = __builtin_fmaf(u2f(pair << 16), zk[d0], zb);
+          zb = __builtin_fmaf(u2f(pair & 0xffff0000u), zk[d1], zb);
+        }
+        qb[ch][j2] = pair;
+        qsum[ch / (GK / 16)] += u2f(pair << 16) + u2f(pair & 0xffff0000u);
+      }
+      if constexpr (CHAN) __builtin_amdgcn_sched_barrier(0);   // one chunk's table entries in registers at a time
     }
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
@@ -364,8 +378,6 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       else bq[s] = u32x4_t{0u, 0u, 0u, 0u};
     }
   };
-  load_q(0);
-
   // ---- tile range: every lane of the workgroup runs the same number of tiles ----
   __shared__ int lds_maxlim;
   if (tid == 0) lds_maxlim = 0;
@@ -374,20 +386,37 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   __syncthreads();
   const int kv_end = lds_maxlim;
   int n_tiles = (kv_end + BN - 1) / BN;
+  // segment ends in LDS: indexing the kernel arguments with a run-time index would move
+  // the whole argument block to scratch memory
+  __shared__ int lds_seg_end[kMaxSegments];
   if constexpr (CHAN) {
     // key tiles never straddle a segment of the tables: count them segment by segment
+    // (literal indices only: a loop index would be a run-time index at the time the
+    // argument block is split into registers)
     n_tiles = 0;
-    for (int s = 0, beg = 0; s < p.nseg && beg < kv_end; beg = p.seg_end[s], ++s)
-      n_tiles += (min(p.seg_end[s], kv_end) - beg + BN - 1) / BN;
+    int beg = 0;
+#define VARQ_SEG(S)                                                                            \
+  {                                                                                            \
+    const int e = p.seg_end[S];                                                                \
+    if (tid == 0) lds_seg_end[S] = e;                                                          \
+    if (S < p.nseg && beg < kv_end) n_tiles += (min(e, kv_end) - beg + BN - 1) / BN;           \
+    beg = e;                                                                                   \
+  }
+    VARQ_SEG(0) VARQ_SEG(1) VARQ_SEG(2) VARQ_SEG(3) VARQ_SEG(4) VARQ_SEG(5) VARQ_SEG(6) VARQ_SEG(7)
+    VARQ_SEG(8) VARQ_SEG(9) VARQ_SEG(10) VARQ_SEG(11) VARQ_SEG(12) VARQ_SEG(13) VARQ_SEG(14) VARQ_SEG(15)
+#undef VARQ_SEG
+    static_assert(kMaxSegments == 16, "the list above names every segment");
+    __syncthreads();
   }
   // Position of a stream of consecutive tiles (the K prefetch, the V prefetch and the
   // attention itself each walk the tiles in order).  Without segments tile t starts at
   // key t * BN; with segments a tile ends where its segment ends.
   struct TileCursor { int seg, start; };
-  auto cursor_advance = [&](TileCursor &c) {
+  auto cursor_advance = [&](TileCursor &c) __attribute__((always_inline)) {
     if constexpr (CHAN) {
       c.start += BN;
-      if (c.start >= p.seg_end[c.seg] && c.seg + 1 < p.nseg) { c.start = p.seg_end[c.seg]; ++c.seg; }
+      const int e = __builtin_amdgcn_readfirstlane(lds_seg_end[c.seg]);
+      if (c.start >= e && c.seg + 1 < p.nseg) { c.start = e; ++c.seg; }
     } else {
       c.start += BN;
     }
@@ -570,7 +599,17 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   if (tid < 3) lds_flag[tid] = 0;
   if (tid < 3 * RSR) lds_wz[((tid / RSR) * 8 + 7) * RSR + tid % RSR] = 0;   // the all-zero row of each slot
   __syncthreads();
-  if (n_tiles > 0) { prefetch_k(0); prefetch(0); stage(0); widen_k(0); }
+  if (n_tiles > 0) { prefetch_k(0); prefetch(0); }
+  if constexpr (CHAN) {
+    for (int i = tid; i < p.nseg * 4 * D; i += NT) {
+      const int seg = i / (4 * D), which = (i / D) & 3, d = i % D;
+      const float *src = which == 0 ? p.k_chan_scale : which == 1 ? p.k_chan_zp : which == 2 ? p.v_chan_scale : p.v_chan_zp;
+      lds_tab[i] = src ? src[((int64_t)seg * p.Hkv + hs) * D + d] : 0.f;
+    }
+    __syncthreads();
+  }
+  load_q(0);   // behind the first tile's requests, so the two latencies overlap
+  if (n_tiles > 0) { stage(0); widen_k(0); }
   if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
   if (n_tiles > 0) widen_v(0);
@@ -614,28 +653,29 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // with rq, l_sum the readings of the extra block; the accumulators are re-expressed so that
   // the same formula holds with the new tables and l_prev = l_sum, and the Q operands are
   // rebuilt with the new K table.
-  auto segment_boundary = [&](int seg_new) {
+  auto segment_boundary = [&](int seg_new) __attribute__((always_inline)) {
     if constexpr (CHAN) {
       const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
       const float dl = l_sum - l_prev;
       constexpr float VM = VCodec<BITS>::kMul;
-      const float *sv_old = p.v_chan_scale + ((int64_t)seg_a * p.Hkv + hs) * D;
-      const float *sv_new = p.v_chan_scale + ((int64_t)seg_new * p.Hkv + hs) * D;
-      const float *zv_old = p.v_chan_zp ? p.v_chan_zp + ((int64_t)seg_a * p.Hkv + hs) * D : nullptr;
+      const float *sv_old = lds_tab + (seg_a * 4 + 2) * D, *zv_old = lds_tab + (seg_a * 4 + 3) * D;
+      const float *sv_new = lds_tab + (seg_new * 4 + 2) * D;
 #pragma unroll
       for (int d = 0; d < NDB; ++d)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int c0 = d * 32 + 8 * g4 + 4 * half;
           const float4 so = *reinterpret_cast<const float4 *>(sv_old + c0), sn = *reinterpret_cast<const float4 *>(sv_new + c0);
-          float4 zo = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (zv_old) zo = *reinterpret_cast<const float4 *>(zv_old + c0);
-          const float ro[4] = {so.x / sn.x, so.y / sn.y, so.z / sn.z, so.w / sn.w};
+          const float4 zo = *reinterpret_cast<const float4 *>(zv_old + c0);
+          // (the hardware reciprocal is accurate to an ulp, which is all a change of units needs)
+          const float ro[4] = {so.x * __builtin_amdgcn_rcpf(sn.x), so.y * __builtin_amdgcn_rcpf(sn.y),
+                               so.z * __builtin_amdgcn_rcpf(sn.z), so.w * __builtin_amdgcn_rcpf(sn.w)};
           const float zz[4] = {zo.x, zo.y, zo.z, zo.w};
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             oacc[d][4 * g4 + j] = (ro[j] * (VM * oacc[d][4 * g4 + j] - rq - zz[j] * dl) + rq) * (1.f / VM);
+          __builtin_amdgcn_sched_barrier(0);   // one slice's registers at a time
         }
       l_prev = l_sum;
       seg_a = seg_new;
@@ -646,8 +686,8 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   auto begin_tile = [&](int tile) {
     if constexpr (CHAN) {
       t0 = cur_a.start;
-      tile_end = min(t0 + BN, p.seg_end[cur_a.seg]);
-      if (cur_a.seg != seg_a) segment_boundary(cur_a.seg);
+      tile_end = min(t0 + BN, __builtin_amdgcn_readfirstlane(lds_seg_end[cur_a.seg]));
+      if (__builtin_expect(cur_a.seg != seg_a, 0)) segment_boundary(cur_a.seg);
       cursor_advance(cur_a);
     } else {
       t0 = tile * BN;
@@ -878,10 +918,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
         if constexpr (CHAN) {
           // weighted mean of the codes -> values: sv * (mean - zv * share) per channel, share
           // = the part of the weights that belongs to the current segment (1 without segments)
-          const int64_t c0 = ((int64_t)seg_a * p.Hkv + hs) * D + d * 32 + 8 * g4 + 4 * half;
-          const float4 sv = *reinterpret_cast<const float4 *>(p.v_chan_scale + c0);
-          float4 zv = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (p.v_chan_zp) zv = *reinterpret_cast<const float4 *>(p.v_chan_zp + c0);
+          const int c0 = d * 32 + 8 * g4 + 4 * half;
+          const float4 sv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * 4 + 2) * D + c0);
+          const float4 zv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * 4 + 3) * D + c0);
           const float share = (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
           o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
           o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
@@ -895,7 +934,8 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 
 template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
-  constexpr int lds_bytes = AttnLds<D, BITS, GK, GV>::kBytes;
+  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * 4 * D * 4 : 0);
+  static_assert(lds_bytes <= 160 * 1024, "LDS budget");
   static bool configured = false;   // above 64 KiB the limit has to be raised once per process
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN>),
@@ -997,8 +1037,9 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
   VARQ_CHECK_ARG((int64_t)B * Hkv * Lk_stride * D < (1ll << 40), "fused_attn_channel: cache too large");
   VARQ_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
                  "fused_attn_channel: q must be 16-byte and out 8-byte aligned");
-  VARQ_CHECK_ARG(((uintptr_t)v_chan_scale & 15) == 0 && ((uintptr_t)v_chan_zp & 15) == 0,
-                 "fused_attn_channel: the V tables must be 16-byte aligned");
+  VARQ_CHECK_ARG(((uintptr_t)k_chan_scale & 15) == 0 && ((uintptr_t)k_chan_zp & 15) == 0 &&
+                     ((uintptr_t)v_chan_scale & 15) == 0 && ((uintptr_t)v_chan_zp & 15) == 0,
+                 "fused_attn_channel: the tables must be 16-byte aligned");
 
   AttnParams p;
   p.q = reinterpret_cast<const __bf16 *>(q);
