@@ -273,7 +273,7 @@ def main():
         'attn_query_tokens_per_s': round(B * LQ / t_at, 1),
         'pack_GBps': round(pack_gbps, 2), 'pack_frac_hbm_peak': round(pack_gbps / HBM_PEAK_GBPS, 4),
         'pack_us_per_tensor': round(t_quant * 1e6, 2), 'pack_tokens_per_s': round(B * L / t_quant, 1),
-        'roofline': {'kernel': 'fused_attn_kernel<128,4,128,128>', 'bound': 'mfma', 'achieved': round(attn_tflops, 2),
+        'roofline': {'kernel': 'fused_attn_kernel<128,4,128,128,token scales>', 'bound': 'mfma', 'achieved': round(attn_tflops, 2),
                      'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s', 'frac': round(attn_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
                      'traffic': None if not traffic else traffic.get('fused_attn')},
         'roofline_pack': {'kernel': 'quant_pack_rows32_kernel<bf16,4,asym,4 lanes per group,dense>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
