@@ -61,7 +61,21 @@ def test_invalid_arguments_are_rejected_on_the_host():
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 8, 128,
                              1, 2, 2, None, 16, 16, 16, 128, None, 1.0, None)
     assert rc == -2
+    # per-channel attention: segment table checks
+    i32 = lambda v: (ctypes.c_int32 * len(v))(*v)
+    chan = lambda nseg, ends, Lk=16, D=128: lib.varq_fused_attn_channel(
+        fake, fake, fake, fake, None, fake, fake, None, nseg, ends, 8, 1, 2, 2, None, 16, Lk, 16, D, None, 1.0, None)
+    assert chan(0, None) == -1 and b'nseg' in lib.varq_last_error()
+    assert chan(17, None) == -1 and b'nseg' in lib.varq_last_error()
+    assert chan(2, None) == -1 and b'segment ends missing' in lib.varq_last_error()
+    assert chan(3, i32([8, 4, 16])) == -1 and b'increase' in lib.varq_last_error()
+    assert chan(2, i32([40, 16])) == -1 and b'beyond' in lib.varq_last_error()
+    assert chan(1, None, D=96) == -1 and b'D must be' in lib.varq_last_error()
+    rc = lib.varq_fused_attn_channel(fake, fake, fake, ctypes.c_void_p(0x1004), None, fake, fake, None, 1, None,
+                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, None)
+    assert rc == -1 and b'aligned' in lib.varq_last_error()
     # empty inputs are a no-op success
+    assert chan(1, None, Lk=0) == -1          # queries but no keys
     assert lib.varq_pack(None, 0, 16, 4, None, None) == 0
     assert lib.varq_quant_pack_rows(fake, 1, 0, 64, 64, 4, 1, 1e-12, None, None, fake, fake, fake, None) == 0
 
