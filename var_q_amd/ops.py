@@ -288,8 +288,8 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
     reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
     (G_TENSOR, G_SCALE) expanded to the table, and the affine per-head-per-dim variant.
     q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32; k_chan_scale,
-    v_chan_scale, v_chan_zp fp32 with nseg*Hkv*D elements (any shape that flattens to
-    [nseg, Hkv, D]).  seg_ends (at most 16 increasing key counts, the last one = Lk) says
+    v_chan_scale, v_chan_zp fp32 with at least nseg*Hkv*D elements (any shape that flattens to
+    [>= nseg, Hkv, D]).  seg_ends (at most 16 increasing key counts, the last one = Lk) says
     where the tables change along the keys: a cache filled step by step by the reference's
     append methods has one table per step (VAR_Q/quant.py:196-201).
     With a single table the zero-point of K may be None even for an affine K: it shifts all
@@ -311,8 +311,8 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                  (v_chan_zp, 'v_chan_zp')):
         if t is not None:
             _gpu(t, n)
-            assert t.dtype == torch.float32 and t.numel() == nseg * Hkv * D and t.is_contiguous(), \
-                f'{n} must be fp32 [nseg, Hkv, D]'
+            assert t.dtype == torch.float32 and t.numel() >= nseg * Hkv * D and t.is_contiguous(), \
+                f'{n} must be fp32 [nseg, Hkv, D] (more tables than segments are allowed)'
     if out is None:
         out = torch.empty_like(q)
     if kv_limit is not None:

@@ -117,8 +117,15 @@ class VAR_Q:
 
     # ---------------- cache views ----------------
     def _reset_cache(self):
-        # (tokens, scale, zp) of every cached step, for the fused attention
-        self._segments: List[Tuple[int, torch.Tensor, Optional[torch.Tensor]]] = []
+        # what the fused attention reads, kept up to date by cache(): the end of every cached
+        # step with its (head, channel) tables for the methods whose scale is shared by the
+        # tokens of a step, a full-size [B,H,capacity,groups] copy of the per-token scales for
+        # the others
+        self._seg_ends: List[int] = []
+        self._tab_scale: Optional[torch.Tensor] = None      # [MAX_TABLE_STEPS, H, c]
+        self._tab_zp: Optional[torch.Tensor] = None
+        self._tok_scale = _Growable(2)
+        self._tok_zp = _Growable(2)
         self._c_item = _Growable(self.dim_cat)
         self._c_scale = _Growable(self.dim_cat)
         self._c_zp = _Growable(self.dim_cat)
@@ -188,15 +195,40 @@ class VAR_Q:
             self._c_scale.append(s_cur)
             if z_cur is not None:
                 self._c_zp.append(z_cur)
-            self._segments.append((q_cur.size(self.dim_cat), self.scale, self.zp))
+            self._note_step(q_cur, replace=False)
         elif m == 'G_HEAD_DIM':
             self._c_item.replace(q_cur)
             self._c_scale.replace(s_cur)
             if z_cur is not None:
                 self._c_zp.replace(z_cur)
-            self._segments = [(q_cur.size(self.dim_cat), self.scale, self.zp)]
+            self._note_step(q_cur, replace=True)
         else:
             raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
+
+    def _note_step(self, q_cur: torch.Tensor, replace: bool):
+        """Book-keeping for `fused_attention` (layout BHLc, packed codes only)."""
+        if self.qkv_format != 'BHLc' or not self.pack_to_int32:
+            return
+        B, H, n, _ = q_cur.shape
+        c = self._pack_meta['orig_c']
+        if self.quant_method in _TABLE_METHODS:
+            if replace:
+                self._seg_ends = []
+            k = len(self._seg_ends)
+            self._seg_ends.append((self._seg_ends[-1] if self._seg_ends else 0) + n)
+            if k >= MAX_TABLE_STEPS:
+                return                                   # fused_attention refuses; the drop-in path is unaffected
+            if self._tab_scale is None:
+                self._tab_scale = torch.empty((MAX_TABLE_STEPS, H, c), dtype=torch.float32, device=q_cur.device)
+                self._tab_zp = None if self.zp is None else torch.empty_like(self._tab_scale)
+            self._tab_scale[k].copy_(self.scale.expand(1, H, 1, c).reshape(H, c))
+            if self.zp is not None:
+                self._tab_zp[k].copy_(self.zp.expand(1, H, 1, c).reshape(H, c))
+        else:
+            ng = self.scale.shape[3]
+            self._tok_scale.append(self.scale.expand(B, H, n, ng))
+            if self.zp is not None:
+                self._tok_zp.append(self.zp.expand(B, H, n, ng))
 
     # ---------------- dequantize ----------------
     def _dequant(self, q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor]) -> torch.Tensor:
@@ -258,8 +290,10 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     c in {64, 128}, after at least one `cache()`.  Methods whose scale is shared by the
     tokens of a step (G_SCALE_HEAD_DIM -- the shipped rule --, G_HEAD_DIM, G_TENSOR, G_SCALE,
     G_HEAD) go through one table per cached step, at most MAX_TABLE_STEPS steps; per-token
-    methods (G_TOKEN, G_TOKEN_HEAD, G_GROUP) through per-token scales.  kv_limit: int32
-    [Lq], query i sees keys j < kv_limit[i].  Returns bf16 [B,H,Lq,c]."""
+    methods (G_TOKEN, G_TOKEN_HEAD, G_GROUP) through per-token scales.  Everything the
+    kernels read is kept current by `cache()`, so a call launches the attention and nothing
+    else.  kv_limit: int32 [Lq], query i sees keys j < kv_limit[i].  Returns bf16
+    [B,H,Lq,c]."""
     for qz, n in ((k_quant, 'k_quant'), (v_quant, 'v_quant')):
         if qz.qkv_format != 'BHLc':
             raise ValueError(f'fused_attention: {n} must use layout BHLc')
@@ -280,31 +314,17 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     assert q.dim() == 4 and q.shape[0] == B and q.shape[1] == H and q.shape[3] == c, 'q must be [B,H,Lq,c]'
     km, vm = k_quant.quant_method, v_quant.quant_method
     if km in _TABLE_METHODS and vm in _TABLE_METHODS:
-        ends, acc = [], 0
-        for (n, _, _), (nv, _, _) in zip(k_quant._segments, v_quant._segments):
-            if n != nv:
-                raise ValueError('fused_attention: K and V were cached in different steps')
-            acc += n
-            ends.append(acc)
-        if len(ends) > MAX_TABLE_STEPS or len(v_quant._segments) != len(ends) or acc != Lk:
+        ends = k_quant._seg_ends
+        if ends != v_quant._seg_ends:
+            raise ValueError('fused_attention: K and V were cached in different steps')
+        if len(ends) > MAX_TABLE_STEPS or not ends or ends[-1] != Lk:
             raise ValueError(f'fused_attention: at most {MAX_TABLE_STEPS} cached steps, the same for K and V')
-
-        def table(segs, idx):
-            rows = [None if seg[idx] is None else seg[idx].expand(1, H, 1, c).reshape(H, c) for seg in segs]
-            return None if rows[0] is None else torch.stack(rows).float().contiguous()
-        return ops.fused_attn_channel(q, kbuf, table(k_quant._segments, 1), table(k_quant._segments, 2),
-                                      vbuf, table(v_quant._segments, 1), table(v_quant._segments, 2),
-                                      bits, Lk, softmax_scale, kv_limit=kv_limit, out=out, seg_ends=ends)
+        return ops.fused_attn_channel(q, kbuf, k_quant._tab_scale, k_quant._tab_zp, vbuf, v_quant._tab_scale,
+                                      v_quant._tab_zp, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out,
+                                      seg_ends=ends)
     if km in _TOKEN_METHODS and vm in _TOKEN_METHODS:
-        def per_token(qz):
-            s, z = qz.cached_scale, qz.cached_zp
-            full = torch.empty((B, H, cap, s.shape[3]), dtype=torch.float32, device=q.device)
-            full[:, :, :Lk] = s
-            fz = None
-            if z is not None:
-                fz = torch.zeros_like(full)
-                fz[:, :, :Lk] = z
-            return full, fz
-        (ks, kz), (vs, vz) = per_token(k_quant), per_token(v_quant)
+        ks, kz, vs, vz = k_quant._tok_scale.buf, k_quant._tok_zp.buf, v_quant._tok_scale.buf, v_quant._tok_zp.buf
+        if ks.shape[2] != cap or vs.shape[2] != cap:
+            raise ValueError('fused_attention: scale buffers and code buffers differ in capacity')
         return ops.fused_attn(q, kbuf, ks, kz, vbuf, vs, vz, bits, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out)
     raise ValueError(f'fused_attention: methods {km} / {vm} cannot be combined')
