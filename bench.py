@@ -10,7 +10,7 @@ After the timed region (and outside `value`) it also replays benchmark configura
 one image batch of the Infinity schedule through the pre-allocated mixed-bit
 cache (append + attend per scale), and reports its latency per image.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5] [--no-c3]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5] [--no-c3] [--no-rule]
 """
 import argparse
 import json
@@ -143,6 +143,48 @@ def c3_rates(torch, dev, reps=20, warm=5):
     return out
 
 
+def shipped_rule_latency(torch, dev, passes=5, warm=2):
+    """The rule of the shipped JSON files (G_SCALE_HEAD_DIM, 8 bits, layout BHLc) over the 13
+    Infinity scales, B=2 (one image, CFG pair), H=16, D=128, one layer: per scale quantize +
+    cache K and V with the drop-in quantizers, then attend.  'dropin' dequantizes the whole
+    cache to fp32 and calls torch's scaled_dot_product_attention in bf16 (what the reference
+    does), 'fused' attends over the packed caches (`fused_attention`)."""
+    import torch.nn.functional as F
+    from var_q_amd import VAR_Q
+    from var_q_amd.quant import fused_attention
+    from var_q_amd.schedules import INFINITY_PATCH_NUMS
+    B, H, D = 2, 16, 128
+    gd = torch.Generator(device=dev).manual_seed(7007)
+    steps = [tuple(torch.randn(B, H, pn * pn, D, device=dev, generator=gd).bfloat16() for _ in range(3))
+             for pn in INFINITY_PATCH_NUMS]
+    scale = 1.0 / math.sqrt(D)
+
+    def one_pass(fused):
+        kq, vq = VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM'), VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM')
+        for q, k, v in steps:
+            if fused:
+                for quantizer, item in ((kq, k), (vq, v)):
+                    quantizer.quant(item)
+                    quantizer.cache()
+                fused_attention(q, kq, vq, scale)
+            else:
+                kk, vv = kq.use_var_q(k), vq.use_var_q(v)
+                F.scaled_dot_product_attention(q, kk.to(torch.bfloat16), vv.to(torch.bfloat16), scale=scale)
+
+    out = {'workload': 'shipped rule G_SCALE_HEAD_DIM 8-bit BHLc, 13 Infinity scales, B=2 H=16 D=128, one layer: '
+                       'quantize + cache + attention per scale'}
+    for name, fused in (('dropin_dequant_sdpa_ms', False), ('fused_ms', True)):
+        for _ in range(warm):
+            one_pass(fused)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            one_pass(fused)
+        torch.cuda.synchronize()
+        out[name] = round((time.perf_counter() - t0) / passes * 1e3, 3)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -151,6 +193,7 @@ def main():
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
     ap.add_argument('--no-c5', action='store_true', help='skip the config-5 latency leg (profiling runs)')
     ap.add_argument('--no-c3', action='store_true', help='skip the config-3 rates leg (profiling runs)')
+    ap.add_argument('--no-rule', action='store_true', help='skip the shipped-rule latency leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -282,6 +325,7 @@ def main():
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
+        'shipped_rule_latency': None if args.no_rule else shipped_rule_latency(torch, dev),
     }
     print(json.dumps(line), flush=True)
 

@@ -655,6 +655,10 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // rebuilt with the new K table.
   auto segment_boundary = [&](int seg_new) __attribute__((always_inline)) {
     if constexpr (CHAN) {
+      // (the Q operands first: with the accumulator arithmetic in front of it the register
+      // allocator spills, and spills here cost scratch traffic at every boundary)
+      load_q(seg_new);
+      __builtin_amdgcn_sched_barrier(0);
       const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
       const float dl = l_sum - l_prev;
@@ -679,7 +683,6 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
         }
       l_prev = l_sum;
       seg_a = seg_new;
-      load_q(seg_new);
     }
   };
 
