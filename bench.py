@@ -193,6 +193,7 @@ def main():
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
     ap.add_argument('--no-c5', action='store_true', help='skip the config-5 latency leg (profiling runs)')
     ap.add_argument('--no-c3', action='store_true', help='skip the config-3 rates leg (profiling runs)')
+    ap.add_argument('--single-launches', action='store_true', help='quantize K and V in two launches instead of one')
     ap.add_argument('--no-rule', action='store_true', help='skip the shipped-rule latency leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
@@ -231,11 +232,17 @@ def main():
     o = torch.empty_like(q)
     rowmap = [1, 1, B * H * L, 0, 0, 1, 0, -1]
 
+    PAIR = not args.single_launches
+
     def step(i, ev=None):
         s, t = i % NBUF, outs[i % NBUF]
         if ev: ev[0].record()
-        ops.quant_pack_rows_into(ks_in[s], GROUP, BITS, True, 1e-12, t['kw'], t['ks'], t['kz'], rowmap)
-        ops.quant_pack_rows_into(vs_in[s], GROUP, BITS, True, 1e-12, t['vw'], t['vs'], t['vz'], rowmap)
+        if PAIR:   # K and V of the step in one launch, as the cache append does
+            ops.quant_pack_rows_pair_into(ks_in[s], vs_in[s], GROUP, BITS, True, 1e-12, (t['kw'], t['ks'], t['kz']),
+                                          (t['vw'], t['vs'], t['vz']), rowmap)
+        else:
+            ops.quant_pack_rows_into(ks_in[s], GROUP, BITS, True, 1e-12, t['kw'], t['ks'], t['kz'], rowmap)
+            ops.quant_pack_rows_into(vs_in[s], GROUP, BITS, True, 1e-12, t['vw'], t['vs'], t['vz'], rowmap)
         if ev: ev[1].record()
         ops.fused_attn(q, t['kw'], t['ks'], t['kz'], t['vw'], t['vs'], t['vz'], BITS, BITS, L, scale, out=o)
         if ev: ev[2].record()
@@ -321,7 +328,8 @@ def main():
                      'traffic': None if not traffic else traffic.get('fused_attn')},
         'roofline_pack': {'kernel': 'quant_pack_rows32_kernel<bf16,4,asym,4 lanes per group,dense>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
                           'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(pack_gbps / HBM_PEAK_GBPS, 4),
-                          'traffic': None if not traffic else traffic.get('quant_pack_rows')},
+                          'traffic': None if not traffic else traffic.get('quant_pack_rows', 0) // (1 if PAIR else 2) or None,
+                          'tensors_per_launch': 2 if PAIR else 1},
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),

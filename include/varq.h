@@ -74,6 +74,17 @@ int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, int c, int 
                          int32_t *words, float *scale, float *zp, void *stream);
 
 /*
+ * The same for two tensors of one shape in one launch -- K and V of a cache step, which
+ * the reference quantizes one after the other (VAR/models/basic_var.py:146-147,
+ * Infinity/infinity/models/basic.py:329-330).  Row map and slot table are shared; each
+ * tensor has its own outputs.  Results are those of two varq_quant_pack_rows calls.
+ */
+int varq_quant_pack_rows2(const void *x0, const void *x1, int x_dtype, int64_t n_rows, int c, int group,
+                          int bits, int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
+                          int32_t *words0, float *scale0, float *zp0, int32_t *words1, float *scale1,
+                          float *zp1, void *stream);
+
+/*
  * General quantizer for the six grouping methods of VAR_Q/quant.py:75-95 and
  * any other reduce set: a group is every element sharing the indices of the
  * dims NOT in reduce_mask (bit d set = dim d reduced).  Two phases: group

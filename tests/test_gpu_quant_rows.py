@@ -157,3 +157,35 @@ def test_error_statistics_match_the_oracle(dev, bits, sym, tmp_path):
     rep = CsvReport(str(tmp_path / 'r.csv'))
     rep.add(st)
     assert float(rep.rows()[0]['l2_norm_error']) == pytest.approx(want, rel=1e-6)
+
+
+@pytest.mark.parametrize('bits,group,asym,dtype', [(4, 128, True, torch.bfloat16), (8, 64, False, torch.float32),
+                                                    (2, 32, True, torch.float16), (4, 16, True, torch.bfloat16)])
+def test_pair_launch_equals_two_launches(dev, bits, group, asym, dtype):
+    """varq_quant_pack_rows2: K and V of one step in one launch, written through a shared row
+    map (a window of a larger cache, heads picked by a slot table); same bytes as two calls."""
+    B, H, n, D, Lmax, start = 2, 5, 37, 128, 64, 11
+    heads = [3, 0, 4]
+    g = torch.Generator().manual_seed(bits * 7 + group)
+    k = (torch.randn(B, H, n, D, generator=g) * 3).to(dtype).to(dev)
+    v = (torch.randn(B, H, n, D, generator=g) * 3).to(dtype).to(dev)
+    slot = torch.full((H,), -1, dtype=torch.int32)
+    for i, h in enumerate(heads):
+        slot[h] = i
+    slot = slot.to(dev)
+    hc, W, ng = len(heads), D * bits // 32, D // group
+    rowmap = [B, H, n, hc * Lmax, Lmax, 1, start, 1]
+
+    def bufs():
+        return (torch.full((B, hc, Lmax, W), 7, dtype=torch.int32, device=dev),
+                torch.full((B, hc, Lmax, ng), 7.0, device=dev), torch.full((B, hc, Lmax, ng), 7.0, device=dev) if asym else None)
+    a_k, a_v, b_k, b_v = bufs(), bufs(), bufs(), bufs()
+    note('quant_pack_rows2', bits, group, asym, dtype)
+    ops.quant_pack_rows_into(k, group, bits, asym, 1e-12, *a_k, rowmap, slot)
+    ops.quant_pack_rows_into(v, group, bits, asym, 1e-12, *a_v, rowmap, slot)
+    ops.quant_pack_rows_pair_into(k, v, group, bits, asym, 1e-12, b_k, b_v, rowmap, slot)
+    torch.cuda.synchronize()
+    for x, y in zip(a_k + a_v, b_k + b_v):
+        if x is not None:
+            assert torch.equal(x, y)
+    assert not torch.equal(a_k[0], a_v[0])        # the two tensors did differ

@@ -14,6 +14,9 @@ SYMBOLS = {
     'varq_last_error': (c_char_p, []),
     'varq_quant_pack_rows': (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_float,
                                      POINTER(c_int64), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'varq_quant_pack_rows2': (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_float,
+                                      POINTER(c_int64), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_void_p]),
     'varq_quant_workspace_bytes': (c_size_t, [POINTER(c_int64), c_int]),
     'varq_quant_pack': (c_int, [c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_int, c_float,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

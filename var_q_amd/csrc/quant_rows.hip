@@ -22,6 +22,12 @@ struct RowsParams {
   int32_t *words;
   float *scale;
   float *zp;
+  // a second tensor of the same shape (K and V of one cache step in one launch), or NULLs;
+  // it takes the upper half of grid.z
+  const void *x1;
+  int32_t *words1;
+  float *scale1;
+  float *zp1;
   const int32_t *slot;
   RowMap map;
   int64_t octets_per_pair;   // n2 * c8
@@ -76,7 +82,12 @@ __device__ __forceinline__ void quantize_octet(const float (&v)[8], float s, flo
 template <int DT, int BITS, bool ASYM, int LPG>
 __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   // grid = (tiles of one pair, n1, n0): no division to find the pair
-  const int64_t i0 = blockIdx.z, i1 = blockIdx.y;
+  const bool second = blockIdx.z >= (unsigned)p.map.n0;   // block-uniform
+  const void *px = second ? p.x1 : p.x;
+  int32_t *pwords = second ? p.words1 : p.words;
+  float *pscale = second ? p.scale1 : p.scale;
+  float *pzp = second ? p.zp1 : p.zp;
+  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
   const int64_t pair = i0 * p.map.n1 + i1;
   const int tile = blockIdx.x;
 
@@ -92,7 +103,7 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   const int64_t in_elem = (pair * p.octets_per_pair + oc) * 8;
 
   float v[8];
-  In8<DT>::load(p.x, in_elem, v);
+  In8<DT>::load(px, in_elem, v);
 
   float mn, mx;
   if (ASYM) {
@@ -136,17 +147,17 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   const int64_t out_row = out_base + (int64_t)i2 * p.map.os2;
 
   if (BITS == 8) {
-    uint2 *dst = reinterpret_cast<uint2 *>(p.words + (out_row * p.c8 + col) * 2);
+    uint2 *dst = reinterpret_cast<uint2 *>(pwords + (out_row * p.c8 + col) * 2);
     *dst = make_uint2(w0, w1);
   } else if (BITS == 4) {
-    p.words[out_row * p.c8 + col] = (int32_t)w0;
+    pwords[out_row * p.c8 + col] = (int32_t)w0;
   } else {
-    if ((threadIdx.x & 1) == 0) p.words[(out_row * p.c8 + col) >> 1] = (int32_t)w0;
+    if ((threadIdx.x & 1) == 0) pwords[(out_row * p.c8 + col) >> 1] = (int32_t)w0;
   }
   if ((col & (LPG - 1)) == 0) {
     const int64_t g = out_row * p.nseg + col / LPG;
-    p.scale[g] = s;
-    if (ASYM) p.zp[g] = zp;
+    pscale[g] = s;
+    if (ASYM) pzp[g] = zp;
   }
 }
 
@@ -168,7 +179,12 @@ template <int DT, int BITS, bool ASYM, int LPG4, bool DENSE>
 __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   __shared__ Raw8<DT> lds_stage[4][256];   // per wave: 256 octets in, then packed words out
 
-  const int64_t i0 = blockIdx.z, i1 = blockIdx.y;
+  const bool second = blockIdx.z >= (unsigned)p.map.n0;   // block-uniform
+  const void *px = second ? p.x1 : p.x;
+  int32_t *pwords = second ? p.words1 : p.words;
+  float *pscale = second ? p.scale1 : p.scale;
+  float *pzp = second ? p.zp1 : p.zp;
+  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
   const int64_t pair = i0 * p.map.n1 + i1;
   int64_t s0 = i0, s1 = i1;
   if (p.map.slot_dim == 0) s0 = p.slot[i0];
@@ -189,7 +205,7 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
     int o = w0 + k * 64 + lane;
     o = o < n_oct ? o : 0;                            // past the end: re-read octet 0, never stored
     Raw8<DT> r;
-    r.load(p.x, pair_elem0 + (int64_t)o * 8);
+    r.load(px, pair_elem0 + (int64_t)o * 8);
     stage[k * 64 + lane] = r;
   }
   __builtin_amdgcn_wave_barrier();
@@ -310,25 +326,25 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
       const u32x4 out4 = reinterpret_cast<const u32x4 *>(wstage)[lane];
       const int o = w0 + 4 * lane;                    // octet == word index for 4-bit codes
       if (o < n_oct)
-        __builtin_nontemporal_store(out4, reinterpret_cast<u32x4 *>(p.words + out_base * p.c8 + o));
+        __builtin_nontemporal_store(out4, reinterpret_cast<u32x4 *>(pwords + out_base * p.c8 + o));
     } else if (live) {
       const int64_t wbase = out_base * p.c8 + oct0;   // in octets
       if (BITS == 8) {
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          *reinterpret_cast<uint2 *>(p.words + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
+          *reinterpret_cast<uint2 *>(pwords + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
       } else if (LPG4 == 1) {
-        *reinterpret_cast<uint2 *>(p.words + (wbase >> 1)) =
+        *reinterpret_cast<uint2 *>(pwords + (wbase >> 1)) =
             make_uint2(w[0][0] | (w[1][0] << 16), w[2][0] | (w[3][0] << 16));
       } else if ((j & 1) == 0) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) p.words[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
+        for (int k = 0; k < 4; ++k) pwords[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
       }
     }
     if (live && j == 0) {
       const int64_t g = out_base * p.nseg + oct0 / (4 * LPG4);
-      p.scale[g] = s;
-      if (ASYM) p.zp[g] = zp;
+      pscale[g] = s;
+      if (ASYM) pzp[g] = zp;
     }
     return;
   }
@@ -344,27 +360,27 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   if (BITS == 8) {
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      *reinterpret_cast<uint2 *>(p.words + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
+      *reinterpret_cast<uint2 *>(pwords + (wbase + k * LPG4) * 2) = make_uint2(w[k][0], w[k][1]);
   } else if (BITS == 4) {
     if (LPG4 == 1) {
-      *reinterpret_cast<uint4 *>(p.words + wbase) = make_uint4(w[0][0], w[1][0], w[2][0], w[3][0]);
+      *reinterpret_cast<uint4 *>(pwords + wbase) = make_uint4(w[0][0], w[1][0], w[2][0], w[3][0]);
     } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) p.words[wbase + k * LPG4] = (int32_t)w[k][0];
+      for (int k = 0; k < 4; ++k) pwords[wbase + k * LPG4] = (int32_t)w[k][0];
     }
   } else {
     if (LPG4 == 1) {
-      *reinterpret_cast<uint2 *>(p.words + (wbase >> 1)) =
+      *reinterpret_cast<uint2 *>(pwords + (wbase >> 1)) =
           make_uint2(w[0][0] | (w[1][0] << 16), w[2][0] | (w[3][0] << 16));
     } else if ((j & 1) == 0) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) p.words[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
+      for (int k = 0; k < 4; ++k) pwords[(wbase + k * LPG4) >> 1] = (int32_t)w[k][0];
     }
   }
   if (j == 0) {
     const int64_t g = out_row * p.nseg + col / (4 * LPG4);
-    p.scale[g] = s;
-    if (ASYM) p.zp[g] = zp;
+    pscale[g] = s;
+    if (ASYM) pzp[g] = zp;
   }
 }
 
@@ -405,40 +421,60 @@ int launch_dt(const RowsParams &p, int bits, int asym, int lpg, dim3 grid, hipSt
 
 }  // namespace
 
-extern "C" int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, int c, int group, int bits,
-                                    int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
-                                    int32_t *words, float *scale, float *zp, void *stream) {
-  VARQ_CHECK_ARG(n_rows == 0 || (x && words && scale), "quant_pack_rows: null pointer");
-  VARQ_CHECK_ARG(n_rows == 0 || !asym || zp, "quant_pack_rows: asym needs zp output");
-  VARQ_CHECK_ARG(bits == 2 || bits == 4 || bits == 8, "quant_pack_rows: bits must be 2, 4 or 8 (got %d)", bits);
-  VARQ_CHECK_ARG(x_dtype >= 0 && x_dtype <= 2, "quant_pack_rows: bad dtype %d", x_dtype);
-  VARQ_CHECK_ARG(n_rows >= 0 && c > 0, "quant_pack_rows: bad shape");
-  VARQ_CHECK_ARG(c % 8 == 0 && (c * bits) % 32 == 0, "quant_pack_rows: c=%d must be a multiple of 8 and fill whole words", c);
-  VARQ_CHECK_ARG(group > 0 && group % 8 == 0 && c % group == 0, "quant_pack_rows: group=%d must be a multiple of 8 dividing c=%d", group, c);
+static int quant_pack_rows_launch(const char *who, const void *x, const void *x1, int x_dtype, int64_t n_rows, int c,
+                                  int group, int bits, int asym, float eps, const int64_t *host_rowmap,
+                                  const int32_t *slot, int32_t *words, float *scale, float *zp, int32_t *words1,
+                                  float *scale1, float *zp1, void *stream) {
+  const bool two = x1 != nullptr;
+  VARQ_CHECK_ARG(n_rows == 0 || (x && words && scale), "%s: null pointer", who);
+  VARQ_CHECK_ARG(n_rows == 0 || !asym || zp, "%s: asym needs zp output", who);
+  VARQ_CHECK_ARG(n_rows == 0 || !two || (words1 && scale1 && (!asym || zp1)), "%s: outputs of the second tensor missing", who);
+  VARQ_CHECK_ARG(bits == 2 || bits == 4 || bits == 8, "%s: bits must be 2, 4 or 8 (got %d)", who, bits);
+  VARQ_CHECK_ARG(x_dtype >= 0 && x_dtype <= 2, "%s: bad dtype %d", who, x_dtype);
+  VARQ_CHECK_ARG(n_rows >= 0 && c > 0, "%s: bad shape", who);
+  VARQ_CHECK_ARG(c % 8 == 0 && (c * bits) % 32 == 0, "%s: c=%d must be a multiple of 8 and fill whole words", who, c);
+  VARQ_CHECK_ARG(group > 0 && group % 8 == 0 && c % group == 0, "%s: group=%d must be a multiple of 8 dividing c=%d", who, group, c);
   const int lpg = group / 8;
-  VARQ_CHECK_ARG(varq_log2_exact(lpg) >= 0 && lpg <= 64, "quant_pack_rows: group/8=%d must be a power of two <= 64 (group <= 512)", lpg);
+  VARQ_CHECK_ARG(varq_log2_exact(lpg) >= 0 && lpg <= 64, "%s: group/8=%d must be a power of two <= 64 (group <= 512)", who, lpg);
   RowMap m = varq_rowmap_from_host(host_rowmap, n_rows);
-  VARQ_CHECK_ARG(m.n0 >= 0 && m.n1 >= 0 && m.n2 >= 0 && m.n0 * m.n1 * m.n2 == n_rows, "quant_pack_rows: row map does not cover n_rows");
-  VARQ_CHECK_ARG(m.slot_dim >= -1 && m.slot_dim <= 2 && (m.slot_dim < 0 || slot), "quant_pack_rows: slot table missing");
+  VARQ_CHECK_ARG(m.n0 >= 0 && m.n1 >= 0 && m.n2 >= 0 && m.n0 * m.n1 * m.n2 == n_rows, "%s: row map does not cover n_rows", who);
+  VARQ_CHECK_ARG(m.slot_dim >= -1 && m.slot_dim <= 2 && (m.slot_dim < 0 || slot), "%s: slot table missing", who);
   if (n_rows == 0) return VARQ_OK;
 
   RowsParams p;
   p.x = x; p.words = words; p.scale = scale; p.zp = zp; p.slot = slot; p.map = m;
+  p.x1 = x1; p.words1 = words1; p.scale1 = scale1; p.zp1 = zp1;
   p.c8 = c / 8;
   p.c8_shift = varq_log2_exact(p.c8);
   p.nseg = c / group;
   p.eps = eps;
   p.octets_per_pair = m.n2 * p.c8;
   p.blocks_per_pair = (p.octets_per_pair + 255) / 256;
-  VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 256, "quant_pack_rows: more than 2^31 octets per (i0,i1) pair");
-  VARQ_CHECK_ARG(m.n1 <= 65535 && m.n0 <= 65535, "quant_pack_rows: n0 and n1 of the row map must be <= 65535");
-  dim3 grid((unsigned)p.blocks_per_pair, (unsigned)m.n1, (unsigned)m.n0);
+  VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 256, "%s: more than 2^31 octets per (i0,i1) pair", who);
+  VARQ_CHECK_ARG(m.n1 <= 65535 && m.n0 * (two ? 2 : 1) <= 65535, "%s: n0 (times the number of tensors) and n1 of the row map must be <= 65535", who);
+  dim3 grid((unsigned)p.blocks_per_pair, (unsigned)m.n1, (unsigned)(m.n0 * (two ? 2 : 1)));
   hipStream_t st = (hipStream_t)stream;
   int rc = -1;
   if (x_dtype == VARQ_F32) rc = launch_dt<VARQ_F32>(p, bits, asym, lpg, grid, st);
   else if (x_dtype == VARQ_BF16) rc = launch_dt<VARQ_BF16>(p, bits, asym, lpg, grid, st);
   else rc = launch_dt<VARQ_F16>(p, bits, asym, lpg, grid, st);
-  if (rc) return varq_set_error(VARQ_ERR_UNSUPPORTED, "quant_pack_rows: no kernel for this configuration");
-  VARQ_CHECK_LAUNCH("quant_pack_rows");
+  if (rc) return varq_set_error(VARQ_ERR_UNSUPPORTED, "%s: no kernel for this configuration", who);
+  VARQ_CHECK_LAUNCH(who);
   return VARQ_OK;
+}
+
+extern "C" int varq_quant_pack_rows(const void *x, int x_dtype, int64_t n_rows, int c, int group, int bits,
+                                    int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
+                                    int32_t *words, float *scale, float *zp, void *stream) {
+  return quant_pack_rows_launch("quant_pack_rows", x, nullptr, x_dtype, n_rows, c, group, bits, asym, eps, host_rowmap, slot,
+                                words, scale, zp, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int varq_quant_pack_rows2(const void *x0, const void *x1, int x_dtype, int64_t n_rows, int c, int group,
+                                     int bits, int asym, float eps, const int64_t *host_rowmap, const int32_t *slot,
+                                     int32_t *words0, float *scale0, float *zp0, int32_t *words1, float *scale1,
+                                     float *zp1, void *stream) {
+  VARQ_CHECK_ARG(n_rows == 0 || x1, "quant_pack_rows2: null pointer");
+  return quant_pack_rows_launch("quant_pack_rows2", x0, x1, x_dtype, n_rows, c, group, bits, asym, eps, host_rowmap, slot,
+                                words0, scale0, zp0, words1, scale1, zp1, stream);
 }

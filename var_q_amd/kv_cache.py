@@ -131,10 +131,15 @@ class PackedKVCache:
             else:
                 rowmap = [B, n, H, hc * self.Lmax, 1, self.Lmax, self.len, 2]
             asym = not self.symmetric
-            ops.quant_pack_rows_into(k, self.group, c.bits, asym, self.eps, c.k_words, c.k_scale,
-                                     c.k_zp if asym else None, rowmap, c.slot)
-            ops.quant_pack_rows_into(v, self.group, c.bits, asym, self.eps, c.v_words, c.v_scale,
-                                     c.v_zp if asym else None, rowmap, c.slot)
+            if k.dtype == v.dtype and 2 * rowmap[0] <= 65535:
+                ops.quant_pack_rows_pair_into(k, v, self.group, c.bits, asym, self.eps,
+                                              (c.k_words, c.k_scale, c.k_zp if asym else None),
+                                              (c.v_words, c.v_scale, c.v_zp if asym else None), rowmap, c.slot)
+            else:   # K and V of different dtypes (Infinity: fp32 K after cos-norm, bf16 V)
+                ops.quant_pack_rows_into(k, self.group, c.bits, asym, self.eps, c.k_words, c.k_scale,
+                                         c.k_zp if asym else None, rowmap, c.slot)
+                ops.quant_pack_rows_into(v, self.group, c.bits, asym, self.eps, c.v_words, c.v_scale,
+                                         c.v_zp if asym else None, rowmap, c.slot)
         self.len += n
 
     def append_from_qkv(self, qkv: torch.Tensor, q_scale_mul: Optional[torch.Tensor] = None, l2norm: bool = False,

@@ -79,6 +79,29 @@ def quant_pack_rows_into(x: torch.Tensor, group: int, bits: int, asym: bool, eps
               'varq_quant_pack_rows')
 
 
+def quant_pack_rows_pair_into(x0: torch.Tensor, x1: torch.Tensor, group: int, bits: int, asym: bool, eps: float,
+                              out0: Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]],
+                              out1: Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]],
+                              rowmap: Sequence[int], slot: Optional[torch.Tensor] = None) -> None:
+    """Two tensors of one shape and dtype (K and V of a cache step) in one launch; out0 / out1
+    = (words, scale, zp) buffers of each, addressed through the shared row map."""
+    _gpu(x0, 'x0'); _gpu(x1, 'x1')
+    assert x0.shape == x1.shape and x0.dtype == x1.dtype and x0.is_contiguous() and x1.is_contiguous()
+    for w, s, z in (out0, out1):
+        _gpu(w, 'words'); _gpu(s, 'scale')
+        assert w.is_contiguous() and s.is_contiguous() and w.dtype == torch.int32 and s.dtype == torch.float32
+    c = x0.shape[-1]
+    n_rows = x0.numel() // c
+    assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
+    lib = _lib.load()
+    with torch.cuda.device(x0.device):
+        check(lib.varq_quant_pack_rows2(x0.data_ptr(), x1.data_ptr(), _dt(x0), n_rows, c, group, bits, int(asym), eps,
+                                        i64arr(rowmap), _ptr(slot),
+                                        out0[0].data_ptr(), out0[1].data_ptr(), _ptr(out0[2]),
+                                        out1[0].data_ptr(), out1[1].data_ptr(), _ptr(out1[2]), _stream(x0)),
+              'varq_quant_pack_rows2')
+
+
 # ---------------------------------------------------------------------------
 # general (cross-row groups) quantize + pack
 # ---------------------------------------------------------------------------
