@@ -52,6 +52,28 @@ def test_incremental_schedule(dev, mixed):
     assert cache.len == L
 
 
+def test_classes_on_side_streams_equal_one_stream(dev):
+    """attend() of a mixed-width cache launches its bit-width classes on one stream each;
+    the result is the one-stream result bit for bit, also when the caller's stream goes
+    straight on to overwrite the inputs."""
+    B, H, D, L = 2, 6, 128, 700
+    gen = torch.Generator().manual_seed(77)
+    cache = PackedKVCache(B, H, L, D, [2, 4, 8, 8, 4, 2], 64, dev)
+    k, v = (torch.randn(B, H, L, D, generator=gen).bfloat16().to(dev) for _ in range(2))
+    q = torch.randn(B, H, 300, D, generator=gen).bfloat16().to(dev)
+    cache.append(k, v)
+    outs = {}
+    for mode in (False, True, True):
+        cache.concurrent_classes = mode
+        note('kv cache attend, side streams', mode)
+        qq = q.clone()
+        o = cache.attend(qq, 0.09)
+        qq.zero_()                       # ordered after all classes on the caller's stream
+        outs.setdefault(mode, []).append(o)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[False][0], outs[True][0]) and torch.equal(outs[True][0], outs[True][1])
+
+
 def test_overflow_is_refused(dev):
     cache = PackedKVCache(1, 2, 4, 64, 4, 64, dev)
     x = torch.randn(1, 2, 3, 64, device=dev).bfloat16()

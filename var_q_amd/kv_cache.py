@@ -38,6 +38,8 @@ class PackedKVCache:
         self.B, self.H, self.Lmax, self.D, self.group = B, H, Lmax, D, group_size
         self.per_head_bits, self.symmetric, self.eps = per_head, symmetric, eps
         self.len = 0
+        self.concurrent_classes = True   # attend(): one stream per bit-width class
+        self._side = self._fork = self._join = None
         self.classes: List[_BitClass] = [
             _BitClass(b, [h for h in range(H) if per_head[h] == b], B, H, Lmax, D, group_size, device)
             for b in sorted(set(per_head))]
@@ -171,12 +173,36 @@ class PackedKVCache:
         if out is None:
             out = torch.empty_like(q)
         asym = not self.symmetric
-        for c in self.classes:
-            ops.fused_attn(q, c.k_words, c.k_scale, c.k_zp if asym else None,
-                           c.v_words, c.v_scale, c.v_zp if asym else None,
-                           c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
-                           head_map=c.head_map if len(self.classes) > 1 else None, out=out)
+        many = len(self.classes) > 1
+        main = torch.cuda.current_stream(q.device)
+        side = self._side_streams(q.device) if many and self.concurrent_classes else None
+        if side:
+            self._fork.record(main)
+        for i, c in enumerate(self.classes):
+            # classes cover disjoint heads and disjoint rows of `out`: with side streams their
+            # launches share the GPU instead of queueing behind each other half-empty
+            stream = side[i - 1] if side and i else main
+            if stream is not main:
+                stream.wait_event(self._fork)
+            with torch.cuda.stream(stream):
+                ops.fused_attn(q, c.k_words, c.k_scale, c.k_zp if asym else None,
+                               c.v_words, c.v_scale, c.v_zp if asym else None,
+                               c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
+                               head_map=c.head_map if many else None, out=out)
+            if stream is not main:
+                self._join[i - 1].record(stream)
+                main.wait_event(self._join[i - 1])
         return out
+
+    def _side_streams(self, device):
+        """One extra stream (default priority) per bit-width class beyond the first, with the
+        events that order them after and before the caller's stream."""
+        if self._side is None:
+            n = len(self.classes) - 1
+            self._side = [torch.cuda.Stream(device=device) for _ in range(n)]
+            self._fork = torch.cuda.Event()
+            self._join = [torch.cuda.Event() for _ in range(n)]
+        return self._side
 
     def dequant(self, which: str = 'k', out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
         """Dequantized [B,H,len,D] copy of the cached K or V (for checking)."""
