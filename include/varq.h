@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 1
+#define VARQ_ABI_VERSION 2
 
 enum varq_status {
   VARQ_OK = 0,
@@ -147,15 +147,28 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *   kv_limit   device int32 [Lq]: query i sees keys j < kv_limit[i]
  *              (block-causal next-scale mask of VAR/models/var.py:110-114,
  *              limit = end of the query's own scale); NULL = all Lk visible.
+ *   workspace, workspace_bytes, splits
+ *              A launch with few query blocks over a long cache (a small batch, a
+ *              step of a few hundred queries) leaves compute units idle or ends in a
+ *              short last round.  The keys of each query block can be shared out over
+ *              up to 8 workgroups; their partial results (fp32) pass through the
+ *              workspace and a second kernel combines them.  splits = 0: the library
+ *              decides, and uses no more shares than the workspace holds (none
+ *              without a workspace); 1: never; 2..8: exactly that many (an error if
+ *              the workspace is too small).  varq_fused_attn_workspace_bytes gives the
+ *              size for a shape (0 when the library would not share the keys out);
+ *              device memory, 16-byte aligned, used only during the call's kernels.
  * Requires D in {64,128}, bits in {2,4,8}, k_group/v_group in {32,64,128}
  * dividing D.
  */
+size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk, int D, int nseg, int splits);
 int varq_fused_attn(const void *q, void *out,
                     const int32_t *k_words, const float *k_scale, const float *k_zp, int k_bits, int k_group,
                     const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                     int B, int Hq, int Hkv, const int32_t *head_map,
                     int Lq, int Lk, int Lk_stride, int D,
-                    const int32_t *kv_limit, float softmax_scale, void *stream);
+                    const int32_t *kv_limit, float softmax_scale,
+                    void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*
  * The same attention over a cache quantized per (head, channel), the layout of the
@@ -181,7 +194,8 @@ int varq_fused_attn_channel(const void *q, void *out,
                             int nseg, const int32_t *host_seg_end,
                             int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                             int Lq, int Lk, int Lk_stride, int D,
-                            const int32_t *kv_limit, float softmax_scale, void *stream);
+                            const int32_t *kv_limit, float softmax_scale,
+                            void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*
  * Producer side of the quantized cache in one pass (an extension: the reference does

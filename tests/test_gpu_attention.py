@@ -56,7 +56,7 @@ def _compare(out, ref, exact, what=''):
     assert err <= 2e-2 * span + e_ref, f'{what}: max-abs {err} vs oracle (oracle itself {e_ref} from fp64, range {span})'
 
 
-def _run(dev, B, H, Lq, Lk, D, bits, gk, gv, seed, kv_limit=None, bias=None, dist='normal', what=''):
+def _run(dev, B, H, Lq, Lk, D, bits, gk, gv, seed, kv_limit=None, bias=None, dist='normal', what='', splits=0):
     g = torch.Generator().manual_seed(seed)
     k = O.synth_kv((B, H, Lk, D), seed + 1, dist).bfloat16()
     v = O.synth_kv((B, H, Lk, D), seed + 2, dist).bfloat16()
@@ -64,9 +64,9 @@ def _run(dev, B, H, Lq, Lk, D, bits, gk, gv, seed, kv_limit=None, bias=None, dis
     kw, ks, kz, kd = _quantize(k, gk, bits)
     vw, vs, vz, vd = _quantize(v, gv, bits)
     scale = 1.0 / math.sqrt(D)
-    note('fused_attn', what, (B, H, Lq, Lk, D), bits, gk, gv)
+    note('fused_attn', what, (B, H, Lq, Lk, D), bits, gk, gv, 'splits', splits)
     out = ops.fused_attn(q.to(dev), kw.to(dev), ks.to(dev), kz.to(dev), vw.to(dev), vs.to(dev), vz.to(dev),
-                         bits, bits, Lk, scale, kv_limit=None if kv_limit is None else kv_limit.to(dev))
+                         bits, bits, Lk, scale, kv_limit=None if kv_limit is None else kv_limit.to(dev), splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, kd, vd, scale, bias)
     _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what)

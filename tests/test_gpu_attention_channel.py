@@ -27,7 +27,7 @@ def _quantize_channel(x, bits, asym, dims=(0, 2)):
     return O.pack_last_dim(q, bits)[0], table(s), table(z), deq
 
 
-def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist='normal', dims=(0, 2), what=''):
+def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist='normal', dims=(0, 2), what='', splits=0):
     g = torch.Generator().manual_seed(seed)
     k = O.synth_kv((B, H, Lk, D), seed + 1, dist).bfloat16()
     v = O.synth_kv((B, H, Lk, D), seed + 2, dist).bfloat16()
@@ -35,12 +35,12 @@ def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist=
     kw, ks, kz, kd = _quantize_channel(k, bits, asym, dims)
     vw, vs, vz, vd = _quantize_channel(v, bits, asym, dims)
     scale = 1.0 / math.sqrt(D)
-    note('fused_attn_channel', what, (B, H, Lq, Lk, D), bits, asym)
+    note('fused_attn_channel', what, (B, H, Lq, Lk, D), bits, asym, 'splits', splits)
     # one table: the zero-point of K cancels, so it is passed in one case of two only
     kz_arg = None if (kz is None or seed % 2) else kz.to(dev)
     out = ops.fused_attn_channel(q.to(dev), kw.to(dev), ks.to(dev), kz_arg, vw.to(dev), vs.to(dev),
                                  None if vz is None else vz.to(dev), bits, Lk, scale,
-                                 kv_limit=None if kv_limit is None else kv_limit.to(dev))
+                                 kv_limit=None if kv_limit is None else kv_limit.to(dev), splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, kd, vd, scale, bias)
     _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what)
@@ -108,7 +108,7 @@ def test_head_subset_and_device_quantizer(dev):
     assert bool((out[:, untouched] == 7.0).all()), 'rows of heads outside the map were written'
 
 
-def _stepwise(dev, B, H, D, steps, bits, asym, Lq, seed, masked=False, what='', outlier_mul=15.0):
+def _stepwise(dev, B, H, D, steps, bits, asym, Lq, seed, masked=False, what='', outlier_mul=15.0, splits=0):
     """A cache filled step by step: every step is quantized on its own with one (scale, zp)
     per (head, channel), as the reference's append methods do (VAR_Q/quant.py:140-201 for the
     symmetric case, run here through the oracle's state machine)."""
@@ -145,11 +145,11 @@ def _stepwise(dev, B, H, D, steps, bits, asym, Lq, seed, masked=False, what='', 
         level_end = torch.tensor([e for e, n in zip(ends, steps) for _ in range(n)], dtype=torch.int32)
         lim = level_end[L - Lq:].contiguous()
         bias = torch.where(torch.arange(L)[None, :] < lim[:, None].long(), 0.0, float('-inf'))[None, None]
-    note('fused_attn_channel', what, (B, H, Lq, L, D), bits, asym, steps)
+    note('fused_attn_channel', what, (B, H, Lq, L, D), bits, asym, steps, 'splits', splits)
     out = ops.fused_attn_channel(q.to(dev), packed[0].to(dev), tables[0][0].to(dev),
                                  None if not asym else tables[0][1].to(dev), packed[1].to(dev),
                                  tables[1][0].to(dev), None if not asym else tables[1][1].to(dev), bits, L, scale,
-                                 kv_limit=None if lim is None else lim.to(dev), seg_ends=ends)
+                                 kv_limit=None if lim is None else lim.to(dev), seg_ends=ends, splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, deq[0], deq[1], scale, bias)
     _compare(out, ref, _exact_fp64(q, deq[0], deq[1], scale, bias, dev), what)

@@ -62,6 +62,7 @@ def test_classes_on_side_streams_equal_one_stream(dev):
     k, v = (torch.randn(B, H, L, D, generator=gen).bfloat16().to(dev) for _ in range(2))
     q = torch.randn(B, H, 300, D, generator=gen).bfloat16().to(dev)
     cache.append(k, v)
+    cache.splits = 1     # (on one stream the library would share the keys out; same arithmetic wanted here)
     outs = {}
     for mode in (False, True, True):
         cache.concurrent_classes = mode

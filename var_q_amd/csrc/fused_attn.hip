@@ -77,6 +77,12 @@ struct AttnParams {
   int B, Hq, Hkv, Lq, Lk, Lstride;
   int q_tiles, bh_total;
   float scale_log2e;
+  // the keys of a query block may be shared out over nsplit workgroups; each leaves its
+  // normalized output (fp32 [nsplit][B*Hkv*Lq][D]) and softmax statistics (reference,
+  // denominator: fp32 [nsplit][B*Hkv*Lq][2]) for the combining kernel.  nsplit = 1: no
+  // workspace, the output is written directly.
+  int nsplit;
+  float *ws_o, *ws_ml;
 };
 
 __device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
@@ -300,7 +306,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // (batch, head) are given ids of one residue class to keep its packed K/V in
   // that XCD's L2.
   const int wg = blockIdx.x;
-  const int xcd = wg & 7, slot = wg >> 3;
+  const int xcd = wg & 7, slot_s = wg >> 3;
+  const int split = p.nsplit > 1 ? slot_s % p.nsplit : 0;
+  const int slot = p.nsplit > 1 ? slot_s / p.nsplit : slot_s;
   const int bh = (slot / p.q_tiles) * 8 + xcd;
   const int qt = slot % p.q_tiles;
   if (bh >= p.bh_total) return;
@@ -421,7 +429,19 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       c.start += BN;
     }
   };
-  TileCursor cur_k{0, 0}, cur_v{0, 0}, cur_a{0, 0};
+  TileCursor cur_k{0, 0};
+  if (p.nsplit > 1) {
+    // this workgroup's share of the tiles: [t_begin, t_end) of the block's tile sequence
+    const int t_begin = n_tiles * split / p.nsplit, t_end = n_tiles * (split + 1) / p.nsplit;
+    if constexpr (CHAN) {
+      for (int i = 0; i < t_begin; ++i) cursor_advance(cur_k);
+    } else {
+      cur_k.start = t_begin * BN;
+    }
+    n_tiles = t_end - t_begin;
+  }
+  TileCursor cur_v = cur_k, cur_a = cur_k;
+  const int tile_base = cur_k.start;   // first key of this workgroup's tiles
   int wave_minlim = q_live ? limit : p.Lk;
   for (int off = 1; off < 64; off <<= 1) wave_minlim = min(wave_minlim, __shfl_xor(wave_minlim, off, 64));
 
@@ -608,7 +628,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     }
     __syncthreads();
   }
-  load_q(0);   // behind the first tile's requests, so the two latencies overlap
+  load_q(cur_a.seg);   // behind the first tile's requests, so the two latencies overlap
   if (n_tiles > 0) { stage(0); widen_k(0); }
   if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
@@ -646,7 +666,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 
   // per-channel tables: segment of the tile being attended, end of the tile's keys, and the
   // softmax denominator as it was when the current segment began
-  int seg_a = 0, tile_end = 0;
+  int seg_a = cur_a.seg, tile_end = 0;
   float l_prev = 0.f;
   // A new segment begins.  The true (unnormalized) output is, per channel,
   //   sv * (kMul * oacc - rq - zv * (l_sum - l_prev))
@@ -693,7 +713,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       if (__builtin_expect(cur_a.seg != seg_a, 0)) segment_boundary(cur_a.seg);
       cursor_advance(cur_a);
     } else {
-      t0 = tile * BN;
+      t0 = tile_base + tile * BN;
     }
     kx = lds_kx + (tile & 1) * BN * KXS;
     par = lds_par + (tile % 3) * L::kParFloats;
@@ -908,6 +928,12 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   for (int s = 0; s < NSV; ++s) rq[s] = __shfl(racc[s], col, 64) + r_run[s];
   if (q_live) {
     __bf16 *optr = p.out + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow) * D;
+    // with the keys shared out: the normalized fp32 output and (reference, denominator) of
+    // this share, for the combining kernel
+    const bool shared_out = p.nsplit > 1;
+    const int64_t prow = ((int64_t)split * p.bh_total + bh) * p.Lq + qrow;
+    float *wptr = p.ws_o + prow * D;
+    if (shared_out && half == 0) *reinterpret_cast<float2 *>(p.ws_ml + prow * 2) = make_float2(m_ref, l_sum);
 #pragma unroll
     for (int d = 0; d < NDB; ++d) {
       constexpr int DBS = GV / 32;
@@ -928,11 +954,47 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
           o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
           o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
         }
-        uint2 v = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
-        *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = v;
+        if (shared_out) {
+          *reinterpret_cast<float4 *>(wptr + d * 32 + 8 * g4 + 4 * half) = make_float4(o0, o1, o2, o3);
+        } else {
+          uint2 v = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
+          *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = v;
+        }
       }
     }
   }
+}
+
+// One thread per (query row, four channels): the shares' outputs weighted by their softmax
+// mass l * 2^(m - M), M the largest reference among the shares that saw a key.
+template <int D>
+__global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
+  const int64_t rows = (int64_t)p.bh_total * p.Lq;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = item / (D / 4);
+  const int c0 = (int)(item % (D / 4)) * 4;
+  if (row >= rows) return;
+  float m_max = -INFINITY;
+  for (int s = 0; s < p.nsplit; ++s) {
+    const float2 ml = *reinterpret_cast<const float2 *>(p.ws_ml + ((int64_t)s * rows + row) * 2);
+    if (ml.y > 0.f) m_max = fmaxf(m_max, ml.x);
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, wsum = 0.f;
+  for (int s = 0; s < p.nsplit; ++s) {
+    const float2 ml = *reinterpret_cast<const float2 *>(p.ws_ml + ((int64_t)s * rows + row) * 2);
+    if (!(ml.y > 0.f)) continue;
+    const float w = ml.y * __builtin_amdgcn_exp2f(ml.x - m_max);
+    const float4 o = *reinterpret_cast<const float4 *>(p.ws_o + ((int64_t)s * rows + row) * D + c0);
+    acc[0] = __builtin_fmaf(w, o.x, acc[0]); acc[1] = __builtin_fmaf(w, o.y, acc[1]);
+    acc[2] = __builtin_fmaf(w, o.z, acc[2]); acc[3] = __builtin_fmaf(w, o.w, acc[3]);
+    wsum += w;
+  }
+  const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+  const int bh = (int)(row / p.Lq), qrow = (int)(row % p.Lq);
+  const int b = bh / p.Hkv, hs = bh % p.Hkv;
+  const int hq = p.head_map ? p.head_map[hs] : hs;
+  __bf16 *optr = p.out + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow) * D + c0;
+  *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_bf16_rne(acc[0] * inv, acc[1] * inv), pack_bf16_rne(acc[2] * inv, acc[3] * inv));
 }
 
 template <int D, int BITS, int GK, int GV, bool CHAN = false>
@@ -946,8 +1008,12 @@ void launch(const AttnParams &p, hipStream_t st) {
     configured = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
-  dim3 grid((unsigned)(bh_pad * p.q_tiles));
+  dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
   hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN>), grid, dim3(NT), lds_bytes, st, p);
+  if (p.nsplit > 1) {
+    const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
+    hipLaunchKernelGGL((combine_splits_kernel<D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
+  }
 }
 
 template <int D, int BITS>
@@ -964,14 +1030,84 @@ int dispatch_groups(const AttnParams &p, int gk, int gv, hipStream_t st) {
   return -1;
 }
 
+// ---- sharing the keys of a query block out over several workgroups ---------------------
+constexpr int kMaxSplits = 8;
+
+int device_cus() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cus[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+
+size_t split_workspace_bytes(int splits, int64_t rows, int D) {
+  return splits > 1 ? (size_t)splits * (size_t)rows * (size_t)(D + 2) * sizeof(float) : 0;
+}
+
+// The split count that minimizes a launch's modelled time: workgroups run one per compute
+// unit in rounds; a workgroup costs its tiles plus a fixed prologue and epilogue; shares
+// cost a second pass over fp32 partial outputs.  Few query blocks on a long cache gain,
+// a grid that already fills the device in whole rounds does not.
+int choose_splits(int64_t wgs, int tiles, int64_t rows, int D) {
+  const double cus = device_cus();
+  const double tile_us = D == 128 ? 2.3 : 1.4, fixed_us = 9.0;
+  double base = 0.0, best = 0.0;
+  int best_s = 1;
+  for (int s = 1; s <= kMaxSplits; ++s) {
+    if (s > 1 && tiles / s < 2) break;
+    const double rounds = (double)((wgs * s + (int64_t)cus - 1) / (int64_t)cus);
+    double t = rounds * ((double)((tiles + s - 1) / s) * tile_us + fixed_us);
+    if (s > 1) t += 4.0 + 2.0 * (double)split_workspace_bytes(s, rows, D) / 4.0e6;   // 4 TB/s, in us
+    if (s == 1) base = best = t;
+    else if (t < 0.9 * base && t < best) { best = t; best_s = s; }   // sharing must gain a tenth
+  }
+  return best_s;
+}
+
+// Fills the split fields of p from the caller's request.  splits: 0 = as the model above
+// says, reduced to what the workspace holds; 1 = none; 2..8 = exactly that many.
+int set_splits(AttnParams &p, int D, int tiles, int splits, void *workspace, size_t workspace_bytes, const char *who) {
+  p.nsplit = 1; p.ws_o = nullptr; p.ws_ml = nullptr;
+  if (splits < 0 || splits > kMaxSplits)
+    return varq_set_error(VARQ_ERR_INVALID, "%s: splits must be 0 (automatic) or 1..%d (got %d)", who, kMaxSplits, splits);
+  const int64_t rows = (int64_t)p.bh_total * p.Lq;
+  int n = splits ? splits : choose_splits((int64_t)p.bh_total * p.q_tiles, tiles, rows, D);
+  if (splits > 1 && (!workspace || workspace_bytes < split_workspace_bytes(n, rows, D)))
+    return varq_set_error(VARQ_ERR_INVALID, "%s: %d splits need a workspace of %zu bytes (got %zu)", who, n,
+                          split_workspace_bytes(n, rows, D), workspace ? workspace_bytes : (size_t)0);
+  while (n > 1 && (!workspace || workspace_bytes < split_workspace_bytes(n, rows, D))) --n;
+  if (n <= 1) return VARQ_OK;
+  if ((uintptr_t)workspace & 15) return varq_set_error(VARQ_ERR_INVALID, "%s: the workspace must be 16-byte aligned", who);
+  if ((int64_t)((p.bh_total + 7) / 8 * 8) * p.q_tiles * n >= (1ll << 31))
+    return varq_set_error(VARQ_ERR_INVALID, "%s: grid too large for %d splits", who, n);
+  p.nsplit = n;
+  p.ws_o = reinterpret_cast<float *>(workspace);
+  p.ws_ml = p.ws_o + (size_t)n * (size_t)rows * (size_t)D;
+  return VARQ_OK;
+}
+
 }  // namespace
+
+extern "C" size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk, int D, int nseg, int splits) {
+  if (B <= 0 || Hkv <= 0 || Lq <= 0 || Lk <= 0 || (D != 64 && D != 128) || splits < 0 || splits > kMaxSplits) return 0;
+  const int64_t rows = (int64_t)B * Hkv * Lq;
+  const int tiles = (Lk + BN - 1) / BN + (nseg > 1 ? nseg - 1 : 0);
+  const int n = splits ? splits : choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), tiles, rows, D);
+  return split_workspace_bytes(n, rows, D);
+}
 
 extern "C" int varq_fused_attn(const void *q, void *out,
                                const int32_t *k_words, const float *k_scale, const float *k_zp, int k_bits, int k_group,
                                const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                                int B, int Hq, int Hkv, const int32_t *head_map,
                                int Lq, int Lk, int Lk_stride, int D,
-                               const int32_t *kv_limit, float softmax_scale, void *stream) {
+                               const int32_t *kv_limit, float softmax_scale,
+                               void *workspace, size_t workspace_bytes, int splits, void *stream) {
   VARQ_CHECK_ARG(q && out && k_words && v_words && k_scale && v_scale, "fused_attn: null pointer");
   VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn: bad sizes");
   VARQ_CHECK_ARG(head_map || Hkv == Hq, "fused_attn: Hkv != Hq needs a head map");
@@ -1001,6 +1137,7 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn")) return e;
   hipStream_t st = (hipStream_t)stream;
   int rc = -1;
   if (D == 128) {
@@ -1025,7 +1162,8 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
                                        int nseg, const int32_t *host_seg_end,
                                        int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                                        int Lq, int Lk, int Lk_stride, int D,
-                                       const int32_t *kv_limit, float softmax_scale, void *stream) {
+                                       const int32_t *kv_limit, float softmax_scale,
+                                       void *workspace, size_t workspace_bytes, int splits, void *stream) {
   VARQ_CHECK_ARG(q && out && k_words && v_words && k_chan_scale && v_chan_scale, "fused_attn_channel: null pointer");
   VARQ_CHECK_ARG(nseg >= 1 && nseg <= kMaxSegments, "fused_attn_channel: nseg must be 1..%d (got %d)", kMaxSegments, nseg);
   VARQ_CHECK_ARG(nseg == 1 || host_seg_end, "fused_attn_channel: segment ends missing");
@@ -1066,6 +1204,8 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  if (int e = set_splits(p, D, (Lk + BN - 1) / BN + nseg - 1, splits, workspace, workspace_bytes, "fused_attn_channel"))
+    return e;
   hipStream_t st = (hipStream_t)stream;
   if (D == 128) {
     if (bits == 4) launch<128, 4, 128, 128, true>(p, st);

@@ -39,6 +39,7 @@ class PackedKVCache:
         self.per_head_bits, self.symmetric, self.eps = per_head, symmetric, eps
         self.len = 0
         self.concurrent_classes = True   # attend(): one stream per bit-width class
+        self.splits = 0                  # attend() on one stream: shares of a query block's keys (0 = library's choice)
         self._side = self._fork = self._join = None
         self.classes: List[_BitClass] = [
             _BitClass(b, [h for h in range(H) if per_head[h] == b], B, H, Lmax, D, group_size, device)
@@ -188,7 +189,8 @@ class PackedKVCache:
                 ops.fused_attn(q, c.k_words, c.k_scale, c.k_zp if asym else None,
                                c.v_words, c.v_scale, c.v_zp if asym else None,
                                c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
-                               head_map=c.head_map if many else None, out=out)
+                               head_map=c.head_map if many else None, out=out,
+                               splits=1 if side else self.splits)   # classes side by side fill the device already
             if stream is not main:
                 self._join[i - 1].record(stream)
                 main.wait_event(self._join[i - 1])
