@@ -59,6 +59,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
 
 constexpr int kMaxSegments = 16;
+constexpr int kChanTableRows = 5;   // LDS rows per segment of the per-channel tables
 
 struct AttnParams {
   const __bf16 *q;
@@ -292,9 +293,12 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   uint16_t *const lds_wz = reinterpret_cast<uint16_t *>(lds_raw + L::kWz);
   float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
   int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
-  // CHAN: the tables of this head for every segment, [nseg][4][D] fp32: K scale, K zero-point,
-  // V scale, V zero-point (zeros where a table is absent); filled once in the prologue
+  // CHAN: the tables of this head for every segment, [nseg][5][D] fp32: K scale, K zero-point,
+  // V scale, V zero-point (zeros where a table is absent) and the ratio of the V scales of the
+  // previous segment and this one; filled once in the prologue
   float *const lds_tab = reinterpret_cast<float *>(lds_raw + (L::kBytes + 15) / 16 * 16);
+  constexpr int TR = kChanTableRows;   // rows per segment: K scale, K zero-point, V scale, V zero-point, sv(seg-1)/sv(seg)
+  const bool k_affine = CHAN && p.k_chan_zp != nullptr, v_affine = CHAN && p.v_chan_zp != nullptr;   // (uniform)
   constexpr int KXS = L::KXS, RSV = L::RSV;
   // parameter block of one tile: ck [NSK][BN]; vr [NSV][BN]; sv [NSV][BN] unless folded
   constexpr bool FOLD_SV = L::kFoldSv;
@@ -349,13 +353,11 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       const int oct = k_octet<GK>(ch, half);
       // the octet's eight channels in one 16-byte load, then into the codec's slot order
       const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
-      float sk[8], zk[8];
+      float sk[8];
       if constexpr (CHAN) {
-        const float *tk = lds_tab + (seg * 4 + 0) * D + oct * 8, *tz = lds_tab + (seg * 4 + 1) * D + oct * 8;
+        const float *tk = lds_tab + (seg * TR + 0) * D + oct * 8;
         const float4 s0 = *reinterpret_cast<const float4 *>(tk), s1 = *reinterpret_cast<const float4 *>(tk + 4);
-        const float4 z0 = *reinterpret_cast<const float4 *>(tz), z1 = *reinterpret_cast<const float4 *>(tz + 4);
         sk[0] = s0.x; sk[1] = s0.y; sk[2] = s0.z; sk[3] = s0.w; sk[4] = s1.x; sk[5] = s1.y; sk[6] = s1.z; sk[7] = s1.w;
-        zk[0] = z0.x; zk[1] = z0.y; zk[2] = z0.z; zk[3] = z0.w; zk[4] = z1.x; zk[5] = z1.y; zk[6] = z1.z; zk[7] = z1.w;
       }
 #pragma unroll
       for (int j2 = 0; j2 < 4; ++j2) {
@@ -366,11 +368,20 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
         if constexpr (CHAN) {
           // q[d] * sk[d], rounded to bf16 like any MFMA operand
           pair = pack_bf16_rne(u2f(lo) * sk[d0], u2f(hi) * sk[d1]);
-          zb = __builtin_fmaf(u2f(pair << 16), zk[d0], zb);
-          zb = __builtin_fmaf(u2f(pair & 0xffff0000u), zk[d1], zb);
         }
         qb[ch][j2] = pair;
         qsum[ch / (GK / 16)] += u2f(pair << 16) + u2f(pair & 0xffff0000u);
+      }
+      if (k_affine) {   // the K zero-points against the rounded operands, for the segment's logit constant
+        const float *tz = lds_tab + (seg * TR + 1) * D + oct * 8;
+        const float4 z0 = *reinterpret_cast<const float4 *>(tz), z1 = *reinterpret_cast<const float4 *>(tz + 4);
+        const float zk[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
+#pragma unroll
+        for (int j2 = 0; j2 < 4; ++j2) {
+          const u32 pair = qb[ch][j2];
+          zb = __builtin_fmaf(u2f(pair << 16), zk[KCodec<BITS>::slot_d(2 * j2)], zb);
+          zb = __builtin_fmaf(u2f(pair & 0xffff0000u), zk[KCodec<BITS>::slot_d(2 * j2 + 1)], zb);
+        }
       }
       if constexpr (CHAN) __builtin_amdgcn_sched_barrier(0);   // one chunk's table entries in registers at a time
     }
@@ -624,7 +635,15 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     for (int i = tid; i < p.nseg * 4 * D; i += NT) {
       const int seg = i / (4 * D), which = (i / D) & 3, d = i % D;
       const float *src = which == 0 ? p.k_chan_scale : which == 1 ? p.k_chan_zp : which == 2 ? p.v_chan_scale : p.v_chan_zp;
-      lds_tab[i] = src ? src[((int64_t)seg * p.Hkv + hs) * D + d] : 0.f;
+      lds_tab[(seg * TR + which) * D + d] = src ? src[((int64_t)seg * p.Hkv + hs) * D + d] : 0.f;
+    }
+    __syncthreads();
+    // change of V units at the entry of a segment, per channel (the hardware reciprocal is
+    // accurate to an ulp, which is all a change of units needs)
+    for (int i = tid; i < p.nseg * D; i += NT) {
+      const int seg = i / D, d = i % D;
+      lds_tab[(seg * TR + 4) * D + d] =
+          seg ? lds_tab[((seg - 1) * TR + 2) * D + d] * __builtin_amdgcn_rcpf(lds_tab[(seg * TR + 2) * D + d]) : 1.f;
     }
     __syncthreads();
   }
@@ -683,22 +702,27 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
       const float dl = l_sum - l_prev;
       constexpr float VM = VCodec<BITS>::kMul;
-      const float *sv_old = lds_tab + (seg_a * 4 + 2) * D, *zv_old = lds_tab + (seg_a * 4 + 3) * D;
-      const float *sv_new = lds_tab + (seg_new * 4 + 2) * D;
+      // segments follow one another, so the ratio sv_old / sv_new is the new segment's entry row;
+      // with t = rq / VM and u = (rq + zv_old * dl) / VM the update is ro * (oacc - u) + t
+      const float *zv_old = lds_tab + (seg_a * TR + 3) * D, *ratio = lds_tab + (seg_new * TR + 4) * D;
+      const float t = rq * (1.f / VM), dlm = dl * (1.f / VM);
 #pragma unroll
       for (int d = 0; d < NDB; ++d)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int c0 = d * 32 + 8 * g4 + 4 * half;
-          const float4 so = *reinterpret_cast<const float4 *>(sv_old + c0), sn = *reinterpret_cast<const float4 *>(sv_new + c0);
-          const float4 zo = *reinterpret_cast<const float4 *>(zv_old + c0);
-          // (the hardware reciprocal is accurate to an ulp, which is all a change of units needs)
-          const float ro[4] = {so.x * __builtin_amdgcn_rcpf(sn.x), so.y * __builtin_amdgcn_rcpf(sn.y),
-                               so.z * __builtin_amdgcn_rcpf(sn.z), so.w * __builtin_amdgcn_rcpf(sn.w)};
-          const float zz[4] = {zo.x, zo.y, zo.z, zo.w};
+          const float4 r4 = *reinterpret_cast<const float4 *>(ratio + c0);
+          const float ro[4] = {r4.x, r4.y, r4.z, r4.w};
+          if (v_affine) {
+            const float4 zo = *reinterpret_cast<const float4 *>(zv_old + c0);
+            const float zz[4] = {zo.x, zo.y, zo.z, zo.w};
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
-            oacc[d][4 * g4 + j] = (ro[j] * (VM * oacc[d][4 * g4 + j] - rq - zz[j] * dl) + rq) * (1.f / VM);
+            for (int j = 0; j < 4; ++j)
+              oacc[d][4 * g4 + j] = __builtin_fmaf(ro[j], oacc[d][4 * g4 + j] - __builtin_fmaf(zz[j], dlm, t), t);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) oacc[d][4 * g4 + j] = __builtin_fmaf(ro[j], oacc[d][4 * g4 + j] - t, t);
+          }
           __builtin_amdgcn_sched_barrier(0);   // one slice's registers at a time
         }
       l_prev = l_sum;
@@ -948,8 +972,8 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
           // weighted mean of the codes -> values: sv * (mean - zv * share) per channel, share
           // = the part of the weights that belongs to the current segment (1 without segments)
           const int c0 = d * 32 + 8 * g4 + 4 * half;
-          const float4 sv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * 4 + 2) * D + c0);
-          const float4 zv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * 4 + 3) * D + c0);
+          const float4 sv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 2) * D + c0);
+          const float4 zv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 3) * D + c0);
           const float share = (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
           o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
           o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
@@ -999,7 +1023,7 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
 
 template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
-  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * 4 * D * 4 : 0);
+  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * kChanTableRows * D * 4 : 0);
   static_assert(lds_bytes <= 160 * 1024, "LDS budget");
   static bool configured = false;   // above 64 KiB the limit has to be raised once per process
   if (!configured) {
