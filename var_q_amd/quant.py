@@ -52,6 +52,19 @@ class _Growable:
 
     def __init__(self, dim: int):
         self.dim, self.buf, self.len = dim, None, 0
+        self._pending = []
+
+    def append_later(self, t: torch.Tensor):
+        """Append when the buffer is next looked at.  The cached scales of the reference are
+        each step's scale expanded over the step's tokens (VAR_Q/quant.py:196-201): fp32 per
+        code, four times the bytes of the 8-bit codes themselves; a caller that attends the packed
+        cache through the tables never reads them."""
+        self._pending.append(t)
+
+    def _flush(self):
+        pending, self._pending = self._pending, []
+        for t in pending:
+            self.append(t)
 
     def append(self, t: torch.Tensor):
         n = t.size(self.dim)
@@ -67,9 +80,11 @@ class _Growable:
         self.len += n
 
     def replace(self, t: torch.Tensor):
+        self._pending = []
         self.buf, self.len = t, t.size(self.dim)
 
     def view(self) -> Optional[torch.Tensor]:
+        self._flush()
         return None if self.buf is None else self.buf.narrow(self.dim, 0, self.len)
 
 
@@ -192,9 +207,9 @@ class VAR_Q:
             if self._c_item.dim != self.dim_cat:   # layout was re-assigned before the first step
                 self._reset_cache()
             self._c_item.append(q_cur)
-            self._c_scale.append(s_cur)
+            self._c_scale.append_later(s_cur)
             if z_cur is not None:
-                self._c_zp.append(z_cur)
+                self._c_zp.append_later(z_cur)
             self._note_step(q_cur, replace=False)
         elif m == 'G_HEAD_DIM':
             self._c_item.replace(q_cur)
