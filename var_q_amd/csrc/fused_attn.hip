@@ -43,6 +43,8 @@
 //  * Online softmax in the log2 domain against a reference that is only moved
 //    when some row's maximum exceeds it by 2^16: the common tile needs no
 //    subtraction and no rescale of the output accumulators.
+#include <type_traits>
+
 #include "varq_common.h"
 
 namespace {
@@ -344,7 +346,9 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // p * vs without a multiplication; the other upper slots are zero.
   float qbias = 0.f;   // CHAN: -softmax_scale*log2(e) * sum_d q'[d] zk[d] of the current segment
   // (called from two places: force the inlining, or its captures would live in memory)
-  auto load_q = [&](int seg) __attribute__((always_inline)) {
+  // (pre: the raw values were requested into qb earlier -- the prologue does, to overlap the
+  // trip with its other loads)
+  auto load_q = [&](int seg, auto pre) __attribute__((always_inline)) {
     float qsum[NSK], zb = 0.f;
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
@@ -352,7 +356,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     for (int ch = 0; ch < NCH; ++ch) {
       const int oct = k_octet<GK>(ch, half);
       // the octet's eight channels in one 16-byte load, then into the codec's slot order
-      const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
+      const u32x4_t raw = decltype(pre)::value ? qb[ch] : *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
       float sk[8];
       if constexpr (CHAN) {
         const float *tk = lds_tab + (seg * TR + 0) * D + oct * 8;
@@ -399,11 +403,14 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   };
   // ---- tile range: every lane of the workgroup runs the same number of tiles ----
   __shared__ int lds_maxlim;
-  if (tid == 0) lds_maxlim = 0;
-  __syncthreads();
-  atomicMax(&lds_maxlim, q_live ? limit : 0);
-  __syncthreads();
-  const int kv_end = lds_maxlim;
+  int kv_end = p.Lk;   // without per-query limits every query sees all keys
+  if (p.kv_limit) {
+    if (tid == 0) lds_maxlim = 0;
+    __syncthreads();
+    atomicMax(&lds_maxlim, q_live ? limit : 0);
+    __syncthreads();
+    kv_end = lds_maxlim;
+  }
   int n_tiles = (kv_end + BN - 1) / BN;
   // segment ends in LDS: indexing the kernel arguments with a run-time index would move
   // the whole argument block to scratch memory
@@ -631,6 +638,10 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   if (tid < 3 * RSR) lds_wz[((tid / RSR) * 8 + 7) * RSR + tid % RSR] = 0;   // the all-zero row of each slot
   __syncthreads();
   if (n_tiles > 0) { prefetch_k(0); prefetch(0); }
+  // the query values, behind the first tile's requests and ahead of the table loads: one
+  // round trip for all three
+#pragma unroll
+  for (int ch = 0; ch < NCH; ++ch) qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
   if constexpr (CHAN) {
     for (int i = tid; i < p.nseg * 4 * D; i += NT) {
       const int seg = i / (4 * D), which = (i / D) & 3, d = i % D;
@@ -647,7 +658,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     }
     __syncthreads();
   }
-  load_q(cur_a.seg);   // behind the first tile's requests, so the two latencies overlap
+  load_q(cur_a.seg, std::true_type{});
   if (n_tiles > 0) { stage(0); widen_k(0); }
   if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
@@ -696,7 +707,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     if constexpr (CHAN) {
       // (the Q operands first: with the accumulator arithmetic in front of it the register
       // allocator spills, and spills here cost scratch traffic at every boundary)
-      load_q(seg_new);
+      load_q(seg_new, std::false_type{});
       __builtin_amdgcn_sched_barrier(0);
       const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
