@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 2
+#define VARQ_ABI_VERSION 3
 
 enum varq_status {
   VARQ_OK = 0,
@@ -39,6 +39,9 @@ enum varq_status {
 };
 
 enum varq_dtype { VARQ_F32 = 0, VARQ_BF16 = 1, VARQ_F16 = 2 };
+
+/* K/V tensor layouts of the reference's quantizer (qkv_format, VAR_Q/quant.py:34-37) */
+enum varq_layout { VARQ_LAYOUT_BHLC = 0, VARQ_LAYOUT_BLHC = 1 };
 
 int varq_abi_version(void);
 const char *varq_last_error(void);
@@ -147,6 +150,11 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *   kv_limit   device int32 [Lq]: query i sees keys j < kv_limit[i]
  *              (block-causal next-scale mask of VAR/models/var.py:110-114,
  *              limit = end of the query's own scale); NULL = all Lk visible.
+ *   layout     VARQ_LAYOUT_BHLC: the shapes above.  VARQ_LAYOUT_BLHC: q, out
+ *              [B, Lq, Hq, D], words [B, Lk_stride, Hkv, D*bits/32], scales
+ *              [B, Lk_stride, Hkv, D/group] -- the layout of the reference's
+ *              flash-attention call (VAR/models/basic_var.py:127-131,157-158) and the
+ *              default qkv_format of its quantizer.
  *   workspace, workspace_bytes, splits
  *              A launch with few query blocks over a long cache (a small batch, a
  *              step of a few hundred queries) leaves compute units idle or ends in a
@@ -167,7 +175,7 @@ int varq_fused_attn(const void *q, void *out,
                     const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                     int B, int Hq, int Hkv, const int32_t *head_map,
                     int Lq, int Lk, int Lk_stride, int D,
-                    const int32_t *kv_limit, float softmax_scale,
+                    const int32_t *kv_limit, float softmax_scale, int layout,
                     void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*
@@ -194,7 +202,7 @@ int varq_fused_attn_channel(const void *q, void *out,
                             int nseg, const int32_t *host_seg_end,
                             int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                             int Lq, int Lk, int Lk_stride, int D,
-                            const int32_t *kv_limit, float softmax_scale,
+                            const int32_t *kv_limit, float softmax_scale, int layout,
                             void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*

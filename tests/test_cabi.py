@@ -25,7 +25,7 @@ def test_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
     assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
-    assert lib.varq_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.varq_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_invalid_arguments_are_rejected_on_the_host():
@@ -56,14 +56,14 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert ws >= 3 * 8 * 2 * 4 and ws % (3 * 8 * 4) == 0
     assert lib.varq_quant_workspace_bytes(i64([2, 5, 3, 7]), 0b0011) == 3 * 7 * 2 * 4
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128,
-                             1, 2, 2, None, 16, 16, 16, 96, None, 1.0, None, 0, 0, None)
+                             1, 2, 2, None, 16, 16, 16, 96, None, 1.0, 0, None, 0, 0, None)
     assert rc == -1 and b'D must be' in lib.varq_last_error()
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 8, 128,
-                             1, 2, 2, None, 16, 16, 16, 128, None, 1.0, None, 0, 0, None)
+                             1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, None, 0, 0, None)
     assert rc == -2
     # keys shared out over workgroups: the split count and its workspace are checked first
     tok = lambda splits, ws=None, nbytes=0: lib.varq_fused_attn(
-        fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128, 1, 2, 2, None, 16, 640, 640, 128, None, 1.0,
+        fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128, 1, 2, 2, None, 16, 640, 640, 128, None, 1.0, 0,
         ws, nbytes, splits, None)
     assert tok(9) == -1 and b'splits' in lib.varq_last_error()
     assert tok(2) == -1 and b'workspace' in lib.varq_last_error()
@@ -79,7 +79,7 @@ def test_invalid_arguments_are_rejected_on_the_host():
     # per-channel attention: segment table checks
     i32 = lambda v: (ctypes.c_int32 * len(v))(*v)
     chan = lambda nseg, ends, Lk=16, D=128: lib.varq_fused_attn_channel(
-        fake, fake, fake, fake, None, fake, fake, None, nseg, ends, 8, 1, 2, 2, None, 16, Lk, 16, D, None, 1.0, None, 0, 0, None)
+        fake, fake, fake, fake, None, fake, fake, None, nseg, ends, 8, 1, 2, 2, None, 16, Lk, 16, D, None, 1.0, 0, None, 0, 0, None)
     assert chan(0, None) == -1 and b'nseg' in lib.varq_last_error()
     assert chan(17, None) == -1 and b'nseg' in lib.varq_last_error()
     assert chan(2, None) == -1 and b'segment ends missing' in lib.varq_last_error()
@@ -87,7 +87,7 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert chan(2, i32([40, 16])) == -1 and b'beyond' in lib.varq_last_error()
     assert chan(1, None, D=96) == -1 and b'D must be' in lib.varq_last_error()
     rc = lib.varq_fused_attn_channel(fake, fake, fake, ctypes.c_void_p(0x1004), None, fake, fake, None, 1, None,
-                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, None, 0, 0, None)
+                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, None, 0, 0, None)
     assert rc == -1 and b'aligned' in lib.varq_last_error()
     # empty inputs are a no-op success
     assert chan(1, None, Lk=0) == -1          # queries but no keys

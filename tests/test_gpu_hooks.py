@@ -177,15 +177,17 @@ def test_var_fused_producer_vs_unfused(dev, layout):
 @pytest.mark.parametrize('method,bits,sym', [('G_SCALE_HEAD_DIM', 8, True), ('G_HEAD_DIM', 8, True), ('G_TENSOR', 8, True),
                                              ('G_SCALE', 8, True), ('G_TOKEN', 8, True), ('G_TOKEN_HEAD', 4, True),
                                              ('G_SCALE_HEAD_DIM', 4, False), ('G_HEAD', 8, True)])
-def test_quantizer_backend_vs_dropin(dev, method, bits, sym):
+@pytest.mark.parametrize('layout', ['BHLc', 'BLHc'])
+def test_quantizer_backend_vs_dropin(dev, method, bits, sym, layout):
     """fused='quantizer': the reference's own rules (quantizer + per-step cache as in the
     drop-in) with the attention reading the packed caches, A/B against the drop-in that
     dequantizes the whole cache and calls SDPA.  Both hold the same caches; the outputs
-    differ by the attention arithmetic only."""
+    differ by the attention arithmetic only.  BLHc is the layout of VAR-VAR_Q-8.json and of
+    the reference's flash-attention call, BHLc that of its SDPA call."""
     torch.manual_seed(6)
     C, H = 512, 8
     pn = (1, 2, 3, 4, 5, 6, 8, 10, 13, 16)
-    kw = dict(embed_dim=C, num_heads=H, layout='BHLc', q_bits=bits, quant_method=method, symmetric=sym,
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, q_bits=bits, quant_method=method, symmetric=sym,
               enable_quantization=True, max_tokens=680)
     a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).to(torch.bfloat16)
     b_mod = hooks.VarSelfAttention(0, fused='quantizer', **kw).to(dev).to(torch.bfloat16)
@@ -193,7 +195,7 @@ def test_quantizer_backend_vs_dropin(dev, method, bits, sym):
     a_mod.kv_caching(True)
     b_mod.kv_caching(True)
     for p in pn:
-        note('hooks quantizer backend', method, bits, sym, p)
+        note('hooks quantizer backend', method, bits, sym, layout, p)
         x = torch.randn(2, p * p, C, device=dev, dtype=torch.bfloat16)
         a, b = a_mod(x).float(), b_mod(x).float()
         rng = a.abs().max().item()

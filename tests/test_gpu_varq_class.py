@@ -88,25 +88,30 @@ def test_per_head_extension_single_call(dev):
 
 @pytest.mark.parametrize('method', list(O.METHODS))
 @pytest.mark.parametrize('bits', [4, 8])
-def test_fused_attention_over_quantizer_caches(dev, method, bits):
+@pytest.mark.parametrize('fmt', ['BHLc', 'BLHc'])
+def test_fused_attention_over_quantizer_caches(dev, method, bits, fmt):
     """`fused_attention` over the packed caches of two drop-in quantizers, all six methods of
-    the reference, four steps, against the oracle class's dequant_all -> bf16 SDPA on the CPU
-    (the path the reference runs: VAR_Q/quant.py:216-230 into the attention backend).
+    the reference in both of its layouts (BLHc is what its flash-attention call and
+    VAR-VAR_Q-8.json use, BHLc what Infinity-VAR_Q-8.json names), four steps, against the
+    oracle class's dequant_all -> bf16 SDPA on the CPU (the path the reference runs:
+    VAR_Q/quant.py:216-230 into the attention backend).
     Tolerance: cosine >= 0.9995, max-abs 2e-2 in units of the output range."""
     from var_q_amd.quant import fused_attention
-    note('fused_attention', method, bits)
-    ks, vs = _steps('BHLc', torch.bfloat16, seed=20 + bits), _steps('BHLc', torch.bfloat16, seed=30 + bits)
-    rk, rv = O.OracleVARQ(bits, 'BHLc', method, pack_to_int32=False), O.OracleVARQ(bits, 'BHLc', method, pack_to_int32=False)
-    gk, gv = VAR_Q(bits, 'BHLc', method), VAR_Q(bits, 'BHLc', method)
+    note('fused_attention', method, bits, fmt)
+    ks, vs = _steps(fmt, torch.bfloat16, seed=20 + bits), _steps(fmt, torch.bfloat16, seed=30 + bits)
+    rk, rv = O.OracleVARQ(bits, fmt, method, pack_to_int32=False), O.OracleVARQ(bits, fmt, method, pack_to_int32=False)
+    gk, gv = VAR_Q(bits, fmt, method), VAR_Q(bits, fmt, method)
     g = torch.Generator().manual_seed(5)
+    bhl = (lambda t: t) if fmt == 'BHLc' else (lambda t: t.transpose(1, 2))   # to the oracle attention's [B,H,L,c]
     for k, v in zip(ks, vs):
         kd, vd = rk.use_var_q(k), rv.use_var_q(v)
         for qz, item in ((gk, k), (gv, v)):
             qz.quant(item.to(dev))
             qz.cache()
         q = torch.randn(k.shape[0], k.shape[1], k.shape[2], k.shape[3], generator=g).bfloat16()
-        out = fused_attention(q.to(dev), gk, gv, 0.125).float().cpu()
-        ref = O.attention_ref(q, kd, vd, 0.125).float()
+        out = bhl(fused_attention(q.to(dev), gk, gv, 0.125).float().cpu())
+        assert out.shape == bhl(q).shape
+        ref = O.attention_ref(bhl(q), bhl(kd), bhl(vd), 0.125).float()
         span = max(1.0, float(ref.abs().max()))
         err = float((out - ref).abs().max())
         cos = float(torch.nn.functional.cosine_similarity(out.flatten().double(), ref.flatten().double(), dim=0))
@@ -123,10 +128,10 @@ def test_fused_attention_refuses_what_it_cannot_serve(dev):
     for qz in (a, b):
         qz.use_var_q(x)
     fused_attention(q, a, b, 1.0)
-    with pytest.raises(ValueError, match='BHLc'):
+    with pytest.raises(ValueError, match='layout'):             # K and V cached in different layouts
         c = VAR_Q(8, 'BLHc', 'G_SCALE_HEAD_DIM')
         c.use_var_q(x.transpose(1, 2).contiguous())
-        fused_attention(q, c, c, 1.0)
+        fused_attention(q, a, c, 1.0)
     with pytest.raises(ValueError, match='bit-width'):
         d = VAR_Q(4, 'BHLc', 'G_SCALE_HEAD_DIM')
         d.use_var_q(x)

@@ -86,6 +86,10 @@ struct AttnParams {
   // workspace, the output is written directly.
   int nsplit;
   float *ws_o, *ws_ml;
+  // memory layout, in rows (a row = the D values of one token of one head):
+  // q/out row = b*q_bs + h*q_hs + i*q_ts, key row = b*kv_bs + slot*kv_hs + j*kv_ts.
+  // BHLc: (H*L, L, 1); BLHc (the layout of the flash-attention call): (L*H, 1, H).
+  int64_t q_bs, q_hs, q_ts, kv_bs, kv_hs, kv_ts;
 };
 
 __device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
@@ -329,7 +333,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   const bool q_live = qrow < p.Lq;
   const bool wave_live = qt * BM + wave * 32 < p.Lq;   // wave-uniform
   const int qrow_c = q_live ? qrow : p.Lq - 1;
-  const __bf16 *qptr = p.q + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow_c) * D;
+  const __bf16 *qptr = p.q + (b * p.q_bs + hq * p.q_hs + qrow_c * p.q_ts) * D;
   int limit = p.kv_limit ? min(p.kv_limit[qrow_c], p.Lk) : p.Lk;
   if (limit < 0) limit = 0;
 
@@ -478,7 +482,8 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int s = 0; s < NSV; ++s) r_run[s] = 0.f;
 
-  const int64_t kv_row0 = (int64_t)(b * p.Hkv + hs) * p.Lstride;
+  const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
+  const int64_t kv_ts = p.kv_ts;
   const u32 *kw = p.k_words + kv_row0 * WPR;
   const u32 *vw = p.v_words + kv_row0 * WPR;
 
@@ -495,7 +500,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       const int piece = tid + i * NT;
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
-        kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + (int64_t)key * WPR + (piece % (WPR / 4)) * 4);
+        kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + key * kv_ts * WPR + (piece % (WPR / 4)) * 4);
       }
     }
   };
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
       const int piece = tid + i * NT;
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
-        vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + (int64_t)key * WPR + (piece % (WPR / 4)) * 4);
+        vreg[i] = *reinterpret_cast<const u32x4_t *>(vw + key * kv_ts * WPR + (piece % (WPR / 4)) * 4);
       }
     }
     // scales: thread t handles key t % 64; wavefront w takes K group w and V group
@@ -518,15 +523,15 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
     } else {
       const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = NW - 1 - seg;
       if (seg < NSK) {
-        const int64_t g = (kv_row0 + key) * NSK + seg;
+        const int64_t g = (kv_row0 + key * kv_ts) * NSK + seg;
         ksc = p.k_scale[g];
         kzp = p.k_zp ? p.k_zp[g] : 0.f;
       }
       if (vseg < NSV) {
-        const int64_t g = (kv_row0 + key) * NSV + vseg;
+        const int64_t g = (kv_row0 + key * kv_ts) * NSV + vseg;
         vsc = p.v_scale[g];
         vzp = p.v_zp ? p.v_zp[g] : 0.f;
-        if (FOLD_SV) ksc0 = p.k_scale[(kv_row0 + key) * NSK];
+        if (FOLD_SV) ksc0 = p.k_scale[(kv_row0 + key * kv_ts) * NSK];
       }
     }
   };
@@ -962,7 +967,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int s = 0; s < NSV; ++s) rq[s] = __shfl(racc[s], col, 64) + r_run[s];
   if (q_live) {
-    __bf16 *optr = p.out + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow) * D;
+    __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D;
     // with the keys shared out: the normalized fp32 output and (reference, denominator) of
     // this share, for the combining kernel
     const bool shared_out = p.nsplit > 1;
@@ -1028,7 +1033,7 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
   const int bh = (int)(row / p.Lq), qrow = (int)(row % p.Lq);
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
   const int hq = p.head_map ? p.head_map[hs] : hs;
-  __bf16 *optr = p.out + ((int64_t)(b * p.Hq + hq) * p.Lq + qrow) * D + c0;
+  __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D + c0;
   *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_bf16_rne(acc[0] * inv, acc[1] * inv), pack_bf16_rne(acc[2] * inv, acc[3] * inv));
 }
 
@@ -1063,6 +1068,19 @@ int dispatch_groups(const AttnParams &p, int gk, int gv, hipStream_t st) {
   VARQ_G(128, 128) VARQ_G(64, 64) VARQ_G(32, 32) VARQ_G(32, 64)
 #undef VARQ_G
   return -1;
+}
+
+int set_layout(AttnParams &p, int layout, const char *who) {
+  if (layout == VARQ_LAYOUT_BHLC) {
+    p.q_bs = (int64_t)p.Hq * p.Lq; p.q_hs = p.Lq; p.q_ts = 1;
+    p.kv_bs = (int64_t)p.Hkv * p.Lstride; p.kv_hs = p.Lstride; p.kv_ts = 1;
+  } else if (layout == VARQ_LAYOUT_BLHC) {
+    p.q_bs = (int64_t)p.Lq * p.Hq; p.q_hs = 1; p.q_ts = p.Hq;
+    p.kv_bs = (int64_t)p.Lstride * p.Hkv; p.kv_hs = 1; p.kv_ts = p.Hkv;
+  } else {
+    return varq_set_error(VARQ_ERR_INVALID, "%s: layout must be VARQ_LAYOUT_BHLC (0) or VARQ_LAYOUT_BLHC (1), got %d", who, layout);
+  }
+  return VARQ_OK;
 }
 
 // ---- sharing the keys of a query block out over several workgroups ---------------------
@@ -1141,7 +1159,7 @@ extern "C" int varq_fused_attn(const void *q, void *out,
                                const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                                int B, int Hq, int Hkv, const int32_t *head_map,
                                int Lq, int Lk, int Lk_stride, int D,
-                               const int32_t *kv_limit, float softmax_scale,
+                               const int32_t *kv_limit, float softmax_scale, int layout,
                                void *workspace, size_t workspace_bytes, int splits, void *stream) {
   VARQ_CHECK_ARG(q && out && k_words && v_words && k_scale && v_scale, "fused_attn: null pointer");
   VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn: bad sizes");
@@ -1172,6 +1190,7 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  if (int e = set_layout(p, layout, "fused_attn")) return e;
   if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn")) return e;
   hipStream_t st = (hipStream_t)stream;
   int rc = -1;
@@ -1197,7 +1216,7 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
                                        int nseg, const int32_t *host_seg_end,
                                        int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                                        int Lq, int Lk, int Lk_stride, int D,
-                                       const int32_t *kv_limit, float softmax_scale,
+                                       const int32_t *kv_limit, float softmax_scale, int layout,
                                        void *workspace, size_t workspace_bytes, int splits, void *stream) {
   VARQ_CHECK_ARG(q && out && k_words && v_words && k_chan_scale && v_chan_scale, "fused_attn_channel: null pointer");
   VARQ_CHECK_ARG(nseg >= 1 && nseg <= kMaxSegments, "fused_attn_channel: nseg must be 1..%d (got %d)", kMaxSegments, nseg);
@@ -1239,6 +1258,7 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  if (int e = set_layout(p, layout, "fused_attn_channel")) return e;
   if (int e = set_splits(p, D, (Lk + BN - 1) / BN + nseg - 1, splits, workspace, workspace_bytes, "fused_attn_channel"))
     return e;
   hipStream_t st = (hipStream_t)stream;

@@ -24,7 +24,7 @@ cached.  Three backends behind the same interface:
   * `fused='quantizer'`: the drop-in quantizers of any rule of the JSON files (the shipped
     G_SCALE_HEAD_DIM rule included) do `quant` + `cache` as in the first backend, and
     `var_q_amd.quant.fused_attention` attends over their packed caches, so the
-    dequantized full-length K/V of `dequant_all` is never built.  Layout BHLc.
+    dequantized full-length K/V of `dequant_all` is never built.  Either layout.
 
 The transformer blocks around the attention (AdaLN, FFN, cross-attention) are
 outside this package.
@@ -104,7 +104,7 @@ class _QuantizedSelfAttention(nn.Module):
             assert enable_quantization and quant_method == 'G_GROUP' and group_size, \
                 'the fused backend needs the row-local group-wise quantizer (quant_method="G_GROUP", group_size=g)'
         if fused == 'quantizer':
-            assert enable_quantization and layout == 'BHLc', "fused='quantizer' needs quantization and layout BHLc"
+            assert enable_quantization, "fused='quantizer' needs quantization"
         self.mat_qkv = nn.Linear(embed_dim, embed_dim * 3, bias=False)
         self.q_bias, self.v_bias = nn.Parameter(torch.zeros(embed_dim)), nn.Parameter(torch.zeros(embed_dim))
         self.register_buffer('zero_k_bias', torch.zeros(embed_dim))
@@ -171,8 +171,10 @@ class _QuantizedSelfAttention(nn.Module):
             for quantizer, item in ((self.k_quant, k), (self.v_quant, v)):
                 quantizer.quant(item)
                 quantizer.cache()
-            o = fused_attention(q, self.k_quant, self.v_quant, scale)                     # [B,H,L,c]
-            return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
+            o = fused_attention(q, self.k_quant, self.v_quant, scale)                     # in the layout of q
+            if self.layout == 'BHLc':
+                o = o.transpose(1, 2)
+            return o.reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
         if self.caching and self.fused:
             if attn_bias is not None:
                 raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')

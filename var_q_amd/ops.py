@@ -263,35 +263,51 @@ def qkv_prepare_append(qkv: torch.Tensor, q_out: torch.Tensor, group: int, bits:
 # ---------------------------------------------------------------------------
 # fused dequant flash-attention
 # ---------------------------------------------------------------------------
-def _attn_workspace(lib, q, Hkv, Lk, nseg, splits):
+_LAYOUTS = {'BHLc': 0, 'BLHc': 1}
+
+
+def _attn_dims(q, k_words, layout):
+    """(B, Hq, Lq, D, Hkv, Lstride, W) of the attention operands in either layout."""
+    assert layout in _LAYOUTS, f'layout must be one of {sorted(_LAYOUTS)}'
+    if layout == 'BHLc':
+        B, Hq, Lq, D = q.shape
+        Bk, Hkv, Lstride, W = k_words.shape
+    else:
+        B, Lq, Hq, D = q.shape
+        Bk, Lstride, Hkv, W = k_words.shape
+    assert Bk == B, 'batch sizes of q and the cache differ'
+    return B, Hq, Lq, D, Hkv, Lstride, W
+
+
+def _attn_workspace(lib, B, Hkv, Lq, Lk, D, nseg, splits, device):
     """Device memory for the partial results of a launch that shares keys out (None if the
     library would not); allocated on the current stream, so its reuse after the call is ordered."""
-    B, _, Lq, D = q.shape
     n = int(lib.varq_fused_attn_workspace_bytes(B, Hkv, Lq, Lk, D, nseg, int(splits)))
     if n == 0:
         return None, 0
-    return torch.empty(n, dtype=torch.uint8, device=q.device), n
+    return torch.empty(n, dtype=torch.uint8, device=device), n
 
 
 def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_zp: Optional[torch.Tensor],
                v_words: torch.Tensor, v_scale: torch.Tensor, v_zp: Optional[torch.Tensor],
                k_bits: int, v_bits: int, Lk: int, softmax_scale: float,
                kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
-               out: Optional[torch.Tensor] = None, splits: int = 0) -> torch.Tensor:
+               out: Optional[torch.Tensor] = None, splits: int = 0, layout: str = 'BHLc') -> torch.Tensor:
     """q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32;
     k/v_scale (zp) [B,Hkv,Lstride,D/group] fp32; attends keys 0..Lk-1.
     Returns out [B,Hq,Lq,D] bf16 (rows of heads not in head_map are untouched).
+    layout 'BLHc': every tensor has tokens before heads instead ([B,Lq,Hq,D], [B,Lstride,Hkv,...]),
+    the layout of the reference's flash-attention call.
     splits: over how many workgroups the keys of a query block are shared out (0: the
     library decides from the shape, 1: never, 2..8: exactly)."""
     for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_scale, 'k_scale'), (v_scale, 'v_scale')):
         _gpu(t, n)
         assert t.is_contiguous(), f'{n} must be contiguous'
     assert q.dtype == torch.bfloat16 and q.dim() == 4
-    B, Hq, Lq, D = q.shape
-    Bk, Hkv, Lstride, Wk = k_words.shape
-    assert Bk == B and v_words.shape[:3] == k_words.shape[:3]
+    B, Hq, Lq, D, Hkv, Lstride, Wk = _attn_dims(q, k_words, layout)
+    assert v_words.shape[:3] == k_words.shape[:3]
     assert Wk * 32 == D * k_bits and v_words.shape[3] * 32 == D * v_bits
-    assert k_scale.shape[:3] == (B, Hkv, Lstride) and v_scale.shape[:3] == (B, Hkv, Lstride)
+    assert k_scale.shape[:3] == k_words.shape[:3] and v_scale.shape[:3] == k_words.shape[:3]
     k_group, v_group = D // k_scale.shape[3], D // v_scale.shape[3]
     if out is None:
         out = torch.empty_like(q)
@@ -305,13 +321,13 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
         assert Hkv == Hq
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        ws, ws_bytes = _attn_workspace(lib, q, Hkv, Lk, 1, splits)
+        ws, ws_bytes = _attn_workspace(lib, B, Hkv, Lq, Lk, D, 1, splits, q.device)
         check(lib.varq_fused_attn(q.data_ptr(), out.data_ptr(),
                                   k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp), k_bits, k_group,
                                   v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), v_bits, v_group,
                                   B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                  _ptr(kv_limit), float(softmax_scale), _ptr(ws), ws_bytes, int(splits),
-                                  _stream(q)), 'varq_fused_attn')
+                                  _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ptr(ws), ws_bytes,
+                                  int(splits), _stream(q)), 'varq_fused_attn')
     return out
 
 
@@ -321,7 +337,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                        bits: int, Lk: int, softmax_scale: float,
                        kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
                        out: Optional[torch.Tensor] = None, seg_ends: Optional[Sequence[int]] = None,
-                       splits: int = 0) -> torch.Tensor:
+                       splits: int = 0, layout: str = 'BHLc') -> torch.Tensor:
     """Attention over a cache quantized per (head, channel): the scale layout of the
     reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
     (G_TENSOR, G_SCALE) expanded to the table, and the affine per-head-per-dim variant.
@@ -331,15 +347,14 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
     where the tables change along the keys: a cache filled step by step by the reference's
     append methods has one table per step (VAR_Q/quant.py:196-201).
     With a single table the zero-point of K may be None even for an affine K: it shifts all
-    logits of a query alike.  splits as in fused_attn."""
+    logits of a query alike.  splits and layout as in fused_attn."""
     for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_chan_scale, 'k_chan_scale'),
                  (v_chan_scale, 'v_chan_scale')):
         _gpu(t, n)
         assert t.is_contiguous(), f'{n} must be contiguous'
     assert q.dtype == torch.bfloat16 and q.dim() == 4
-    B, Hq, Lq, D = q.shape
-    Bk, Hkv, Lstride, W = k_words.shape
-    assert Bk == B and v_words.shape == k_words.shape and W * 32 == D * bits
+    B, Hq, Lq, D, Hkv, Lstride, W = _attn_dims(q, k_words, layout)
+    assert v_words.shape == k_words.shape and W * 32 == D * bits
     nseg = 1 if seg_ends is None else len(seg_ends)
     ends = None
     if seg_ends is not None:
@@ -363,11 +378,11 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
         assert Hkv == Hq
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        ws, ws_bytes = _attn_workspace(lib, q, Hkv, Lk, nseg, splits)
+        ws, ws_bytes = _attn_workspace(lib, B, Hkv, Lq, Lk, D, nseg, splits, q.device)
         check(lib.varq_fused_attn_channel(q.data_ptr(), out.data_ptr(),
                                           k_words.data_ptr(), k_chan_scale.data_ptr(), _ptr(k_chan_zp),
                                           v_words.data_ptr(), v_chan_scale.data_ptr(), _ptr(v_chan_zp),
                                           nseg, ends, bits, B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                          _ptr(kv_limit), float(softmax_scale), _ptr(ws), ws_bytes, int(splits),
-                                          _stream(q)), 'varq_fused_attn_channel')
+                                          _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ptr(ws), ws_bytes,
+                                          int(splits), _stream(q)), 'varq_fused_attn_channel')
     return out

@@ -134,13 +134,13 @@ class VAR_Q:
     def _reset_cache(self):
         # what the fused attention reads, kept up to date by cache(): the end of every cached
         # step with its (head, channel) tables for the methods whose scale is shared by the
-        # tokens of a step, a full-size [B,H,capacity,groups] copy of the per-token scales for
-        # the others
+        # tokens of a step, a full-size copy of the per-token scales (shaped like the code buffer,
+        # [.., capacity, .., groups]) for the others
         self._seg_ends: List[int] = []
         self._tab_scale: Optional[torch.Tensor] = None      # [MAX_TABLE_STEPS, H, c]
         self._tab_zp: Optional[torch.Tensor] = None
-        self._tok_scale = _Growable(2)
-        self._tok_zp = _Growable(2)
+        self._tok_scale = _Growable(self.dim_cat)
+        self._tok_zp = _Growable(self.dim_cat)
         self._c_item = _Growable(self.dim_cat)
         self._c_scale = _Growable(self.dim_cat)
         self._c_zp = _Growable(self.dim_cat)
@@ -221,11 +221,15 @@ class VAR_Q:
             raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
 
     def _note_step(self, q_cur: torch.Tensor, replace: bool):
-        """Book-keeping for `fused_attention` (layout BHLc, packed codes only)."""
-        if self.qkv_format != 'BHLc' or not self.pack_to_int32:
+        """Book-keeping for `fused_attention` (packed codes only)."""
+        if not self.pack_to_int32:
             return
-        B, H, n, _ = q_cur.shape
+        if self._tok_scale.dim != self.dim_cat:   # layout was re-assigned before the first step
+            self._tok_scale, self._tok_zp = _Growable(self.dim_cat), _Growable(self.dim_cat)
+        bhl = self.qkv_format == 'BHLc'
+        B, H, n = q_cur.shape[0], q_cur.shape[1 if bhl else 2], q_cur.shape[2 if bhl else 1]
         c = self._pack_meta['orig_c']
+        full = (1, H, 1, c) if bhl else (1, 1, H, c)
         if self.quant_method in _TABLE_METHODS:
             if replace:
                 self._seg_ends = []
@@ -236,14 +240,15 @@ class VAR_Q:
             if self._tab_scale is None:
                 self._tab_scale = torch.empty((MAX_TABLE_STEPS, H, c), dtype=torch.float32, device=q_cur.device)
                 self._tab_zp = None if self.zp is None else torch.empty_like(self._tab_scale)
-            self._tab_scale[k].copy_(self.scale.expand(1, H, 1, c).reshape(H, c))
+            self._tab_scale[k].copy_(self.scale.expand(*full).reshape(H, c))
             if self.zp is not None:
-                self._tab_zp[k].copy_(self.zp.expand(1, H, 1, c).reshape(H, c))
+                self._tab_zp[k].copy_(self.zp.expand(*full).reshape(H, c))
         else:
             ng = self.scale.shape[3]
-            self._tok_scale.append(self.scale.expand(B, H, n, ng))
+            shape = (B, H, n, ng) if bhl else (B, n, H, ng)
+            self._tok_scale.append(self.scale.expand(*shape))
             if self.zp is not None:
-                self._tok_zp.append(self.zp.expand(B, H, n, ng))
+                self._tok_zp.append(self.zp.expand(*shape))
 
     # ---------------- dequantize ----------------
     def _dequant(self, q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor]) -> torch.Tensor:
@@ -301,17 +306,19 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     exactly that and hands it to its attention backend: VAR_Q/quant.py:216-230,
     Infinity/infinity/models/basic.py:339-351).
 
-    q [B,H,Lq,c] (cast to bf16); both quantizers in layout 'BHLc', packed, same bit-width,
-    c in {64, 128}, after at least one `cache()`.  Methods whose scale is shared by the
+    q [B,H,Lq,c] for quantizers in layout 'BHLc', [B,Lq,H,c] for 'BLHc' (the layout of the
+    reference's flash-attention call and of VAR-VAR_Q-8.json), cast to bf16; both quantizers in
+    the same layout, packed, same bit-width, c in {64, 128}, after at least one `cache()`.  Methods whose scale is shared by the
     tokens of a step (G_SCALE_HEAD_DIM -- the shipped rule --, G_HEAD_DIM, G_TENSOR, G_SCALE,
     G_HEAD) go through one table per cached step, at most MAX_TABLE_STEPS steps; per-token
     methods (G_TOKEN, G_TOKEN_HEAD, G_GROUP) through per-token scales.  Everything the
     kernels read is kept current by `cache()`, so a call launches the attention and nothing
     else.  kv_limit: int32 [Lq], query i sees keys j < kv_limit[i].  Returns bf16
-    [B,H,Lq,c]."""
+    in the shape of q."""
+    layout = k_quant.qkv_format
+    if v_quant.qkv_format != layout:
+        raise ValueError(f'fused_attention: K is cached in layout {layout}, V in {v_quant.qkv_format}')
     for qz, n in ((k_quant, 'k_quant'), (v_quant, 'v_quant')):
-        if qz.qkv_format != 'BHLc':
-            raise ValueError(f'fused_attention: {n} must use layout BHLc')
         if not qz.pack_to_int32 or qz.cached_item is None:
             raise ValueError(f'fused_attention: {n} needs a packed cache (pack_to_int32=True, after cache())')
     bits = k_quant.quant_bits
@@ -321,12 +328,14 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     Lk = k_quant._c_item.len
     if v_quant._c_item.len != Lk or kbuf.shape != vbuf.shape:
         raise ValueError('fused_attention: the K and V caches differ in length or capacity')
-    B, H, cap, _ = kbuf.shape
+    bhl = layout == 'BHLc'
+    B, H, cap = kbuf.shape[0], kbuf.shape[1 if bhl else 2], kbuf.shape[2 if bhl else 1]
     c = k_quant._pack_meta['orig_c']
     if c not in (64, 128):
         raise ValueError(f'fused_attention: head dim {c} not supported (64 or 128)')
     q = q.to(torch.bfloat16).contiguous()
-    assert q.dim() == 4 and q.shape[0] == B and q.shape[1] == H and q.shape[3] == c, 'q must be [B,H,Lq,c]'
+    assert q.dim() == 4 and q.shape[0] == B and q.shape[1 if bhl else 2] == H and q.shape[3] == c, \
+        'q must be [B,H,Lq,c] (BHLc) or [B,Lq,H,c] (BLHc)'
     km, vm = k_quant.quant_method, v_quant.quant_method
     if km in _TABLE_METHODS and vm in _TABLE_METHODS:
         ends = k_quant._seg_ends
@@ -336,10 +345,11 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
             raise ValueError(f'fused_attention: at most {MAX_TABLE_STEPS} cached steps, the same for K and V')
         return ops.fused_attn_channel(q, kbuf, k_quant._tab_scale, k_quant._tab_zp, vbuf, v_quant._tab_scale,
                                       v_quant._tab_zp, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out,
-                                      seg_ends=ends)
+                                      seg_ends=ends, layout=layout)
     if km in _TOKEN_METHODS and vm in _TOKEN_METHODS:
         ks, kz, vs, vz = k_quant._tok_scale.buf, k_quant._tok_zp.buf, v_quant._tok_scale.buf, v_quant._tok_zp.buf
-        if ks.shape[2] != cap or vs.shape[2] != cap:
+        if ks.shape[:3] != kbuf.shape[:3] or vs.shape[:3] != kbuf.shape[:3]:
             raise ValueError('fused_attention: scale buffers and code buffers differ in capacity')
-        return ops.fused_attn(q, kbuf, ks, kz, vbuf, vs, vz, bits, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out)
+        return ops.fused_attn(q, kbuf, ks, kz, vbuf, vs, vz, bits, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out,
+                              layout=layout)
     raise ValueError(f'fused_attention: methods {km} / {vm} cannot be combined')
