@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 3
+#define VARQ_ABI_VERSION 4
 
 enum varq_status {
   VARQ_OK = 0,
@@ -97,13 +97,20 @@ int varq_quant_pack_rows2(const void *x0, const void *x1, int x_dtype, int64_t n
  *   words   packed output [rows, ceil(c/(32/bits))] or NULL
  *   codes   int8 output [rows, c] or NULL (the pack_to_int32=False mode,
  *           VAR_Q/quant.py:174-175).  At least one of words/codes is non-NULL.
+ *   host_out_map  NULL: output rows are the input rows.  Else 3 host int64
+ *           {rows per block, extra rows per block, first row}: input row r is
+ *           written to output row r + (r / rows_per_block) * extra + first, which
+ *           puts a step straight into its tokens of a larger cache buffer instead
+ *           of the torch.cat of VAR_Q/quant.py:200-201 -- a [B,H,n,c] step at token
+ *           len of a [B,H,cap,..] buffer is {n, cap - n, len}, a [B,n,H,c] step in
+ *           a [B,cap,H,..] buffer {n*H, (cap - n)*H, len*H}.
  *   workspace  >= varq_quant_workspace_bytes(...) bytes, any contents
  * bits in 2..8 when only codes are requested, {2,4,8} when words are.
  */
 size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask);
 int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
                     int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
-                    void *workspace, size_t workspace_bytes, void *stream);
+                    const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream);
 
 /* VAR_Q/pack_unpack.py:107-134 (and its CPU twin 177-196): int8 codes [rows,c]
  * -> int32 words [rows, ceil(c*bits/32)], zero padding in the last word. */

@@ -25,7 +25,7 @@ def test_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
     assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
-    assert lib.varq_abi_version() == _lib.ABI_VERSION == 3
+    assert lib.varq_abi_version() == _lib.ABI_VERSION == 4
 
 
 def test_invalid_arguments_are_rejected_on_the_host():
@@ -44,12 +44,14 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert rc == -1
     rc = lib.varq_unpack(fake, 4, 16, 3, fake, None)
     assert rc == -1
-    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 9, 0, 1e-12, fake, None, fake, None, fake, 1 << 20, None)
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 9, 0, 1e-12, fake, None, fake, None, None, fake, 1 << 20, None)
     assert rc == -1
-    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 3, 0, 1e-12, fake, None, fake, None, fake, 1 << 20, None)
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 3, 0, 1e-12, fake, None, fake, None, None, fake, 1 << 20, None)
     assert rc == -1 and b'2/4/8' in lib.varq_last_error()
-    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 4, 0, 1e-12, fake, None, fake, None, fake, 4, None)
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 4, 0, 1e-12, fake, None, fake, None, None, fake, 4, None)
     assert rc == -4
+    rc = lib.varq_quant_pack(fake, 0, i64([2, 2, 2, 8]), 3, 4, 0, 1e-12, fake, None, fake, None, i64([3, 5, 0]), fake, 1 << 20, None)
+    assert rc == -1 and b'output map' in lib.varq_last_error()   # 8 rows are not whole blocks of 3
     # 24 groups: room for scale reciprocal + flag per group plus per-chunk partial min/max (a multiple of
     # the group count), never less than two words per group; odd channel counts use two words per group
     ws = lib.varq_quant_workspace_bytes(i64([2, 5, 3, 8]), 0b0011)

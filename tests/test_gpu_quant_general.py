@@ -155,3 +155,35 @@ def test_all_ones_scale_significand_in_general_path(dev):
     assert int(q[1, 1, 7, 0]) == 1
     note('general all-ones scale')
     _check(x, (0, 2), 8, False, True, dev)
+
+
+@pytest.mark.parametrize('token_dim', [1, 2])
+@pytest.mark.parametrize('mask', [0b0101, 0b0011, 0b1111, 0b1000, 0b0111])
+def test_codes_written_into_a_window_of_a_larger_buffer(dev, token_dim, mask):
+    """The output map: a step lands at a token offset of a cache buffer with more room along
+    the token dim, scale and zero-point in caller-provided buffers; the rest of the buffer is
+    untouched and the window holds what the plain call returns.  Tiled shapes (c a multiple
+    of 8) and the scalar kernels (c = 20)."""
+    dims = tuple(d for d in range(4) if (mask >> d) & 1)
+    g = torch.Generator().manual_seed(900 + mask + token_dim)
+    for shape, bits, asym, pack in [((2, 5, 7, 64), 8, False, True), ((3, 4, 6, 128), 4, True, True),
+                                    ((2, 3, 5, 20), 8, True, False), ((2, 9, 3, 32), 2, True, True)]:
+        x = (torch.randn(*shape, generator=g) * 3).bfloat16().to(dev)
+        want_q, want_s, want_z = ops.quant_pack(x, dims, bits, asym=asym, pack=pack)
+        cap, at = shape[token_dim] + 11, 4
+        big = list(want_q.shape)
+        big[token_dim] = cap
+        buf = torch.full(big, 0x5a if not pack else 0x5a5a5a5a, dtype=want_q.dtype, device=dev)
+        s_out = torch.empty(want_s.numel(), dtype=torch.float32, device=dev)
+        z_out = torch.empty(want_s.numel(), dtype=torch.float32, device=dev) if asym else None
+        note('general out map', mask, shape, bits, asym, pack, token_dim)
+        q, s, z = ops.quant_pack(x, dims, bits, asym=asym, pack=pack, out=buf, out_token_dim=token_dim, out_token=at,
+                                 scale_out=s_out, zp_out=z_out)
+        torch.cuda.synchronize()
+        assert q.data_ptr() == buf.narrow(token_dim, at, shape[token_dim]).data_ptr()
+        assert torch.equal(q, want_q) and torch.equal(s, want_s) and torch.equal(s_out.view(want_s.shape), want_s)
+        if asym:
+            assert torch.equal(z, want_z) and torch.equal(z_out.view(want_s.shape), want_z)
+        fill = buf.new_full((), 0x5a if not pack else 0x5a5a5a5a)
+        assert bool((buf.narrow(token_dim, 0, at) == fill).all())
+        assert bool((buf.narrow(token_dim, at + shape[token_dim], cap - at - shape[token_dim]) == fill).all())

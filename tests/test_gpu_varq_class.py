@@ -145,3 +145,33 @@ def test_fused_attention_refuses_what_it_cannot_serve(dev):
             for qz in (a, b):
                 qz.use_var_q(x)
         fused_attention(q, a, b, 1.0)
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('pack', [True, False])
+def test_quant_writes_into_the_cache_buffer(dev, fmt, pack):
+    """The appending methods quantize a step straight into the cache buffer: `quantized_item`
+    is a window of it and cache() copies nothing.  A second quant() before cache() replaces
+    the first; an item put there by the caller is appended by copy as before.  Contents as
+    the oracle class's."""
+    ref = O.OracleVARQ(8, fmt, 'G_SCALE_HEAD_DIM', pack_to_int32=False)
+    gpu = VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM', pack_to_int32=pack)
+    items = _steps(fmt, torch.bfloat16, seed=77)
+    note('staged quant', fmt, pack)
+    gpu.quant((items[0] * 3).to(dev))          # dropped: the next quant() takes its place
+    for i, x in enumerate(items):
+        ref.use_var_q(x)
+        gpu.quant(x.to(dev))
+        buf = gpu._c_item.buf
+        lo, hi = buf.data_ptr(), buf.data_ptr() + buf.numel() * buf.element_size()
+        assert lo <= gpu.quantized_item.data_ptr() < hi, 'the step was not quantized into the cache buffer'
+        if i == 2:                              # the caller swaps the item: copied in as before
+            gpu.quantized_item = gpu.quantized_item.clone()
+        gpu.cache()
+    codes = gpu.cached_item
+    if pack:
+        from var_q_amd import ops
+        codes = ops.unpack(codes.contiguous(), items[0].shape[-1], 8)
+    assert torch.equal(codes.cpu(), ref.cached_item)
+    assert torch.equal(gpu.cached_scale.cpu(), ref.cached_scale)
+    assert torch.equal(gpu.dequant_all().cpu(), ref.dequant_all())

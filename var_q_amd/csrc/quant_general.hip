@@ -41,7 +41,20 @@ struct GenParams {
   int bits, qmin, qmax, wpr; // wpr = words per row
   int asym;
   float eps;
+  // Output rows (codes / words) may land in a larger buffer: input row r goes to output row
+  // r + (r / out_inner) * out_delta + out_off -- a step [B,H,n,c] into tokens len.. of a cache
+  // [B,H,cap,..] is (n, cap - n, len), a step [B,n,H,c] into [B,cap,H,..] is (n*H, (cap - n)*H, len*H).
+  int out_mapped;
+  int64_t out_inner, out_delta, out_off;
 };
+
+__device__ __forceinline__ int64_t out_row(const GenParams &p, int64_t row) {
+  return p.out_mapped ? row + (row / p.out_inner) * p.out_delta + p.out_off : row;
+}
+// (rows of the tiled kernels fit 31 bits)
+__device__ __forceinline__ int64_t out_row32(const GenParams &p, int64_t row) {
+  return p.out_mapped ? row + (int64_t)((u32)row / (u32)p.out_inner) * p.out_delta + p.out_off : row;
+}
 
 __global__ void init_ws_kernel(u32 *ws_max, u32 *ws_min, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -274,7 +287,8 @@ __global__ __launch_bounds__(256) void quant_tiled_kernel(GenParams p, Plan pl, 
 #pragma unroll
       for (int j = 0; j < 8; ++j) q[j] = (int)__builtin_amdgcn_fmed3f(rintf(v[j] / s[j % NV]) + z[j % NV], qmin, qmax);
     }
-    const int64_t o = row * p.c8 + l.col;
+    const int64_t orow = out_row32(p, row);
+    const int64_t o = orow * p.c8 + l.col;
     if (p.codes) {
       u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
       u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
@@ -284,16 +298,16 @@ __global__ __launch_bounds__(256) void quant_tiled_kernel(GenParams p, Plan pl, 
       if (p.bits == 8) {
         u32 lo = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | ((u32)q[3] << 24);
         u32 hi = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | ((u32)q[7] << 24);
-        *reinterpret_cast<uint2 *>(p.words + row * p.wpr + l.col * 2) = make_uint2(lo, hi);
+        *reinterpret_cast<uint2 *>(p.words + orow * p.wpr + l.col * 2) = make_uint2(lo, hi);
       } else {
         u32 w = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) w |= ((u32)q[j] & mask) << (j * p.bits);
         if (p.bits == 4) {
-          p.words[row * p.wpr + l.col] = (int32_t)w;
+          p.words[orow * p.wpr + l.col] = (int32_t)w;
         } else {  // 2 bits: 16 codes per word = two adjacent octets (c % 16 == 0 on this path)
           u32 other = __shfl_xor(w, 1, 64);
-          if ((l.col & 1) == 0) p.words[row * p.wpr + (l.col >> 1)] = (int32_t)(w | (other << 16));
+          if ((l.col & 1) == 0) p.words[orow * p.wpr + (l.col >> 1)] = (int32_t)(w | (other << 16));
         }
       }
     }
@@ -360,10 +374,10 @@ __global__ void quant_scalar_kernel(GenParams p) {
     const int64_t g = gb + (p.keepc ? ch : 0);
     const int q = quant_one(In8<DT>::load1(p.x, r * p.c + ch), p.scale[g], p.asym ? p.zp[g] : 0.f, p.asym,
                             (float)p.qmin, (float)p.qmax);
-    if (p.codes) p.codes[r * p.c + ch] = (int8_t)q;
+    if (p.codes) p.codes[out_row(p, r) * p.c + ch] = (int8_t)q;
     w |= ((u32)q & mask) << (j * p.bits);
   }
-  if (p.words) p.words[r * wpr + wi] = (int32_t)w;
+  if (p.words) p.words[out_row(p, r) * wpr + wi] = (int32_t)w;
 }
 
 // Host side of the tiled path: canonical form of the leading dims and the launch shape.
@@ -507,7 +521,7 @@ extern "C" size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int red
 
 extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
                                int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
-                               void *workspace, size_t workspace_bytes, void *stream) {
+                               const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
   VARQ_CHECK_ARG(host_shape4, "quant_pack: null shape");
   const int64_t *s = host_shape4;
   VARQ_CHECK_ARG(s[0] >= 0 && s[1] >= 0 && s[2] >= 0 && s[3] > 0 && s[3] <= (1 << 20), "quant_pack: bad shape");
@@ -534,6 +548,13 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   p.ws_max = reinterpret_cast<u32 *>(workspace);
   p.ws_min = p.ws_max + ng;
   p.scale = scale; p.zp = zp; p.words = words; p.codes = codes;
+  p.out_mapped = 0; p.out_inner = 1; p.out_delta = 0; p.out_off = 0;
+  if (host_out_map) {
+    VARQ_CHECK_ARG(host_out_map[0] > 0 && host_out_map[1] >= 0 && host_out_map[2] >= 0 && rows % host_out_map[0] == 0,
+                   "quant_pack: output map {rows per block, extra rows per block, first row} = {%lld, %lld, %lld} does not fit %lld rows",
+                   (long long)host_out_map[0], (long long)host_out_map[1], (long long)host_out_map[2], (long long)rows);
+    p.out_mapped = 1; p.out_inner = host_out_map[0]; p.out_delta = host_out_map[1]; p.out_off = host_out_map[2];
+  }
   p.n0 = s[0]; p.n1 = s[1]; p.n2 = s[2];
   p.c = (int)s[3];
   p.keepc = !(reduce_mask & 8);

@@ -106,9 +106,15 @@ def quant_pack_rows_pair_into(x0: torch.Tensor, x1: torch.Tensor, group: int, bi
 # general (cross-row groups) quantize + pack
 # ---------------------------------------------------------------------------
 def quant_pack(x: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: bool = False, eps: float = 1e-12,
-               pack: bool = True) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+               pack: bool = True, out: Optional[torch.Tensor] = None, out_token_dim: Optional[int] = None,
+               out_token: int = 0, scale_out: Optional[torch.Tensor] = None,
+               zp_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """Quantize a 4-D tensor with one group per index of the non-reduced dims.
-    Returns (packed int32 words or int8 codes, scale with keepdim shape, zp or None)."""
+    Returns (packed int32 words or int8 codes, scale with keepdim shape, zp or None).
+    out / out_token_dim / out_token: write the codes into tokens out_token.. of a larger
+    contiguous buffer that has the shape of the result except for more room along
+    out_token_dim (1 or 2); the returned codes are that window of `out`.  scale_out, zp_out:
+    contiguous fp32 buffers of n_groups elements that receive the scale and zero-point."""
     _gpu(x, 'x')
     assert x.dim() == 4, 'expected a 4-D [B,L,H,c] / [B,H,L,c] tensor'
     x = x.contiguous()
@@ -117,22 +123,48 @@ def quant_pack(x: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: boo
     for d in reduce_dims:
         mask |= 1 << (d % 4)
     sshape = [1 if (mask >> d) & 1 else shape[d] for d in range(4)]
-    scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
-    zp = torch.empty_like(scale) if asym else None
-    c = shape[3]
-    if pack:
-        vals = 32 // bits
-        q = torch.empty((*shape[:3], (c + vals - 1) // vals), dtype=torch.int32, device=x.device)
+    n_groups = sshape[0] * sshape[1] * sshape[2] * sshape[3]
+    if scale_out is not None:
+        _gpu(scale_out, 'scale_out')
+        assert scale_out.dtype == torch.float32 and scale_out.is_contiguous() and scale_out.numel() == n_groups
+        scale = scale_out.view(sshape)
     else:
-        q = torch.empty(shape, dtype=torch.int8, device=x.device)
+        scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    zp = None
+    if asym:
+        if zp_out is not None:
+            _gpu(zp_out, 'zp_out')
+            assert zp_out.dtype == torch.float32 and zp_out.is_contiguous() and zp_out.numel() == n_groups
+            zp = zp_out.view(sshape)
+        else:
+            zp = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    c = shape[3]
+    last = (c + 32 // bits - 1) // (32 // bits) if pack else c
+    out_map = None
+    if out is not None:
+        _gpu(out, 'out')
+        d = out_token_dim
+        assert d in (1, 2) and out.is_contiguous() and out.dtype == (torch.int32 if pack else torch.int8)
+        want = shape[:3] + [last]
+        assert all(out.shape[i] == want[i] for i in range(4) if i != d) and 0 <= out_token <= out.shape[d] - shape[d], \
+            f'out {tuple(out.shape)} has no room for {want} at token {out_token} of dim {d}'
+        inner = shape[d] * (shape[2] if d == 1 else 1)            # rows of one block along the token dim
+        per_tok = shape[2] if d == 1 else 1
+        out_map = i64arr([inner, (out.shape[d] - shape[d]) * per_tok, out_token * per_tok])
+        q = out.narrow(d, out_token, shape[d])
+        dst = out
+    else:
+        q = torch.empty((*shape[:3], last), dtype=torch.int32 if pack else torch.int8, device=x.device)
+        dst = q
     lib = _lib.load()
     sh = i64arr(shape)
     ws_bytes = lib.varq_quant_workspace_bytes(sh, mask)
     ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         check(lib.varq_quant_pack(x.data_ptr(), _dt(x), sh, mask, bits, int(asym), eps,
-                                  q.data_ptr() if pack else None, None if pack else q.data_ptr(),
-                                  scale.data_ptr(), _ptr(zp), ws.data_ptr(), ws.numel(), _stream(x)), 'varq_quant_pack')
+                                  dst.data_ptr() if pack else None, None if pack else dst.data_ptr(),
+                                  scale.data_ptr(), _ptr(zp), out_map, ws.data_ptr(), ws.numel(), _stream(x)),
+              'varq_quant_pack')
     return q, scale, zp
 
 

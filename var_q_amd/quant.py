@@ -79,6 +79,24 @@ class _Growable:
         self.buf.narrow(self.dim, self.len, n).copy_(t)
         self.len += n
 
+    def reserve(self, step_shape, dtype, device) -> Optional[torch.Tensor]:
+        """Room for one more step of this shape behind the valid prefix (growing like append);
+        the buffer, or None if it holds tensors of another shape or type."""
+        n = step_shape[self.dim]
+        if self.buf is not None:
+            other = [i for i in range(len(step_shape)) if i != self.dim]
+            if self.buf.dtype != dtype or self.buf.dim() != len(step_shape) or \
+                    any(self.buf.size(i) != step_shape[i] for i in other):
+                return None
+        if self.buf is None or self.len + n > self.buf.size(self.dim):
+            shape = list(step_shape)
+            shape[self.dim] = max(2 * (self.len + n), 64)
+            new = torch.empty(shape, dtype=dtype, device=device)
+            if self.buf is not None and self.len:
+                new.narrow(self.dim, 0, self.len).copy_(self.buf.narrow(self.dim, 0, self.len))
+            self.buf = new
+        return self.buf
+
     def replace(self, t: torch.Tensor):
         self._pending = []
         self.buf, self.len = t, t.size(self.dim)
@@ -114,6 +132,7 @@ class VAR_Q:
         self.scale: Optional[torch.Tensor] = None
         self.zp: Optional[torch.Tensor] = None
         self._pack_meta: Optional[Dict[str, int]] = None
+        self._staged = None
         self._reset_cache()
 
     # The reference derives dim_cat/dim_map once in __init__ and callers later
@@ -136,6 +155,7 @@ class VAR_Q:
         # step with its (head, channel) tables for the methods whose scale is shared by the
         # tokens of a step, a full-size copy of the per-token scales (shaped like the code buffer,
         # [.., capacity, .., groups]) for the others
+        self._staged = None
         self._seg_ends: List[int] = []
         self._tab_scale: Optional[torch.Tensor] = None      # [MAX_TABLE_STEPS, H, c]
         self._tab_zp: Optional[torch.Tensor] = None
@@ -162,11 +182,26 @@ class VAR_Q:
         if not isinstance(x, torch.Tensor) or not x.is_cuda:
             raise VarqError('VAR_Q requires GPU tensors; there is no CPU path in this package')
         m = self.quant_method
+        self._staged = None
         if m == 'G_GROUP':
             q, s, z = ops.quant_pack_rows(x, self.group_size, self.quant_bits, asym=not self.symmetric, eps=self.eps)
-        else:
-            q, s, z = ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
-                                     pack=self.pack_to_int32)
+            return q, s, z
+        # The methods that append (VAR_Q/quant.py:196-201) write the step's codes where cache()
+        # would copy them: behind the valid prefix of the cache buffer.  `quantized_item` is then
+        # a window of that buffer, and cache() only moves the end of the prefix.
+        buf = None
+        if m not in ('G_HEAD_DIM', 'G_TENSOR') and x.dim() == 4 and self._c_item.dim == self.dim_cat:
+            c = x.shape[3]
+            last = (c + 32 // self.quant_bits - 1) // (32 // self.quant_bits) if self.pack_to_int32 else c
+            buf = self._c_item.reserve(list(x.shape[:3]) + [last], torch.int32 if self.pack_to_int32 else torch.int8,
+                                       x.device)
+        if buf is None:
+            return ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
+                                  pack=self.pack_to_int32)
+        q, s, z = ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
+                                 pack=self.pack_to_int32, out=buf, out_token_dim=self.dim_cat,
+                                 out_token=self._c_item.len)
+        self._staged = (buf, self._c_item.len, q)
         return q, s, z
 
     def quant(self, item: torch.Tensor):
@@ -206,7 +241,11 @@ class VAR_Q:
         if m in ('G_SCALE_HEAD_DIM', 'G_SCALE', 'G_TOKEN', 'G_TOKEN_HEAD', 'G_TENSOR', 'G_GROUP', 'G_HEAD'):
             if self._c_item.dim != self.dim_cat:   # layout was re-assigned before the first step
                 self._reset_cache()
-            self._c_item.append(q_cur)
+            st, self._staged = self._staged, None
+            if st is not None and st[0] is self._c_item.buf and st[1] == self._c_item.len and st[2] is q_cur:
+                self._c_item.len += q_cur.size(self.dim_cat)      # the codes are in place already
+            else:
+                self._c_item.append(q_cur)
             self._c_scale.append_later(s_cur)
             if z_cur is not None:
                 self._c_zp.append_later(z_cur)
