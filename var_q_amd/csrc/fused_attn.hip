@@ -1041,11 +1041,14 @@ template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
   constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * kChanTableRows * D * 4 : 0);
   static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-  static bool configured = false;   // above 64 KiB the limit has to be raised once per process
-  if (!configured) {
+  // above 64 KiB the limit has to be raised, once per device the process launches on
+  static bool configured[64] = {false};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev < 0 || !configured[dev]) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    configured = true;
+    if (dev >= 0) configured[dev] = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));

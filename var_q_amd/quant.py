@@ -198,11 +198,25 @@ class VAR_Q:
         if buf is None:
             return ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
                                   pack=self.pack_to_int32)
+        # likewise the scale of a per-(head, channel) method goes straight into the row of the
+        # step tables that cache() would copy it to (`scale` is then a view of that row)
+        s_out = z_out = None
+        k = len(self._seg_ends)
+        if m == 'G_SCALE_HEAD_DIM' and self.pack_to_int32 and k < MAX_TABLE_STEPS:
+            H = x.shape[1 if self.qkv_format == 'BHLc' else 2]
+            self._table_rows(H, x.shape[3], x.device)
+            s_out = self._tab_scale[k]
+            z_out = None if self.symmetric else self._tab_zp[k]
         q, s, z = ops.quant_pack(x, self.dim_map[m], self.quant_bits, asym=not self.symmetric, eps=self.eps,
                                  pack=self.pack_to_int32, out=buf, out_token_dim=self.dim_cat,
-                                 out_token=self._c_item.len)
+                                 out_token=self._c_item.len, scale_out=s_out, zp_out=z_out)
         self._staged = (buf, self._c_item.len, q)
         return q, s, z
+
+    def _table_rows(self, H: int, c: int, device):
+        if self._tab_scale is None or self._tab_scale.shape[1:] != (H, c):
+            self._tab_scale = torch.empty((MAX_TABLE_STEPS, H, c), dtype=torch.float32, device=device)
+            self._tab_zp = None if self.symmetric else torch.empty_like(self._tab_scale)
 
     def quant(self, item: torch.Tensor):
         m = self.quant_method
@@ -277,11 +291,11 @@ class VAR_Q:
             if k >= MAX_TABLE_STEPS:
                 return                                   # fused_attention refuses; the drop-in path is unaffected
             if self._tab_scale is None:
-                self._tab_scale = torch.empty((MAX_TABLE_STEPS, H, c), dtype=torch.float32, device=q_cur.device)
-                self._tab_zp = None if self.zp is None else torch.empty_like(self._tab_scale)
-            self._tab_scale[k].copy_(self.scale.expand(*full).reshape(H, c))
-            if self.zp is not None:
-                self._tab_zp[k].copy_(self.zp.expand(*full).reshape(H, c))
+                self._table_rows(H, c, q_cur.device)
+            if self.scale.data_ptr() != self._tab_scale[k].data_ptr():   # (else quant() wrote the row itself)
+                self._tab_scale[k].copy_(self.scale.expand(*full).reshape(H, c))
+                if self.zp is not None:
+                    self._tab_zp[k].copy_(self.zp.expand(*full).reshape(H, c))
         else:
             ng = self.scale.shape[3]
             shape = (B, H, n, ng) if bhl else (B, n, H, ng)
