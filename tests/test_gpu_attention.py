@@ -150,3 +150,44 @@ def test_head_map_and_strided_cache(dev):
     ref = O.attention_ref(q[:, heads], kd, vd, 0.1)
     _compare(out[:, heads], ref, O.attention_exact(q[:, heads].float(), kd, vd, 0.1), what='head map')
     assert float(out[:, [0, 3]].abs().max()) == 0.0        # other heads untouched
+
+
+def test_full_size_invariants(dev):
+    """Benchmark configuration 4 at its full size (all 32 (batch, head) pairs, 4096 queries,
+    10 521 keys), checked through what the mathematics fixes whatever the size:
+    (i) a V cache whose every element dequantizes to the same value gives that value for every
+    query (the softmax weights sum to one: the denominator and the zero-point terms);
+    (ii) a key limit equal to the cache length is no limit (bit for bit);
+    (iii) the order of the keys does not matter: K and V rows permuted together give the same
+    output to fp32 summation order;
+    (iv) keys beyond the limit have no influence: garbage in rows >= Lk of a longer buffer."""
+    B, H, Lq, Lk, D, bits, g = 2, 16, 4096, 10521, 128, 4, 128
+    gen = torch.Generator(device=dev).manual_seed(404)
+    k = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    v = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    q = torch.randn(B, H, Lq, D, device=dev, generator=gen).bfloat16()
+    kq, vq = ops.quant_pack_rows(k, g, bits, True), ops.quant_pack_rows(v, g, bits, True)
+    scale = 1 / math.sqrt(D)
+    note('fused_attn full size: constant V')
+    code = 5                                              # every nibble of every word
+    vw = torch.full_like(vq[0], int.from_bytes(bytes([code * 17] * 4), 'little', signed=True))
+    vs = torch.rand(B, H, Lk, 1, device=dev, generator=gen) + 0.5
+    vz = code - 1.25 / vs                                  # (code - zp) * scale = 1.25 for every token
+    out = ops.fused_attn(q, *kq, vw, vs, vz, bits, bits, Lk, scale)
+    assert float((out.float() - 1.25).abs().max()) <= 2 ** -7, 'softmax weights do not sum to one'
+    note('fused_attn full size: limit == length')
+    base = ops.fused_attn(q, *kq, *vq, bits, bits, Lk, scale)
+    lim = torch.full((Lq,), Lk, dtype=torch.int32, device=dev)
+    assert torch.equal(ops.fused_attn(q, *kq, *vq, bits, bits, Lk, scale, kv_limit=lim), base)
+    note('fused_attn full size: permuted keys')
+    perm = torch.randperm(Lk, device=dev, generator=gen)
+    pk, pv = [t[:, :, perm].contiguous() for t in kq], [t[:, :, perm].contiguous() for t in vq]
+    other = ops.fused_attn(q, *pk, *pv, bits, bits, Lk, scale)
+    span = max(1.0, float(base.float().abs().max()))
+    assert float((other.float() - base.float()).abs().max()) <= 2e-2 * span / 4
+    assert float(torch.nn.functional.cosine_similarity(other.flatten().double(), base.flatten().double(), dim=0)) >= 0.99999
+    note('fused_attn full size: rows beyond the length')
+    longer = [torch.cat([t, torch.full_like(t[:, :, :300], 0x7f if t.dtype == torch.int32 else 1e30)], dim=2).contiguous()
+              for t in (*kq, *vq)]
+    assert torch.equal(ops.fused_attn(q, *longer, bits, bits, Lk, scale), base)
+    torch.cuda.synchronize()
