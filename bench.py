@@ -144,44 +144,56 @@ def c3_rates(torch, dev, reps=20, warm=5):
 
 
 def shipped_rule_latency(torch, dev, passes=5, warm=2):
-    """The rule of the shipped JSON files (G_SCALE_HEAD_DIM, 8 bits, layout BHLc) over the 13
-    Infinity scales, B=2 (one image, CFG pair), H=16, D=128, one layer: per scale quantize +
-    cache K and V with the drop-in quantizers, then attend.  'dropin' dequantizes the whole
-    cache to fp32 and calls torch's scaled_dot_product_attention in bf16 (what the reference
-    does), 'fused' attends over the packed caches (`fused_attention`)."""
+    """The rules of the shipped JSON files (G_SCALE_HEAD_DIM, 8 bits), one layer, per scale
+    quantize + cache K and V with the drop-in quantizers, then attend:
+    Infinity-VAR_Q-8.json (layout BHLc) over the 13 Infinity scales, B=2 (one image, CFG pair),
+    H=16, D=128; VAR-VAR_Q-8.json (layout BLHc) over the 10 VAR scales, B=64, H=16, D=64.
+    'dropin' dequantizes the whole cache to fp32 and calls torch's
+    scaled_dot_product_attention in bf16 (what the reference does), 'fused' attends over the
+    packed caches (`fused_attention`)."""
     import torch.nn.functional as F
     from var_q_amd import VAR_Q
     from var_q_amd.quant import fused_attention
-    from var_q_amd.schedules import INFINITY_PATCH_NUMS
-    B, H, D = 2, 16, 128
-    gd = torch.Generator(device=dev).manual_seed(7007)
-    steps = [tuple(torch.randn(B, H, pn * pn, D, device=dev, generator=gd).bfloat16() for _ in range(3))
-             for pn in INFINITY_PATCH_NUMS]
-    scale = 1.0 / math.sqrt(D)
+    from var_q_amd.schedules import INFINITY_PATCH_NUMS, VAR_PATCH_NUMS
 
-    def one_pass(fused):
-        kq, vq = VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM'), VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM')
-        for q, k, v in steps:
-            if fused:
-                for quantizer, item in ((kq, k), (vq, v)):
-                    quantizer.quant(item)
-                    quantizer.cache()
-                fused_attention(q, kq, vq, scale)
-            else:
-                kk, vv = kq.use_var_q(k), vq.use_var_q(v)
-                F.scaled_dot_product_attention(q, kk.to(torch.bfloat16), vv.to(torch.bfloat16), scale=scale)
+    def run(fmt, B, H, D, patch_nums, seed):
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        shape = (lambda n: (B, H, n, D)) if fmt == 'BHLc' else (lambda n: (B, n, H, D))
+        steps = [tuple(torch.randn(*shape(pn * pn), device=dev, generator=gd).bfloat16() for _ in range(3))
+                 for pn in patch_nums]
+        scale = 1.0 / math.sqrt(D)
+        heads_first = (lambda t: t) if fmt == 'BHLc' else (lambda t: t.transpose(1, 2))
+
+        def one_pass(fused):
+            kq, vq = VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM'), VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM')
+            for q, k, v in steps:
+                if fused:
+                    for quantizer, item in ((kq, k), (vq, v)):
+                        quantizer.quant(item)
+                        quantizer.cache()
+                    fused_attention(q, kq, vq, scale)
+                else:
+                    kk, vv = kq.use_var_q(k), vq.use_var_q(v)
+                    F.scaled_dot_product_attention(heads_first(q), heads_first(kk.to(torch.bfloat16)),
+                                                   heads_first(vv.to(torch.bfloat16)), scale=scale)
+
+        res = {}
+        for name, fused in (('dropin_dequant_sdpa_ms', False), ('fused_ms', True)):
+            for _ in range(warm):
+                one_pass(fused)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(passes):
+                one_pass(fused)
+            torch.cuda.synchronize()
+            res[name] = round((time.perf_counter() - t0) / passes * 1e3, 3)
+        return res
 
     out = {'workload': 'shipped rule G_SCALE_HEAD_DIM 8-bit BHLc, 13 Infinity scales, B=2 H=16 D=128, one layer: '
                        'quantize + cache + attention per scale'}
-    for name, fused in (('dropin_dequant_sdpa_ms', False), ('fused_ms', True)):
-        for _ in range(warm):
-            one_pass(fused)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(passes):
-            one_pass(fused)
-        torch.cuda.synchronize()
-        out[name] = round((time.perf_counter() - t0) / passes * 1e3, 3)
+    out.update(run('BHLc', 2, 16, 128, INFINITY_PATCH_NUMS, 7007))
+    out['var_d16'] = {'workload': 'shipped rule G_SCALE_HEAD_DIM 8-bit BLHc, 10 VAR scales, B=64 H=16 D=64, one layer'}
+    out['var_d16'].update(run('BLHc', 64, 16, 64, VAR_PATCH_NUMS, 7008))
     return out
 
 
