@@ -25,8 +25,34 @@ def _gpu(t: torch.Tensor, name: str) -> torch.Tensor:
     return t
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """Handle of the current stream of the tensor's device."""
+    if _raw_stream is not None:
+        idx = t.device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` that does nothing when d is current already (every call here
+    is on the hot path of a generation step)."""
+    __slots__ = ('idx', 'prev')
+
+    def __init__(self, device: torch.device):
+        self.idx, self.prev = device.index, -1
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -55,7 +81,7 @@ def quant_pack_rows(x: torch.Tensor, group: int, bits: int, asym: bool = True, e
     scale = torch.empty((*lead, c // group), dtype=torch.float32, device=x.device)
     zp = torch.empty_like(scale) if asym else None
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         check(lib.varq_quant_pack_rows(x.data_ptr(), _dt(x), n_rows, c, group, bits, int(asym), eps, None, None,
                                        words.data_ptr(), scale.data_ptr(), _ptr(zp), _stream(x)), 'varq_quant_pack_rows')
     return words, scale, zp
@@ -73,7 +99,7 @@ def quant_pack_rows_into(x: torch.Tensor, group: int, bits: int, asym: bool, eps
     n_rows = x.numel() // c
     assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         check(lib.varq_quant_pack_rows(x.data_ptr(), _dt(x), n_rows, c, group, bits, int(asym), eps, i64arr(rowmap),
                                        _ptr(slot), words.data_ptr(), scale.data_ptr(), _ptr(zp), _stream(x)),
               'varq_quant_pack_rows')
@@ -94,7 +120,7 @@ def quant_pack_rows_pair_into(x0: torch.Tensor, x1: torch.Tensor, group: int, bi
     n_rows = x0.numel() // c
     assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
     lib = _lib.load()
-    with torch.cuda.device(x0.device):
+    with _on_device(x0.device):
         check(lib.varq_quant_pack_rows2(x0.data_ptr(), x1.data_ptr(), _dt(x0), n_rows, c, group, bits, int(asym), eps,
                                         i64arr(rowmap), _ptr(slot),
                                         out0[0].data_ptr(), out0[1].data_ptr(), _ptr(out0[2]),
@@ -160,7 +186,7 @@ def quant_pack(x: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: boo
     sh = i64arr(shape)
     ws_bytes = lib.varq_quant_workspace_bytes(sh, mask)
     ws = torch.empty(max(ws_bytes, 8), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         check(lib.varq_quant_pack(x.data_ptr(), _dt(x), sh, mask, bits, int(asym), eps,
                                   dst.data_ptr() if pack else None, None if pack else dst.data_ptr(),
                                   scale.data_ptr(), _ptr(zp), out_map, ws.data_ptr(), ws.numel(), _stream(x)),
@@ -179,7 +205,7 @@ def pack(codes: torch.Tensor, bits: int) -> torch.Tensor:
     rows = codes.numel() // c if c else 0
     words = torch.empty((*lead, (c + vals - 1) // vals), dtype=torch.int32, device=codes.device)
     lib = _lib.load()
-    with torch.cuda.device(codes.device):
+    with _on_device(codes.device):
         check(lib.varq_pack(codes.data_ptr(), rows, c, bits, words.data_ptr(), _stream(codes)), 'varq_pack')
     return words
 
@@ -191,7 +217,7 @@ def unpack(words: torch.Tensor, c: int, bits: int) -> torch.Tensor:
     rows = words.numel() // w if w else 0
     codes = torch.empty((*lead, c), dtype=torch.int8, device=words.device)
     lib = _lib.load()
-    with torch.cuda.device(words.device):
+    with _on_device(words.device):
         check(lib.varq_unpack(words.data_ptr(), rows, c, bits, codes.data_ptr(), _stream(words)), 'varq_unpack')
     return codes
 
@@ -232,7 +258,7 @@ def dequant(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], c:
         shape = [1, 1, n0 * n1 * n2, c]
     elif strides[0] == 0 and strides[1] == 0:
         pass
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         check(lib.varq_dequant(q.data_ptr() if packed else None, None if packed else q.data_ptr(),
                                scale.data_ptr(), _ptr(zp), i64arr(shape), i64arr(strides), group, bits, None,
                                out.data_ptr(), _DT[out_dtype], _stream(q)), 'varq_dequant')
@@ -249,7 +275,7 @@ def dequant_window(words: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.
     assert packed or words.dtype == torch.int8
     out = torch.empty(tuple(shape4), dtype=out_dtype, device=words.device)
     lib = _lib.load()
-    with torch.cuda.device(words.device):
+    with _on_device(words.device):
         check(lib.varq_dequant(words.data_ptr() if packed else None, None if packed else words.data_ptr(),
                                scale.data_ptr(), _ptr(zp), i64arr(shape4),
                                i64arr(scale_strides4), group, bits, i64arr(in_rowmap), out.data_ptr(),
@@ -284,7 +310,7 @@ def qkv_prepare_append(qkv: torch.Tensor, q_out: torch.Tensor, group: int, bits:
         _gpu(q_scale_mul, 'q_scale_mul')
         assert q_scale_mul.dtype == torch.float32 and q_scale_mul.numel() == H and q_scale_mul.is_contiguous()
     lib = _lib.load()
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         check(lib.varq_qkv_prepare_append(qkv.data_ptr(), _dt(qkv), B, L, H, c, _ptr(q_scale_mul), int(l2norm), norm_eps,
                                           _ptr(cos), _ptr(sin), token_start, q_out.data_ptr(), group, bits, int(asym), eps,
                                           i64arr(rowmap), _ptr(slot), k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp),
@@ -352,7 +378,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     else:
         assert Hkv == Hq
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         ws, ws_bytes = _attn_workspace(lib, B, Hkv, Lq, Lk, D, 1, splits, q.device)
         check(lib.varq_fused_attn(q.data_ptr(), out.data_ptr(),
                                   k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp), k_bits, k_group,
@@ -409,7 +435,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
     else:
         assert Hkv == Hq
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         ws, ws_bytes = _attn_workspace(lib, B, Hkv, Lq, Lk, D, nseg, splits, q.device)
         check(lib.varq_fused_attn_channel(q.data_ptr(), out.data_ptr(),
                                           k_words.data_ptr(), k_chan_scale.data_ptr(), _ptr(k_chan_zp),
