@@ -103,3 +103,54 @@ def test_library_choice_matches_one_workgroup(dev):
     one = ops.fused_attn(q, *kq, *vq, bits, bits, Lk, 1 / math.sqrt(D), splits=1)
     torch.cuda.synchronize()
     assert float((auto.double() - one.double()).abs().max()) <= 2e-2 * max(1.0, float(one.abs().max())) / 4
+
+
+@pytest.mark.parametrize('Lq', [1, 20, 64, 65, 128])
+@pytest.mark.parametrize('D,gk,gv,bits', [(64, 64, 64, 4), (64, 32, 32, 8), (64, 32, 64, 2)])
+def test_many_heads_few_queries_token_scales(dev, Lq, D, gk, gv, bits):
+    """More (batch, head) pairs than compute units with at most 128 queries each -- the first
+    steps of a schedule at a large batch -- run as workgroups of two or four wavefronts, two
+    to a compute unit.  Against the oracle, and bit for bit against the same data attended in two halves
+    (each half has too few pairs for that path)."""
+    B, H, Lk = 33, 8, 150
+    run_token(dev, B, H, Lq, Lk, D, bits, gk, gv, seed=700 + Lq + bits, what='small workgroups', splits=1)
+    gen = torch.Generator(device=dev).manual_seed(Lq + bits)
+    k = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    v = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    q = torch.randn(B, H, Lq, D, device=dev, generator=gen).bfloat16()
+    kq = [ops.quant_pack_rows(k, gk, bits, True)[i] for i in range(3)]
+    vq = [ops.quant_pack_rows(v, gv, bits, True)[i] for i in range(3)]
+    note('small workgroups vs halves', (Lq, D, gk, gv, bits))
+    whole = ops.fused_attn(q, *kq, *vq, bits, bits, Lk, 0.125, splits=1)
+    halves = [ops.fused_attn(q[a:b].contiguous(), *[t[a:b].contiguous() for t in kq], *[t[a:b].contiguous() for t in vq],
+                             bits, bits, Lk, 0.125, splits=1) for a, b in ((0, 16), (16, 33))]
+    torch.cuda.synchronize()
+    assert torch.equal(whole, torch.cat(halves, 0))
+
+
+@pytest.mark.parametrize('fmt_blhc', [False, True])
+def test_many_heads_few_queries_stepwise_tables(dev, fmt_blhc):
+    """The same for a cache filled step by step with per-(head, channel) tables (the VAR
+    rule at a large batch), in both layouts."""
+    B, H, D, bits = 40, 8, 64, 8
+    steps = [1, 4, 9, 16, 25, 36]
+    _stepwise(dev, B, H, D, steps, bits, False, 36, seed=801, what='small workgroups stepwise', outlier_mul=1.0)
+    _stepwise(dev, B, H, D, steps, 4, True, 20, seed=802, what='small workgroups stepwise asym', outlier_mul=1.0, splits=1)
+    _stepwise(dev, B, H, D, steps + [49], 8, False, 100, seed=803, what='small workgroups stepwise, four wavefronts',
+              outlier_mul=1.0, splits=1)
+    L, nseg = sum(steps), len(steps)
+    ends = [sum(steps[:i + 1]) for i in range(nseg)]
+    gen = torch.Generator(device=dev).manual_seed(9)
+    kw = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, L, D * bits // 32), device=dev, generator=gen, dtype=torch.int64).int()
+    vw = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, L, D * bits // 32), device=dev, generator=gen, dtype=torch.int64).int()
+    ks = (torch.rand(nseg, H, D, device=dev, generator=gen) * 0.02 + 0.01).contiguous()
+    vs = (torch.rand(nseg, H, D, device=dev, generator=gen) * 0.02 + 0.01).contiguous()
+    q = torch.randn(B, H, 36, D, device=dev, generator=gen).bfloat16()
+    tr = (lambda t: t.transpose(1, 2).contiguous()) if fmt_blhc else (lambda t: t)
+    lay = 'BLHc' if fmt_blhc else 'BHLc'
+    note('small workgroups stepwise vs halves', lay)
+    whole = ops.fused_attn_channel(tr(q), tr(kw), ks, None, tr(vw), vs, None, bits, L, 0.1, seg_ends=ends, splits=1, layout=lay)
+    halves = [ops.fused_attn_channel(tr(q[a:b]), tr(kw[a:b]), ks, None, tr(vw[a:b]), vs, None, bits, L, 0.1, seg_ends=ends,
+                                     splits=1, layout=lay) for a, b in ((0, 20), (20, 40))]
+    torch.cuda.synchronize()
+    assert torch.equal(whole, torch.cat(halves, 0))

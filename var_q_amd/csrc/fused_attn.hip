@@ -56,6 +56,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(u32)))) u32 u32x4_t;
 constexpr int NW = 8;          // wavefronts per workgroup
 constexpr int NT = NW * 64;    // threads per workgroup
 constexpr int BM = NW * 32;    // queries per workgroup (32 per wavefront)
+// Smaller workgroups for launches of many (batch, head) pairs with at most 64 or 128
+// queries each (the first steps of a scale schedule at a large batch): two or four
+// wavefronts, so that two workgroups share a compute unit instead of one workgroup whose
+// other wavefronts have no queries.
 constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
@@ -272,10 +276,12 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
 // When the tables change along the keys (segments), key tiles never straddle a segment:
 // at a boundary the Q operands are rebuilt with the new K table and the output
 // accumulators are re-expressed in units of the new V table.
-template <int D, int BITS, int GK, int GV, bool CHAN>
-__global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8>
+__global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
+  constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
+  static_assert(NW >= NSK && NW >= NSV && NW >= 2, "one wavefront per K group and per V group stages the parameters");
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
   constexpr int NDB = D / 32;               // 32-row blocks of O^T
@@ -640,7 +646,7 @@ __global__ __launch_bounds__(NT, 2) void fused_attn_kernel(AttnParams p) {
   // ---- prologue: V tiles 0 and 1 staged, K and V of tile 0 widened, K of tile 1 and V
   //      of tile 2 in registers ------------------------------------------------------------
   if (tid < 3) lds_flag[tid] = 0;
-  if (tid < 3 * RSR) lds_wz[((tid / RSR) * 8 + 7) * RSR + tid % RSR] = 0;   // the all-zero row of each slot
+  for (int i = tid; i < 3 * RSR; i += NT) lds_wz[((i / RSR) * 8 + 7) * RSR + i % RSR] = 0;   // the all-zero row of each slot
   __syncthreads();
   if (n_tiles > 0) { prefetch_k(0); prefetch(0); }
   // the query values, behind the first tile's requests and ahead of the table loads: one
@@ -1037,8 +1043,10 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
   *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_bf16_rne(acc[0] * inv, acc[1] * inv), pack_bf16_rne(acc[2] * inv, acc[3] * inv));
 }
 
-template <int D, int BITS, int GK, int GV, bool CHAN = false>
-void launch(const AttnParams &p, hipStream_t st) {
+int device_cus();
+
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV>
+void launch_shape(const AttnParams &p, hipStream_t st) {
   constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * kChanTableRows * D * 4 : 0);
   static_assert(lds_bytes <= 160 * 1024, "LDS budget");
   // above 64 KiB the limit has to be raised, once per device the process launches on
@@ -1046,17 +1054,31 @@ void launch(const AttnParams &p, hipStream_t st) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !configured[dev]) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (dev >= 0) configured[dev] = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN>), grid, dim3(NT), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV>), grid, dim3(NWV * 64), lds_bytes, st, p);
   if (p.nsplit > 1) {
     const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
     hipLaunchKernelGGL((combine_splits_kernel<D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
   }
+}
+
+template <int D, int BITS, int GK, int GV, bool CHAN = false>
+void launch(const AttnParams &p, hipStream_t st) {
+  if constexpr (D == 64) {
+    // more (batch, head) pairs than compute units, at most four wavefronts of queries each:
+    // small workgroups, two to a compute unit (same arithmetic, same results)
+    if (p.Lq <= 128 && p.bh_total > device_cus()) {
+      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2>(p, st);
+      else launch_shape<D, BITS, GK, GV, CHAN, 4>(p, st);
+      return;
+    }
+  }
+  launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
 }
 
 template <int D, int BITS>
