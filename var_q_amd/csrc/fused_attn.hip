@@ -718,7 +718,16 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     if constexpr (CHAN) {
       // (the Q operands first: with the accumulator arithmetic in front of it the register
       // allocator spills, and spills here cost scratch traffic at every boundary)
-      load_q(seg_new, std::false_type{});
+      // The old Q operands are dead: at D=64 their registers receive the new query values at
+      // once, in flight under the accumulator arithmetic.  At D=128 that order makes the
+      // register allocator spill (and gains nothing): there the operands are rebuilt first.
+      constexpr bool OVERLAP_Q = (D == 64);
+      if constexpr (OVERLAP_Q) {
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
+      } else {
+        load_q(seg_new, std::false_type{});
+      }
       __builtin_amdgcn_sched_barrier(0);
       const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
@@ -747,6 +756,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
           }
           __builtin_amdgcn_sched_barrier(0);   // one slice's registers at a time
         }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (OVERLAP_Q) load_q(seg_new, std::true_type{});
       l_prev = l_sum;
       seg_a = seg_new;
     }
