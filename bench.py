@@ -149,11 +149,11 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
     Infinity-VAR_Q-8.json (layout BHLc) over the 13 Infinity scales, B=2 (one image, CFG pair),
     H=16, D=128; VAR-VAR_Q-8.json (layout BLHc) over the 10 VAR scales, B=64, H=16, D=64.
     'dropin' dequantizes the whole cache to fp32 and calls torch's
-    scaled_dot_product_attention in bf16 (what the reference does), 'fused' attends over the
-    packed caches (`fused_attention`)."""
+    scaled_dot_product_attention in bf16 (what the reference does), 'fused' quantizes, caches and
+    attends over the packed caches (`fused_step`)."""
     import torch.nn.functional as F
     from var_q_amd import VAR_Q
-    from var_q_amd.quant import fused_attention
+    from var_q_amd.quant import fused_step
     from var_q_amd.schedules import INFINITY_PATCH_NUMS, VAR_PATCH_NUMS
 
     def run(fmt, B, H, D, patch_nums, seed):
@@ -168,10 +168,7 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
             kq, vq = VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM'), VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM')
             for q, k, v in steps:
                 if fused:
-                    for quantizer, item in ((kq, k), (vq, v)):
-                        quantizer.quant(item)
-                        quantizer.cache()
-                    fused_attention(q, kq, vq, scale)
+                    fused_step(q, k, v, kq, vq, scale)
                 else:
                     kk, vv = kq.use_var_q(k), vq.use_var_q(v)
                     F.scaled_dot_product_attention(heads_first(q), heads_first(kk.to(torch.bfloat16)),

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 4
+#define VARQ_ABI_VERSION 5
 
 enum varq_status {
   VARQ_OK = 0,
@@ -111,6 +111,16 @@ size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask);
 int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
                     int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
                     const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream);
+/*
+ * The same for two tensors of one shape and dtype with separate outputs and a shared output
+ * map -- K and V of a step, which the reference quantizes one after the other
+ * (Infinity/infinity/models/basic.py:329-330) -- in the same three launches.  The workspace
+ * holds 2 * varq_quant_workspace_bytes(...) bytes.  Results are those of two varq_quant_pack calls.
+ */
+int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, const int64_t *host_shape4, int reduce_mask,
+                     int bits, int asym, float eps, int32_t *words0, int8_t *codes0, float *scale0, float *zp0,
+                     int32_t *words1, int8_t *codes1, float *scale1, float *zp1,
+                     const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream);
 
 /* VAR_Q/pack_unpack.py:107-134 (and its CPU twin 177-196): int8 codes [rows,c]
  * -> int32 words [rows, ceil(c*bits/32)], zero padding in the last word. */

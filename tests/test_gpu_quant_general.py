@@ -187,3 +187,25 @@ def test_codes_written_into_a_window_of_a_larger_buffer(dev, token_dim, mask):
         fill = buf.new_full((), 0x5a if not pack else 0x5a5a5a5a)
         assert bool((buf.narrow(token_dim, 0, at) == fill).all())
         assert bool((buf.narrow(token_dim, at + shape[token_dim], cap - at - shape[token_dim]) == fill).all())
+
+
+@pytest.mark.parametrize('mask', [0b0101, 0b0011, 0b1111, 0b1000, 0b0110, 0b0001])
+def test_two_tensors_in_the_same_launches(dev, mask):
+    """K and V of a step through `varq_quant_pack2`: the results of two separate calls, bit
+    for bit, on tiled shapes (one launch set for both) and on a shape of the scalar kernels
+    (c = 20: one after the other through the same workspace)."""
+    dims = tuple(d for d in range(4) if (mask >> d) & 1)
+    g = torch.Generator().manual_seed(1200 + mask)
+    for shape, dtype, bits, asym, pack in [((2, 16, 300, 128), torch.bfloat16, 8, False, True),
+                                           ((3, 40, 5, 64), torch.float32, 4, True, True),
+                                           ((2, 3, 50, 20), torch.bfloat16, 8, True, False),
+                                           ((64, 2, 33, 32), torch.float16, 2, True, True)]:
+        x0 = (torch.randn(*shape, generator=g) * 2).to(dtype).to(dev)
+        x1 = (torch.randn(*shape, generator=g) * 5 + 1).to(dtype).to(dev)
+        note('general pair', mask, shape, dtype, bits, asym, pack)
+        a, b = ops.quant_pack_pair(x0, x1, dims, bits, asym=asym, pack=pack)
+        torch.cuda.synchronize()
+        for got, x in ((a, x0), (b, x1)):
+            want = ops.quant_pack(x, dims, bits, asym=asym, pack=pack)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+            assert (got[2] is None) == (want[2] is None) and (got[2] is None or torch.equal(got[2], want[2]))

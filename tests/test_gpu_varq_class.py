@@ -175,3 +175,36 @@ def test_quant_writes_into_the_cache_buffer(dev, fmt, pack):
     assert torch.equal(codes.cpu(), ref.cached_item)
     assert torch.equal(gpu.cached_scale.cpu(), ref.cached_scale)
     assert torch.equal(gpu.dequant_all().cpu(), ref.dequant_all())
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('bits,sym', [(8, True), (4, False)])
+def test_fused_step_leaves_the_state_of_quant_and_cache(dev, fmt, bits, sym):
+    """`fused_step` (one library call per tensor for the shipped rule) against the general
+    sequence quant(), cache(), fused_attention(): same attention output bit for bit and the
+    same quantizer state afterwards -- current item, scale, caches, tables, segment ends --
+    at every step; other rules take the general methods inside fused_step."""
+    from var_q_amd.quant import fused_attention, fused_step
+    ks, vs = _steps(fmt, torch.bfloat16, seed=61), _steps(fmt, torch.bfloat16, seed=62)
+    g = torch.Generator().manual_seed(63)
+    for method in ('G_SCALE_HEAD_DIM', 'G_TOKEN'):
+        a = [VAR_Q(bits, fmt, method, symmetric=sym) for _ in range(2)]
+        b = [VAR_Q(bits, fmt, method, symmetric=sym) for _ in range(2)]
+        for k, v in zip(ks, vs):
+            q = torch.randn(*k.shape, generator=g).bfloat16().to(dev)
+            k, v = k.to(dev), v.to(dev)
+            note('fused_step', fmt, bits, sym, method, tuple(k.shape))
+            for qz, item in ((a[0], k), (a[1], v)):
+                qz.quant(item)
+                qz.cache()
+            want = fused_attention(q, a[0], a[1], 0.125)
+            got = fused_step(q, k, v, b[0], b[1], 0.125)
+            assert torch.equal(got, want)
+            for x, y in zip(a, b):
+                assert torch.equal(x.quantized_item, y.quantized_item) and torch.equal(x.scale, y.scale)
+                assert x.scale.shape == y.scale.shape and x._pack_meta == y._pack_meta and x._seg_ends == y._seg_ends
+                assert (x.zp is None) == (y.zp is None) and (x.zp is None or torch.equal(x.zp, y.zp))
+                assert torch.equal(x.cached_item, y.cached_item) and torch.equal(x.cached_scale, y.cached_scale)
+                assert x.cached_scale.shape == y.cached_scale.shape
+                assert (x.cached_zp is None) == (y.cached_zp is None) and (x.cached_zp is None or torch.equal(x.cached_zp, y.cached_zp))
+                assert torch.equal(x.dequant_all(), y.dequant_all())

@@ -46,7 +46,21 @@ struct GenParams {
   // [B,H,cap,..] is (n, cap - n, len), a step [B,n,H,c] into [B,cap,H,..] is (n*H, (cap - n)*H, len*H).
   int out_mapped;
   int64_t out_inner, out_delta, out_off;
+  // a second tensor of the same shape in the same launches (blockIdx.y == 1): its input,
+  // its outputs and the distance (in 4-byte words) to its part of the workspace
+  const void *x1;
+  float *scale1, *zp1;
+  int32_t *words1;
+  int8_t *codes1;
+  int64_t ws1;
 };
+
+// the tensor a workgroup of the tiled kernels works on
+__device__ __forceinline__ bool take_second(GenParams &p) {
+  if (blockIdx.y == 0) return false;
+  p.x = p.x1; p.scale = p.scale1; p.zp = p.zp1; p.words = p.words1; p.codes = p.codes1;
+  return true;
+}
 
 __device__ __forceinline__ int64_t out_row(const GenParams &p, int64_t row) {
   return p.out_mapped ? row + (row / p.out_inner) * p.out_delta + p.out_off : row;
@@ -143,6 +157,7 @@ __global__ __launch_bounds__(256) void minmax_tiled_kernel(GenParams p, Plan pl,
   constexpr int NV = KEEPC ? 8 : 1;
   __shared__ float lds_mx[256 * NV];
   __shared__ float lds_mn[ASYM ? 256 * NV : 1];
+  if (take_second(p)) { part_max += p.ws1; part_min += p.ws1; }
   const Lane l = decode(pl);
   float mx[NV], mn[NV];
 #pragma unroll
@@ -215,6 +230,7 @@ __global__ __launch_bounds__(256) void finalize_tiled_kernel(GenParams p, int Z,
                                                              const float *part_min, float *rinv, u32 *plain) {
   __shared__ float lds_mx[256];
   __shared__ float lds_mn[256];
+  if (take_second(p)) { part_max += p.ws1; part_min += p.ws1; rinv += p.ws1; plain += p.ws1; }
   const int gpb = 256 / ZL;                       // groups per block
   const int gl = threadIdx.x % gpb, zl = threadIdx.x / gpb;
   const int64_t g = (int64_t)blockIdx.x * gpb + gl;
@@ -255,6 +271,7 @@ __global__ __launch_bounds__(256) void finalize_tiled_kernel(GenParams p, int Z,
 template <int DT, bool KEEPC>
 __global__ __launch_bounds__(256) void quant_tiled_kernel(GenParams p, Plan pl, const float *rinv, const u32 *plain) {
   constexpr int NV = KEEPC ? 8 : 1;
+  if (take_second(p)) { rinv += p.ws1; plain += p.ws1; }
   const Lane l = decode(pl);
   // 2-bit words are assembled from two adjacent column lanes: idle lanes must still reach the shuffle
   const bool live = l.live;
@@ -447,7 +464,9 @@ int run_tiled(GenParams &p, const Plan &pl, void *workspace, hipStream_t st) {
   u32 *plain = reinterpret_cast<u32 *>(rinv + ng);
   float *part_max = rinv + 2 * ng;
   float *part_min = part_max + (int64_t)pl.Z * ng;
-  dim3 grid((unsigned)((int64_t)pl.nko * pl.tilesQ * pl.Z));
+  const unsigned nt = p.x1 ? 2u : 1u;   // tensors per launch (grid.y)
+  p.ws1 = (int64_t)(plan_workspace_bytes(pl, ng) / sizeof(float));
+  dim3 grid((unsigned)((int64_t)pl.nko * pl.tilesQ * pl.Z), nt);
   if (p.asym) {
     if (p.keepc) hipLaunchKernelGGL((minmax_tiled_kernel<DT, true, true>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
     else hipLaunchKernelGGL((minmax_tiled_kernel<DT, true, false>), grid, dim3(256), 0, st, p, pl, part_max, part_min);
@@ -458,7 +477,7 @@ int run_tiled(GenParams &p, const Plan &pl, void *workspace, hipStream_t st) {
   // z-lanes per group in the finalize kernel: enough threads in total, no more lanes than partials
   int ZL = 1;
   while (ZL < 256 && ZL < pl.Z && ng * ZL < 65536) ZL <<= 1;
-  dim3 fgrid((unsigned)((ng + 256 / ZL - 1) / (256 / ZL)));
+  dim3 fgrid((unsigned)((ng + 256 / ZL - 1) / (256 / ZL)), nt);
   if (p.asym)
     hipLaunchKernelGGL((finalize_tiled_kernel<true>), fgrid, dim3(256), 0, st, p, pl.Z, ZL, part_max, part_min, rinv, plain);
   else
@@ -470,7 +489,7 @@ int run_tiled(GenParams &p, const Plan &pl, void *workspace, hipStream_t st) {
     pb.steps_per_chunk = min_spc < pb.steps ? min_spc : pb.steps;
     pb.Z = (pb.steps + pb.steps_per_chunk - 1) / pb.steps_per_chunk;
   }
-  dim3 bgrid((unsigned)((int64_t)pb.nko * pb.tilesQ * pb.Z));
+  dim3 bgrid((unsigned)((int64_t)pb.nko * pb.tilesQ * pb.Z), nt);
   if (p.keepc) hipLaunchKernelGGL((quant_tiled_kernel<DT, true>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
   else hipLaunchKernelGGL((quant_tiled_kernel<DT, false>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
   return 0;
@@ -519,9 +538,13 @@ extern "C" size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int red
   return (size_t)ng * 2 * sizeof(u32);
 }
 
-extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
-                               int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
-                               const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
+namespace {
+// x1 != NULL: a second tensor of the same shape with its own outputs, in the same launches
+// where the tiled kernels apply, one after the other through the same workspace otherwise
+int quant_pack_impl(const void *x, const void *x1, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
+                    int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
+                    int32_t *words1, int8_t *codes1, float *scale1, float *zp1,
+                    const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
   VARQ_CHECK_ARG(host_shape4, "quant_pack: null shape");
   const int64_t *s = host_shape4;
   VARQ_CHECK_ARG(s[0] >= 0 && s[1] >= 0 && s[2] >= 0 && s[3] > 0 && s[3] <= (1 << 20), "quant_pack: bad shape");
@@ -534,11 +557,15 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   VARQ_CHECK_ARG(words || codes, "quant_pack: no output requested");
   VARQ_CHECK_ARG(scale && (!asym || zp), "quant_pack: scale/zp output missing");
   VARQ_CHECK_ARG(x && workspace, "quant_pack: null pointer");
+  if (x1) {
+    VARQ_CHECK_ARG((!words == !words1) && (!codes == !codes1) && scale1 && (!asym || zp1),
+                   "quant_pack: the second tensor needs the same kinds of output as the first");
+  }
   const int64_t ng = count_groups(s, reduce_mask);
   Plan pl;
   // the tiled kernels pack whole words per octet: c*bits must fill words (always true for 4 and 8 bits)
   const bool tiled = make_plan(s, reduce_mask, ng, pl) && (!words || (s[3] * bits) % 32 == 0);
-  const size_t need = tiled ? plan_workspace_bytes(pl, ng) : (size_t)ng * 2 * sizeof(u32);
+  const size_t need = tiled ? plan_workspace_bytes(pl, ng) * (x1 ? 2 : 1) : (size_t)ng * 2 * sizeof(u32);
   if (workspace_bytes < need)
     return varq_set_error(VARQ_ERR_WORKSPACE, "quant_pack: workspace %zu < %zu bytes", workspace_bytes, need);
   VARQ_CHECK_ARG(rows * s[3] < (1ll << 40), "quant_pack: tensor too large");
@@ -548,6 +575,7 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   p.ws_max = reinterpret_cast<u32 *>(workspace);
   p.ws_min = p.ws_max + ng;
   p.scale = scale; p.zp = zp; p.words = words; p.codes = codes;
+  p.x1 = nullptr; p.scale1 = nullptr; p.zp1 = nullptr; p.words1 = nullptr; p.codes1 = nullptr; p.ws1 = 0;
   p.out_mapped = 0; p.out_inner = 1; p.out_delta = 0; p.out_off = 0;
   if (host_out_map) {
     VARQ_CHECK_ARG(host_out_map[0] > 0 && host_out_map[1] >= 0 && host_out_map[2] >= 0 && rows % host_out_map[0] == 0,
@@ -576,12 +604,35 @@ extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_s
   p.eps = eps;
   hipStream_t st = (hipStream_t)stream;
   if (tiled) {
+    if (x1) { p.x1 = x1; p.scale1 = scale1; p.zp1 = zp1; p.words1 = words1; p.codes1 = codes1; }
     if (x_dtype == VARQ_F32) run_tiled<VARQ_F32>(p, pl, workspace, st);
     else if (x_dtype == VARQ_BF16) run_tiled<VARQ_BF16>(p, pl, workspace, st);
     else run_tiled<VARQ_F16>(p, pl, workspace, st);
-  } else if (x_dtype == VARQ_F32) run_general<VARQ_F32>(p, st);
-  else if (x_dtype == VARQ_BF16) run_general<VARQ_BF16>(p, st);
-  else run_general<VARQ_F16>(p, st);
+  } else {
+    for (int t = 0; t < (x1 ? 2 : 1); ++t) {   // stream order keeps the shared workspace safe
+      if (t == 1) { p.x = x1; p.scale = scale1; p.zp = zp1; p.words = words1; p.codes = codes1; }
+      if (x_dtype == VARQ_F32) run_general<VARQ_F32>(p, st);
+      else if (x_dtype == VARQ_BF16) run_general<VARQ_BF16>(p, st);
+      else run_general<VARQ_F16>(p, st);
+    }
+  }
   VARQ_CHECK_LAUNCH("quant_pack");
   return VARQ_OK;
+}
+}  // namespace
+
+extern "C" int varq_quant_pack(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
+                               int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
+                               const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
+  return quant_pack_impl(x, nullptr, x_dtype, host_shape4, reduce_mask, bits, asym, eps, words, codes, scale, zp,
+                         nullptr, nullptr, nullptr, nullptr, host_out_map, workspace, workspace_bytes, stream);
+}
+
+extern "C" int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, const int64_t *host_shape4, int reduce_mask,
+                                int bits, int asym, float eps, int32_t *words0, int8_t *codes0, float *scale0, float *zp0,
+                                int32_t *words1, int8_t *codes1, float *scale1, float *zp1,
+                                const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
+  VARQ_CHECK_ARG(x1, "quant_pack2: null second tensor");
+  return quant_pack_impl(x0, x1, x_dtype, host_shape4, reduce_mask, bits, asym, eps, words0, codes0, scale0, zp0,
+                         words1, codes1, scale1, zp1, host_out_map, workspace, workspace_bytes, stream);
 }

@@ -37,7 +37,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .kv_cache import PackedKVCache
-from .quant import VAR_Q, fused_attention
+from .quant import VAR_Q, fused_step
 
 
 def rope2d_tables(head_dim: int, scale_hw: Sequence[Tuple[int, int]], normalized_by_hw: int = 2,
@@ -168,10 +168,7 @@ class _QuantizedSelfAttention(nn.Module):
         if self.caching and self.fused == 'quantizer':
             if attn_bias is not None:
                 raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')
-            for quantizer, item in ((self.k_quant, k), (self.v_quant, v)):
-                quantizer.quant(item)
-                quantizer.cache()
-            o = fused_attention(q, self.k_quant, self.v_quant, scale)                     # in the layout of q
+            o = fused_step(q, k, v, self.k_quant, self.v_quant, scale)                    # in the layout of q
             if self.layout == 'BHLc':
                 o = o.transpose(1, 2)
             return o.reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)

@@ -194,6 +194,39 @@ def quant_pack(x: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: boo
     return q, scale, zp
 
 
+def quant_pack_pair(x0: torch.Tensor, x1: torch.Tensor, reduce_dims: Sequence[int], bits: int, asym: bool = False,
+                    eps: float = 1e-12, pack: bool = True):
+    """`quant_pack` of two tensors of one shape and dtype (K and V of a step) in the same
+    launches.  Returns ((q0, scale0, zp0), (q1, scale1, zp1)), each as from `quant_pack`."""
+    _gpu(x0, 'x0')
+    _gpu(x1, 'x1')
+    assert x0.dim() == 4 and x0.shape == x1.shape and x0.dtype == x1.dtype and x0.device == x1.device
+    x0, x1 = x0.contiguous(), x1.contiguous()
+    shape = list(x0.shape)
+    mask = 0
+    for d in reduce_dims:
+        mask |= 1 << (d % 4)
+    sshape = [1 if (mask >> d) & 1 else shape[d] for d in range(4)]
+    c = shape[3]
+    last = (c + 32 // bits - 1) // (32 // bits) if pack else c
+    outs = []
+    for _ in range(2):
+        outs.append((torch.empty((*shape[:3], last), dtype=torch.int32 if pack else torch.int8, device=x0.device),
+                     torch.empty(sshape, dtype=torch.float32, device=x0.device),
+                     torch.empty(sshape, dtype=torch.float32, device=x0.device) if asym else None))
+    lib = _lib.load()
+    sh = i64arr(shape)
+    ws_bytes = 2 * max(int(lib.varq_quant_workspace_bytes(sh, mask)), 8)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x0.device)
+    (q0, s0, z0), (q1, s1, z1) = outs
+    with _on_device(x0.device):
+        check(lib.varq_quant_pack2(x0.data_ptr(), x1.data_ptr(), _dt(x0), sh, mask, bits, int(asym), eps,
+                                   q0.data_ptr() if pack else None, None if pack else q0.data_ptr(), s0.data_ptr(), _ptr(z0),
+                                   q1.data_ptr() if pack else None, None if pack else q1.data_ptr(), s1.data_ptr(), _ptr(z1),
+                                   None, ws.data_ptr(), ws_bytes, _stream(x0)), 'varq_quant_pack2')
+    return outs[0], outs[1]
+
+
 # ---------------------------------------------------------------------------
 # pack / unpack of int8 codes
 # ---------------------------------------------------------------------------

@@ -32,8 +32,8 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from . import ops
-from ._lib import VarqError
+from . import _lib, ops
+from ._lib import VarqError, check, i64arr
 
 _REF_METHODS = ('G_TENSOR', 'G_SCALE_HEAD_DIM', 'G_HEAD_DIM', 'G_SCALE', 'G_TOKEN', 'G_TOKEN_HEAD')
 _EXT_METHODS = ('G_GROUP', 'G_HEAD')
@@ -64,7 +64,7 @@ class _Growable:
     def _flush(self):
         pending, self._pending = self._pending, []
         for t in pending:
-            self.append(t)
+            self.append(t() if callable(t) else t)     # (a callable builds the expanded view when asked)
 
     def append(self, t: torch.Tensor):
         n = t.size(self.dim)
@@ -133,6 +133,7 @@ class VAR_Q:
         self.zp: Optional[torch.Tensor] = None
         self._pack_meta: Optional[Dict[str, int]] = None
         self._staged = None
+        self._fast_plans: Dict[Tuple[int, int, int, int], tuple] = {}
         self._reset_cache()
 
     # The reference derives dim_cat/dim_map once in __init__ and callers later
@@ -237,6 +238,105 @@ class VAR_Q:
                 assert meta['pad_len'] == self._pack_meta['pad_len']
             self._pack_meta = meta
         self.quantized_item, self.scale, self.zp = q, s, z
+
+    def _fast_prepare(self, x: torch.Tensor):
+        """First half of the one-call step (see `_step_fast`): room in the cache buffer and the
+        table row for a step of the shipped rule, nothing launched, no state changed.  None
+        when the quantizer or the item is of another kind."""
+        bits = self.quant_bits
+        if self.quant_method != 'G_SCALE_HEAD_DIM' or not self.pack_to_int32 or bits not in (2, 4, 8):
+            return None
+        if not isinstance(x, torch.Tensor) or x.dim() != 4 or not x.is_cuda or not x.is_contiguous() \
+                or x.dtype not in ops._DT or self._c_item.dim != self.dim_cat:
+            return None
+        k = len(self._seg_ends)
+        s0, s1, s2, c = x.shape
+        vals = 32 // bits
+        if k >= MAX_TABLE_STEPS or c % vals or s0 * s1 * s2 == 0:
+            return None
+        bhl = self._qkv_format == 'BHLc'
+        H, n = (s1, s2) if bhl else (s2, s1)
+        buf = self._c_item.reserve([s0, s1, s2, c // vals], torch.int32, x.device)
+        if buf is None:
+            return None
+        meta = {'orig_c': int(c), 'vals_per_word': int(vals), 'pad_len': 0, 'bits': int(bits)}
+        if self._pack_meta is not None and self._pack_meta != meta:
+            return None                       # (quant() raises the reference's assertion for this)
+        self._table_rows(H, c, x.device)
+        plan = self._fast_plans.get((s0, s1, s2, c))
+        if plan is None:
+            sh = i64arr([s0, s1, s2, c])
+            mask = 0b0101 if bhl else 0b0011                      # reduce batch and tokens
+            ws_bytes = max(int(_lib.load().varq_quant_workspace_bytes(sh, mask)), 8)
+            plan = self._fast_plans[(s0, s1, s2, c)] = (sh, mask, ws_bytes)
+        start, cap, per_tok = self._c_item.len, buf.shape[self.dim_cat], (1 if bhl else H)
+        out_map = (n * per_tok, (cap - n) * per_tok, start * per_tok)
+        srow = self._tab_scale[k]
+        zrow = None if self.symmetric else self._tab_zp[k]
+        return (x, buf, srow, zrow, plan, out_map, meta, bhl, H, n, c, start)
+
+    def _fast_commit(self, prep):
+        """Second half: the state that quant() followed by cache() leaves, the kernels having
+        written the codes and the table row in place."""
+        x, buf, srow, zrow, plan, out_map, meta, bhl, H, n, c, start = prep
+        sshape = (1, H, 1, c) if bhl else (1, 1, H, c)
+        self.quantized_item = buf.narrow(self.dim_cat, start, n)
+        self.scale = srow.view(sshape)
+        self.zp = None if zrow is None else zrow.view(sshape)
+        self._pack_meta = meta
+        self._staged = None
+        self._c_item.len = start + n
+        eshape = (-1, -1, n, -1) if bhl else (-1, n, -1, -1)
+        scale, zp = self.scale, self.zp
+        self._c_scale.append_later(lambda: scale.expand(*eshape))
+        if zp is not None:
+            self._c_zp.append_later(lambda: zp.expand(*eshape))
+        self._seg_ends.append((self._seg_ends[-1] if self._seg_ends else 0) + n)
+
+    def _step_fast(self, x: torch.Tensor) -> bool:
+        """quant(x) followed by cache() for the shipped rule (G_SCALE_HEAD_DIM, packed codes)
+        with the host work of a generation step cut to one library call: same kernels, same
+        state afterwards.  False (nothing done) when the quantizer or the item is of another
+        kind; the caller then takes the two general calls."""
+        prep = self._fast_prepare(x)
+        if prep is None:
+            return False
+        _, buf, srow, zrow, (sh, mask, ws_bytes), out_map, *_ = prep
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        with ops._on_device(x.device):
+            check(_lib.load().varq_quant_pack(x.data_ptr(), ops._DT[x.dtype], sh, mask, self.quant_bits,
+                                              int(not self.symmetric), self.eps, buf.data_ptr(), None, srow.data_ptr(),
+                                              None if zrow is None else zrow.data_ptr(), i64arr(out_map),
+                                              ws.data_ptr(), ws_bytes, ops._stream(x)), 'varq_quant_pack')
+        self._fast_commit(prep)
+        return True
+
+    @staticmethod
+    def _step_fast_pair(kq: 'VAR_Q', vq: 'VAR_Q', k: torch.Tensor, v: torch.Tensor) -> bool:
+        """`_step_fast` for K and V of a step in the same three launches, when the two
+        quantizers are configured alike and their caches stand at the same place."""
+        if kq is vq or kq.quant_bits != vq.quant_bits or kq.symmetric != vq.symmetric or kq.eps != vq.eps \
+                or kq._qkv_format != vq._qkv_format or k.shape != v.shape or k.dtype != v.dtype or k.device != v.device:
+            return False
+        pk = kq._fast_prepare(k)
+        if pk is None:
+            return False
+        pv = vq._fast_prepare(v)
+        if pv is None or pk[5] != pv[5]:          # (same window of the two cache buffers)
+            return False
+        sh, mask, ws_bytes = pk[4]
+        ws = torch.empty(2 * ws_bytes, dtype=torch.uint8, device=k.device)
+        zk, zv = pk[3], pv[3]
+        with ops._on_device(k.device):
+            check(_lib.load().varq_quant_pack2(k.data_ptr(), v.data_ptr(), ops._DT[k.dtype], sh, mask, kq.quant_bits,
+                                               int(not kq.symmetric), kq.eps,
+                                               pk[1].data_ptr(), None, pk[2].data_ptr(), None if zk is None else zk.data_ptr(),
+                                               pv[1].data_ptr(), None, pv[2].data_ptr(), None if zv is None else zv.data_ptr(),
+                                               i64arr(pk[5]), ws.data_ptr(), 2 * ws_bytes, ops._stream(k)),
+                  'varq_quant_pack2')
+        kq._fast_commit(pk)
+        vq._fast_commit(pv)
+        return True
 
     # ---------------- cache ----------------
     def _expand_scale_like_L(self, q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
@@ -406,3 +506,18 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
         return ops.fused_attn(q, kbuf, ks, kz, vbuf, vs, vz, bits, bits, Lk, softmax_scale, kv_limit=kv_limit, out=out,
                               layout=layout)
     raise ValueError(f'fused_attention: methods {km} / {vm} cannot be combined')
+
+
+def fused_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_scale: float,
+               kv_limit: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One generation step on the packed caches: quantize and cache the step's K and V with
+    their quantizers (`quant` + `cache`, VAR_Q/quant.py:232-235 without the dequantization),
+    then `fused_attention` of q over everything cached.  For the shipped rule K and V are
+    quantized by one library call (three launches for both); any other rule goes through the
+    general methods."""
+    if not VAR_Q._step_fast_pair(k_quant, v_quant, k, v):
+        for quantizer, item in ((k_quant, k), (v_quant, v)):
+            if not quantizer._step_fast(item):
+                quantizer.quant(item)
+                quantizer.cache()
+    return fused_attention(q, k_quant, v_quant, softmax_scale, kv_limit=kv_limit, out=out)
