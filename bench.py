@@ -162,10 +162,13 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
         steps = [tuple(torch.randn(*shape(pn * pn), device=dev, generator=gd).bfloat16() for _ in range(3))
                  for pn in patch_nums]
         scale = 1.0 / math.sqrt(D)
+        total = sum(pn * pn for pn in patch_nums)
         heads_first = (lambda t: t) if fmt == 'BHLc' else (lambda t: t.transpose(1, 2))
 
         def one_pass(fused):
             kq, vq = VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM'), VAR_Q(8, fmt, 'G_SCALE_HEAD_DIM')
+            for quantizer in (kq, vq):            # (both paths: the cache buffers never have to grow)
+                quantizer.reserve_tokens(total)
             for q, k, v in steps:
                 if fused:
                     fused_step(q, k, v, kq, vq, scale)

@@ -208,3 +208,23 @@ def test_fused_step_leaves_the_state_of_quant_and_cache(dev, fmt, bits, sym):
                 assert x.cached_scale.shape == y.cached_scale.shape
                 assert (x.cached_zp is None) == (y.cached_zp is None) and (x.cached_zp is None or torch.equal(x.cached_zp, y.cached_zp))
                 assert torch.equal(x.dequant_all(), y.dequant_all())
+
+
+def test_reserve_tokens_keeps_the_buffers_in_place(dev):
+    """With the schedule's length reserved the cache buffers are allocated once; contents as
+    without the reservation."""
+    from var_q_amd.quant import fused_step
+    items = _steps('BHLc', torch.bfloat16, seed=91)
+    total = sum(x.shape[2] for x in items)
+    a, b = VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM'), VAR_Q(8, 'BHLc', 'G_SCALE_HEAD_DIM')
+    b.reserve_tokens(1000)
+    ptrs = set()
+    for x in items:
+        note('reserve_tokens', tuple(x.shape))
+        a.use_var_q(x.to(dev))
+        b.use_var_q(x.to(dev))
+        ptrs.add(b._c_item.buf.data_ptr())
+        assert b._c_item.buf.shape[2] >= 1000
+    assert len(ptrs) == 1 and a._c_item.buf.shape[2] < 1000
+    assert torch.equal(a.cached_item, b.cached_item) and torch.equal(a.cached_scale, b.cached_scale)
+    assert a.cached_item.shape[2] == total

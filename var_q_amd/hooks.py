@@ -124,6 +124,9 @@ class _QuantizedSelfAttention(nn.Module):
                 kw.update(group_size=self.group_size, symmetric=self.symmetric)
             self.k_quant = self._quantizer_factory(**kw)
             self.v_quant = self._quantizer_factory(**kw)
+            for quantizer in (self.k_quant, self.v_quant):
+                if self.max_tokens and hasattr(quantizer, 'reserve_tokens'):
+                    quantizer.reserve_tokens(self.max_tokens)     # no buffer growth during a schedule
 
     def _qkv(self, x):
         B, L, _ = x.shape

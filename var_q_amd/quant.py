@@ -50,8 +50,9 @@ def _dim_map(qkv_format: str) -> Dict[str, Tuple[int, ...]]:
 class _Growable:
     """Buffer that grows along one dim; `view()` is the valid prefix."""
 
-    def __init__(self, dim: int):
+    def __init__(self, dim: int, min_capacity: int = 64):
         self.dim, self.buf, self.len = dim, None, 0
+        self.min_capacity = min_capacity       # room of the first allocation (tokens)
         self._pending = []
 
     def append_later(self, t: torch.Tensor):
@@ -69,7 +70,7 @@ class _Growable:
     def append(self, t: torch.Tensor):
         n = t.size(self.dim)
         if self.buf is None or self.len + n > self.buf.size(self.dim):
-            cap = max(2 * (self.len + n), 64)
+            cap = max(2 * (self.len + n), self.min_capacity)
             shape = list(t.shape)
             shape[self.dim] = cap
             new = torch.empty(shape, dtype=t.dtype, device=t.device)
@@ -90,7 +91,7 @@ class _Growable:
                 return None
         if self.buf is None or self.len + n > self.buf.size(self.dim):
             shape = list(step_shape)
-            shape[self.dim] = max(2 * (self.len + n), 64)
+            shape[self.dim] = max(2 * (self.len + n), self.min_capacity)
             new = torch.empty(shape, dtype=dtype, device=device)
             if self.buf is not None and self.len:
                 new.narrow(self.dim, 0, self.len).copy_(self.buf.narrow(self.dim, 0, self.len))
@@ -160,11 +161,21 @@ class VAR_Q:
         self._seg_ends: List[int] = []
         self._tab_scale: Optional[torch.Tensor] = None      # [MAX_TABLE_STEPS, H, c]
         self._tab_zp: Optional[torch.Tensor] = None
-        self._tok_scale = _Growable(self.dim_cat)
-        self._tok_zp = _Growable(self.dim_cat)
-        self._c_item = _Growable(self.dim_cat)
-        self._c_scale = _Growable(self.dim_cat)
-        self._c_zp = _Growable(self.dim_cat)
+        room = max(64, getattr(self, '_reserved_tokens', 0))
+        self._tok_scale = _Growable(self.dim_cat, room)
+        self._tok_zp = _Growable(self.dim_cat, room)
+        self._c_item = _Growable(self.dim_cat, room)
+        self._c_scale = _Growable(self.dim_cat, room)
+        self._c_zp = _Growable(self.dim_cat, room)
+
+    def reserve_tokens(self, n_tokens: int):
+        """Size the cache buffers for n_tokens at their first allocation (an extension: the
+        reference grows its cache by torch.cat, VAR_Q/quant.py:200-201; here the buffers double
+        when they run out, and a caller that knows the schedule's length avoids those copies).
+        Takes effect for buffers not allocated yet."""
+        self._reserved_tokens = int(n_tokens)
+        for g in (self._tok_scale, self._tok_zp, self._c_item, self._c_scale, self._c_zp):
+            g.min_capacity = max(64, self._reserved_tokens)
 
     @property
     def cached_item(self) -> Optional[torch.Tensor]:
@@ -378,7 +389,8 @@ class VAR_Q:
         if not self.pack_to_int32:
             return
         if self._tok_scale.dim != self.dim_cat:   # layout was re-assigned before the first step
-            self._tok_scale, self._tok_zp = _Growable(self.dim_cat), _Growable(self.dim_cat)
+            room = self._c_item.min_capacity
+            self._tok_scale, self._tok_zp = _Growable(self.dim_cat, room), _Growable(self.dim_cat, room)
         bhl = self.qkv_format == 'BHLc'
         B, H, n = q_cur.shape[0], q_cur.shape[1 if bhl else 2], q_cur.shape[2 if bhl else 1]
         c = self._pack_meta['orig_c']
