@@ -959,8 +959,12 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   for (int tile = 0; tile < n_tiles; ++tile) {
     begin_tile(tile);
+    // a tile with at most 32 keys (the end of a segment or of the cache) has nothing for
+    // the second key block: every weight there would be exp2(-inf) = 0
+    const bool half_tile = (CHAN ? min(kv_end, tile_end) : kv_end) - t0 <= 32;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
+      if (kb == 1 && half_tile) continue;
       load_scales(kb);
       qk(kb);
       if constexpr (HOIST) {
