@@ -346,6 +346,10 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // Q^T operands, gathered in the slot order of the K codec
   u32x4_t qb[NCH];
   u32x4_t bq[NSK];
+  // per-channel tables at D=64: the query values as loaded stay in registers (16 of them), so
+  // that a segment boundary rebuilds the operands without going back to memory
+  constexpr bool KEEP_Q = CHAN && D == 64;
+  u32x4_t qraw[KEEP_Q ? NCH : 1];
   // The K zero-point term -(kzp+kOff)/kMul * sum(q) is a rank-1 update of S^T and
   // rides on one more MFMA per key block and group.  Both factors are split into
   // three bf16 pieces (a0+a1+a2, b0+b1+b2, exact) and the 9 products are laid on
@@ -366,7 +370,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int ch = 0; ch < NCH; ++ch) {
       const int oct = k_octet<GK>(ch, half);
       // the octet's eight channels in one 16-byte load, then into the codec's slot order
-      const u32x4_t raw = decltype(pre)::value ? qb[ch] : *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
+      u32x4_t raw;
+      if constexpr (KEEP_Q) raw = qraw[ch];
+      else raw = decltype(pre)::value ? qb[ch] : *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
       float sk[8];
       if constexpr (CHAN) {
         const float *tk = lds_tab + (seg * TR + 0) * D + oct * 8;
@@ -652,7 +658,10 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // the query values, behind the first tile's requests and ahead of the table loads: one
   // round trip for all three
 #pragma unroll
-  for (int ch = 0; ch < NCH; ++ch) qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
+  for (int ch = 0; ch < NCH; ++ch) {
+    if constexpr (KEEP_Q) qraw[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
+    else qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
+  }
   if constexpr (CHAN) {
     for (int i = tid; i < p.nseg * 4 * D; i += NT) {
       const int seg = i / (4 * D), which = (i / D) & 3, d = i % D;
@@ -718,16 +727,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     if constexpr (CHAN) {
       // (the Q operands first: with the accumulator arithmetic in front of it the register
       // allocator spills, and spills here cost scratch traffic at every boundary)
-      // The old Q operands are dead: at D=64 their registers receive the new query values at
-      // once, in flight under the accumulator arithmetic.  At D=128 that order makes the
-      // register allocator spill (and gains nothing): there the operands are rebuilt first.
-      constexpr bool OVERLAP_Q = (D == 64);
-      if constexpr (OVERLAP_Q) {
-#pragma unroll
-        for (int ch = 0; ch < NCH; ++ch) qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
-      } else {
-        load_q(seg_new, std::false_type{});
-      }
+      // the Q operands with the new K table: from the kept registers at D=64, reloaded at D=128
+      load_q(seg_new, std::false_type{});
       __builtin_amdgcn_sched_barrier(0);
       const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
       const float rq = __shfl(racc[0], col, 64) + r_run[0];
@@ -756,8 +757,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
           }
           __builtin_amdgcn_sched_barrier(0);   // one slice's registers at a time
         }
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (OVERLAP_Q) load_q(seg_new, std::true_type{});
       l_prev = l_sum;
       seg_a = seg_new;
     }
