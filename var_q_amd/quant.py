@@ -326,6 +326,8 @@ class VAR_Q:
     def _step_fast_pair(kq: 'VAR_Q', vq: 'VAR_Q', k: torch.Tensor, v: torch.Tensor) -> bool:
         """`_step_fast` for K and V of a step in the same three launches, when the two
         quantizers are configured alike and their caches stand at the same place."""
+        if not (isinstance(k, torch.Tensor) and isinstance(v, torch.Tensor)):
+            return False
         if kq is vq or kq.quant_bits != vq.quant_bits or kq.symmetric != vq.symmetric or kq.eps != vq.eps \
                 or kq._qkv_format != vq._qkv_format or k.shape != v.shape or k.dtype != v.dtype or k.device != v.device:
             return False
@@ -527,6 +529,8 @@ def fused_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_quant: VAR_Q
     then `fused_attention` of q over everything cached.  For the shipped rule K and V are
     quantized by one library call (three launches for both); any other rule goes through the
     general methods."""
+    if isinstance(k, torch.Tensor) and isinstance(v, torch.Tensor):
+        k, v = k.contiguous(), v.contiguous()      # (views of a qkv projection; the quantizers need dense rows)
     if not VAR_Q._step_fast_pair(k_quant, v_quant, k, v):
         for quantizer, item in ((k_quant, k), (v_quant, v)):
             if not quantizer._step_fast(item):
