@@ -79,6 +79,11 @@ struct AttnParams {
   // (fp32 [nseg, Hkv, D]); this is a cache that was quantized step by step
   int nseg;
   int seg_end[kMaxSegments];
+  // The first nconv segments (tiny first steps of a schedule, together at most one key tile)
+  // are attended in the units of segment nconv: their codes are turned into values relative
+  // to that segment's tables when the tile is widened (rounded to bf16, as the reference rounds
+  // the dequantized cache), so they share key tiles and cost no change of tables.
+  int nconv;
   const int32_t *head_map;
   const int32_t *kv_limit;
   int B, Hq, Hkv, Lq, Lk, Lstride;
@@ -171,6 +176,13 @@ __device__ __forceinline__ void split3_bf16(float x, u32 &h0, u32 &h1, u32 &h2) 
   const float x1 = u2f(f2u(r1) & 0xffff0000u);
   const float x2 = r1 - x1;
   h0 = f2u(x0) >> 16; h1 = f2u(x1) >> 16; h2 = f2u(x2) >> 16;
+}
+
+// Code held in `bits` bits at `shift` of a word that was staged with the codec's xor: 4- and
+// 2-bit fields hold code + 2^(bits-1) as unsigned numbers, bytes are signed as they are.
+template <int BITS> __device__ __forceinline__ float staged_code(u32 w, int shift) {
+  if constexpr (BITS == 8) return (float)((int)(w << (24 - shift)) >> 24);
+  else return (float)((int)((w >> shift) & ((1u << BITS) - 1u)) - (1 << (BITS - 1)));
 }
 
 // MFMA row r (0..31) of the S^T block carries key kperm(r) of the 32-key block
@@ -441,8 +453,10 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   {                                                                                            \
     const int e = p.seg_end[S];                                                                \
     if (tid == 0) lds_seg_end[S] = e;                                                          \
-    if (S < p.nseg && beg < kv_end) n_tiles += (min(e, kv_end) - beg + BN - 1) / BN;           \
-    beg = e;                                                                                   \
+    if (S + 1 >= p.nconv) { /* (a merged segment is counted with the last one of its run) */   \
+      if (S < p.nseg && beg < kv_end) n_tiles += (min(e, kv_end) - beg + BN - 1) / BN;         \
+      beg = e;                                                                                 \
+    }                                                                                          \
   }
     VARQ_SEG(0) VARQ_SEG(1) VARQ_SEG(2) VARQ_SEG(3) VARQ_SEG(4) VARQ_SEG(5) VARQ_SEG(6) VARQ_SEG(7)
     VARQ_SEG(8) VARQ_SEG(9) VARQ_SEG(10) VARQ_SEG(11) VARQ_SEG(12) VARQ_SEG(13) VARQ_SEG(14) VARQ_SEG(15)
@@ -463,10 +477,12 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       c.start += BN;
     }
   };
-  TileCursor cur_k{0, 0};
+  TileCursor cur_k{(CHAN && p.nconv > 0) ? p.nconv - 1 : 0, 0};   // (the merged run walks as one segment)
+  int tbase = 0;   // index of this workgroup's first tile in the block's tile sequence
   if (p.nsplit > 1) {
     // this workgroup's share of the tiles: [t_begin, t_end) of the block's tile sequence
     const int t_begin = n_tiles * split / p.nsplit, t_end = n_tiles * (split + 1) / p.nsplit;
+    tbase = t_begin;
     if constexpr (CHAN) {
       for (int i = 0; i < t_begin; ++i) cursor_advance(cur_k);
     } else {
@@ -476,6 +492,21 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   }
   TileCursor cur_v = cur_k, cur_a = cur_k;
   const int tile_base = cur_k.start;   // first key of this workgroup's tiles
+  // tiles of the merged run: the first npre of the sequence, dense from key 0
+  int npre = 0;
+  if constexpr (CHAN) {
+    if (p.nconv > 0) npre = (min(__builtin_amdgcn_readfirstlane(lds_seg_end[p.nconv - 1]), kv_end) + BN - 1) / BN;
+  }
+  // (at D=128 the conversion code costs registers that the main loop has not got: the host
+  // merges nothing there, and the code is left out)
+  constexpr bool MERGE = CHAN && D == 64;
+  auto merged_tile = [&](int tile) { return MERGE && tbase + tile < npre; };
+  // segment (< nconv) of a key of the merged run
+  auto merged_segment = [&](int key) {
+    int sgm = 0;
+    while (sgm + 1 < p.nconv && key >= lds_seg_end[sgm]) ++sgm;
+    return sgm;
+  };
   int wave_minlim = q_live ? limit : p.Lk;
   for (int off = 1; off < 64; off <<= 1) wave_minlim = min(wave_minlim, __shfl_xor(wave_minlim, off, 64));
 
@@ -570,10 +601,12 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       const float c = ks * p.scale_log2e * KCodec<BITS>::kMul;
       return __builtin_fabsf(c) < 1e-30f ? 1e-30f : c;
     };
+    // keys of the merged run carry values, not code images: no image factor, no offset terms
+    const bool merged = merged_tile(tile);
     if (seg < NSK) {
-      par[P_CK + seg * BN + key] = ck_of(ksc);
+      par[P_CK + seg * BN + key] = merged ? p.scale_log2e : ck_of(ksc);
       u32 a0, a1, a2;
-      split3_bf16(-(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
+      split3_bf16(merged ? 0.f : -(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
       u32x4_t *dst = &lds_kz[((sl * NSK + seg) * BN + key) * 2];
       dst[0] = u32x4_t{a0 | (a0 << 16), a0 | (a1 << 16), a1 | (a1 << 16), a2 | (a2 << 16)};
       if (!(FOLD_SV && seg == 0)) dst[1] = u32x4_t{0u, 0u, 0u, 0u};
@@ -592,7 +625,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       if (!FOLD_SV) par[P_SV + seg * BN + key] = vsc;
       par[P_VR + seg * BN + key] = zr;
       uint16_t *rows = lds_wz + sl * 8 * RSR;
-      rows[seg * RSR + key] = (uint16_t)(f2u(zc + VCodec<BITS>::kOff) >> 16);
+      rows[seg * RSR + key] = merged ? (uint16_t)0 : (uint16_t)(f2u(zc + VCodec<BITS>::kOff) >> 16);
       if (seg == 0) {
         u32 i0, i1, i2;
         split3_bf16(__builtin_amdgcn_rcpf(vsc), i0, i1, i2);
@@ -614,14 +647,34 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   // packed V of `tile` -> V^T bf16: a work item is 2 adjacent keys x 8 channels (one
   // packed word of each key), written as 8 dwords of the transposed tile
-  auto widen_v = [&](int tile) {
+  // (first: the call may meet the tile of the merged run, which is always the first of the
+  // sequence -- only the prologue's calls carry the conversion code, the loop's stay lean)
+  auto widen_v = [&](int tile, auto first) {
     const u32 *vp = lds_vp + (tile % 3) * BN * RSV;
     uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
+    const bool merged = decltype(first)::value && merged_tile(tile);
     for (int item = tid; item < (BN / 2) * (D / 8); item += NT) {
       const int kp2 = item & (BN / 2 - 1), oct = item / (BN / 2);
       const u32 *row = &vp[kp2 * 2 * RSV];
       u32 pr[8];
-      VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
+      if (merged) {
+        if constexpr (MERGE && decltype(first)::value) {
+          // values of the two keys in the V units of the base segment: (code - zv) * sv / sv_base,
+          // divided by the image factor that the epilogue multiplies back
+          const int k0 = min((tbase + tile) * BN + 2 * kp2, p.Lk - 1), k1 = min(k0 + 1, p.Lk - 1);
+          const float *tb = lds_tab + (p.nconv * TR + 2) * D + oct * 8;
+          const float *t0s = lds_tab + (merged_segment(k0) * TR + 2) * D + oct * 8, *t1s = lds_tab + (merged_segment(k1) * TR + 2) * D + oct * 8;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int off = (oct * 8 + j) * BITS;
+            const float rb = __builtin_amdgcn_rcpf(tb[j]) * (1.f / VCodec<BITS>::kMul);
+            const float c0 = staged_code<BITS>(row[off >> 5], off & 31), c1 = staged_code<BITS>(row[RSV + (off >> 5)], off & 31);
+            pr[j] = pack_bf16_rne((c0 - t0s[D + j]) * t0s[j] * rb, (c1 - t1s[D + j]) * t1s[j] * rb);
+          }
+        }
+      } else {
+        VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * VTS + kp2 * 2]) = pr[j];
     }
@@ -629,7 +682,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   // packed K of `tile` (in kreg) -> widened bf16 rows: each 16-byte piece holds OPQ octets
   // of one key, every octet becomes one 16-byte MFMA A operand
-  auto widen_k = [&](int tile) {
+  auto widen_k = [&](int tile, auto first) {
     uint16_t *kx = lds_kx + (tile & 1) * BN * KXS;
     constexpr int OPQ = 16 / BITS;            // octets per 16-byte piece
 #pragma unroll
@@ -639,6 +692,29 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         const int key = piece / (WPR / 4), oct0 = (piece % (WPR / 4)) * OPQ;
         constexpr u32 KX = KCodec<BITS>::kStageXor;
         const u32 q4[4] = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
+        if (decltype(first)::value && merged_tile(tile)) {
+          if constexpr (MERGE && decltype(first)::value) {
+            // the key's values in the K units of the base segment, (code - zk) * sk / sk_base, in
+            // the operand's slot order
+            const int kabs = min((tbase + tile) * BN + key, p.Lk - 1);
+            const float *ts = lds_tab + (merged_segment(kabs) * TR + 0) * D, *tb = lds_tab + (p.nconv * TR + 0) * D;
+#pragma unroll
+            for (int j = 0; j < OPQ; ++j) {
+              float val[8];
+#pragma unroll
+              for (int c = 0; c < 8; ++c) {
+                const int off = (j * 8 + c) * BITS, d = (oct0 + j) * 8 + c;
+                val[c] = (staged_code<BITS>(q4[off >> 5], off & 31) - ts[D + d]) * ts[d] * __builtin_amdgcn_rcpf(tb[d]);
+              }
+              u32 a[4];
+#pragma unroll
+              for (int j2 = 0; j2 < 4; ++j2)
+                a[j2] = pack_bf16_rne(val[KCodec<BITS>::slot_d(2 * j2)], val[KCodec<BITS>::slot_d(2 * j2 + 1)]);
+              *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
+            }
+          }
+          continue;
+        }
 #pragma unroll
         for (int j = 0; j < OPQ; ++j) {
           u32 a[4];
@@ -678,11 +754,11 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     }
     __syncthreads();
   }
-  load_q(cur_a.seg, std::true_type{});
-  if (n_tiles > 0) { stage(0); widen_k(0); }
+  load_q(max(cur_a.seg, p.nconv), std::true_type{});   // (the merged run is attended with the base segment's tables)
+  if (n_tiles > 0) { stage(0); widen_k(0, std::true_type{}); }
   if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
-  if (n_tiles > 0) widen_v(0);
+  if (n_tiles > 0) widen_v(0, std::true_type{});
   if (n_tiles > 2) prefetch(2);
   __syncthreads();
 
@@ -692,7 +768,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int tile = 0; tile < n_tiles; ++tile) {
       if (tile + 2 < n_tiles) stage(tile + 2);
       if (tile + 3 < n_tiles) prefetch(tile + 3);
-      if (tile + 1 < n_tiles) { widen_v(tile + 1); widen_k(tile + 1); }
+      if (tile + 1 < n_tiles) { widen_v(tile + 1, std::false_type{}); widen_k(tile + 1, std::false_type{}); }
       if (tile + 2 < n_tiles) prefetch_k(tile + 2);
       __syncthreads();
     }
@@ -716,7 +792,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   // per-channel tables: segment of the tile being attended, end of the tile's keys, and the
   // softmax denominator as it was when the current segment began
-  int seg_a = cur_a.seg, tile_end = 0;
+  int seg_a = max(cur_a.seg, p.nconv), tile_end = 0;
+  bool in_merged = false;   // the tile being attended belongs to the merged run
   float l_prev = 0.f;
   // A new segment begins.  The true (unnormalized) output is, per channel,
   //   sv * (kMul * oacc - rq - zv * (l_sum - l_prev))
@@ -766,7 +843,16 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     if constexpr (CHAN) {
       t0 = cur_a.start;
       tile_end = min(t0 + BN, __builtin_amdgcn_readfirstlane(lds_seg_end[cur_a.seg]));
-      if (__builtin_expect(cur_a.seg != seg_a, 0)) segment_boundary(cur_a.seg);
+      const int seg_t = max(cur_a.seg, p.nconv);
+      const bool was_merged = in_merged;
+      in_merged = merged_tile(tile);
+      if (__builtin_expect(seg_t != seg_a, 0)) {
+        segment_boundary(seg_t);
+      } else if (was_merged && !in_merged) {
+        // from the merged run into its base segment: same tables, but the zero-point term of
+        // the output belongs to the weights from here on only
+        l_prev = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
+      }
       cursor_advance(cur_a);
     } else {
       t0 = tile_base + tile * BN;
@@ -784,8 +870,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // with the PV MFMAs of a block in flight: widen the next tile's K and V into the other slots
   auto widen_next = [&](int tile) {
     if (tile + 1 < n_tiles) {
-      widen_v(tile + 1);
-      widen_k(tile + 1);
+      widen_v(tile + 1, std::false_type{});
+      widen_k(tile + 1, std::false_type{});
       if (tile + 2 < n_tiles) prefetch_k(tile + 2);
     }
   };
@@ -844,7 +930,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     float z[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      float v = CHAN ? qbias - m_ref : -m_ref;
+      float v = CHAN ? (in_merged ? 0.f : qbias) - m_ref : -m_ref;
 #pragma unroll
       for (int s = 0; s < NSK; ++s) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
@@ -1010,7 +1096,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
           const int c0 = d * 32 + 8 * g4 + 4 * half;
           const float4 sv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 2) * D + c0);
           const float4 zv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 3) * D + c0);
-          const float share = (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
+          // (a share that ended inside the merged run has no weight in the current segment)
+          const float share = in_merged ? 0.f : (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
           o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
           o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
         }
@@ -1223,6 +1310,7 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.k_scale = k_scale; p.k_zp = k_zp; p.v_scale = v_scale; p.v_zp = v_zp;
   p.k_chan_scale = nullptr; p.k_chan_zp = nullptr; p.v_chan_scale = nullptr; p.v_chan_zp = nullptr;
   p.nseg = 1;
+  p.nconv = 0;
   for (int s = 0; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
   p.head_map = head_map; p.kv_limit = kv_limit;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
@@ -1292,6 +1380,10 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
     prev = e;
   }
   for (int s = nseg; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
+  // leading segments that together fit one key tile are merged into the segment behind them
+  p.nconv = 0;
+  // (one tile: the kernel converts codes to values in its prologue only)
+  while (D == 64 && p.nconv + 1 < nseg && p.seg_end[p.nconv] <= BN) ++p.nconv;
   p.head_map = head_map; p.kv_limit = kv_limit;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
   p.q_tiles = (Lq + BM - 1) / BM;
