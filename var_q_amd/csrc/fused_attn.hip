@@ -288,8 +288,12 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
 // When the tables change along the keys (segments), key tiles never straddle a segment:
 // at a boundary the Q operands are rebuilt with the new K table and the output
 // accumulators are re-expressed in units of the new V table.
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8>
+// SEGS: the tables change along the keys (more than one segment).  A single table needs none
+// of what makes boundaries cheap (kept query registers, merged first steps), and is compiled
+// without it.
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8, bool SEGS = false>
 __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
+  static_assert(CHAN || !SEGS, "segments belong to the per-channel tables");
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
@@ -360,7 +364,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   u32x4_t bq[NSK];
   // per-channel tables at D=64: the query values as loaded stay in registers (16 of them), so
   // that a segment boundary rebuilds the operands without going back to memory
-  constexpr bool KEEP_Q = CHAN && D == 64;
+  constexpr bool KEEP_Q = SEGS && D == 64;
   u32x4_t qraw[KEEP_Q ? NCH : 1];
   // The K zero-point term -(kzp+kOff)/kMul * sum(q) is a rank-1 update of S^T and
   // rides on one more MFMA per key block and group.  Both factors are split into
@@ -499,7 +503,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   }
   // (at D=128 the conversion code costs registers that the main loop has not got: the host
   // merges nothing there, and the code is left out)
-  constexpr bool MERGE = CHAN && D == 64;
+  constexpr bool MERGE = SEGS && D == 64;
   auto merged_tile = [&](int tile) { return MERGE && tbase + tile < npre; };
   // segment (< nconv) of a key of the merged run
   auto merged_segment = [&](int key) {
@@ -1146,7 +1150,7 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
 
 int device_cus();
 
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV>
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, bool SEGS>
 void launch_shape(const AttnParams &p, hipStream_t st) {
   constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * kChanTableRows * D * 4 : 0);
   static_assert(lds_bytes <= 160 * 1024, "LDS budget");
@@ -1155,31 +1159,42 @@ void launch_shape(const AttnParams &p, hipStream_t st) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !configured[dev]) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, SEGS>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (dev >= 0) configured[dev] = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV>), grid, dim3(NWV * 64), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, SEGS>), grid, dim3(NWV * 64), lds_bytes, st, p);
   if (p.nsplit > 1) {
     const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
     hipLaunchKernelGGL((combine_splits_kernel<D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
   }
 }
 
-template <int D, int BITS, int GK, int GV, bool CHAN = false>
-void launch(const AttnParams &p, hipStream_t st) {
+template <int D, int BITS, int GK, int GV, bool CHAN, bool SEGS>
+void launch_nw(const AttnParams &p, hipStream_t st) {
   if constexpr (D == 64) {
     // more (batch, head) pairs than compute units, at most four wavefronts of queries each:
     // small workgroups, two to a compute unit (same arithmetic, same results)
     if (p.Lq <= 128 && p.bh_total > device_cus()) {
-      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2>(p, st);
-      else launch_shape<D, BITS, GK, GV, CHAN, 4>(p, st);
+      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2, SEGS>(p, st);
+      else launch_shape<D, BITS, GK, GV, CHAN, 4, SEGS>(p, st);
       return;
     }
   }
-  launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
+  launch_shape<D, BITS, GK, GV, CHAN, 8, SEGS>(p, st);
+}
+
+template <int D, int BITS, int GK, int GV, bool CHAN = false>
+void launch(const AttnParams &p, hipStream_t st) {
+  if constexpr (CHAN && D == 64) {   // (at D=128 the two kinds are the same code)
+    if (p.nseg > 1) {
+      launch_nw<D, BITS, GK, GV, true, true>(p, st);
+      return;
+    }
+  }
+  launch_nw<D, BITS, GK, GV, CHAN, false>(p, st);
 }
 
 template <int D, int BITS>
