@@ -444,6 +444,11 @@ bool make_plan(const int64_t *sh, int reduce_mask, int64_t n_groups, Plan &pl) {
   int64_t Z = (4096 + kept_blocks - 1) / kept_blocks;
   const int64_t zcap = (8ll << 20) / (n_groups > 0 ? n_groups : 1);   // partials stay below 64 MiB
   if (Z > zcap) Z = zcap;
+  // ... and below a sixteenth of the input: with few kept blocks (groups indexed by the
+  // innermost leading dim only, the BLHc layouts) thousands of chunks would write and re-read
+  // as many partials as half the tensor
+  const int64_t zvol = rows * c / (16 * (n_groups > 0 ? n_groups : 1));
+  if (Z > zvol) Z = zvol;
   if (Z > steps) Z = steps;
   if (Z < 1) Z = 1;
   const int64_t spc = (steps + Z - 1) / Z;
