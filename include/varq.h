@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 5
+#define VARQ_ABI_VERSION 6
 
 enum varq_status {
   VARQ_OK = 0,
@@ -121,6 +121,24 @@ int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, const int64_t 
                      int bits, int asym, float eps, int32_t *words0, int8_t *codes0, float *scale0, float *zp0,
                      int32_t *words1, int8_t *codes1, float *scale1, float *zp1,
                      const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * varq_quant_pack for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
+ * in the reference.  Same arguments and results as varq_quant_pack, without a workspace:
+ * the partial min/max and the group parameters go through a static device array of
+ * VARQ_STATIC_SCRATCH_BYTES that each GPU the library runs on holds until the process
+ * ends.  Calls no hipMalloc/hipFree and no allocating routine.  A shape and grouping
+ * whose varq_quant_workspace_bytes exceeds the array is rejected with VARQ_ERR_WORKSPACE
+ * (the six methods of VAR_Q/quant.py:75-95 need at most 8 MiB at the benchmark shapes).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams,
+ * two threads) race; calls ordered on one stream do not.
+ */
+#define VARQ_STATIC_SCRATCH_BYTES (16u << 20)
+size_t varq_quant_static_scratch_bytes(void);
+int varq_quant_pack_static(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
+                           int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
+                           const int64_t *host_out_map, void *stream);
 
 /* VAR_Q/pack_unpack.py:107-134 (and its CPU twin 177-196): int8 codes [rows,c]
  * -> int32 words [rows, ceil(c*bits/32)], zero padding in the last word. */

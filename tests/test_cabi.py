@@ -25,7 +25,7 @@ def test_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
     assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
-    assert lib.varq_abi_version() == _lib.ABI_VERSION == 5
+    assert lib.varq_abi_version() == _lib.ABI_VERSION == 6
 
 
 def test_invalid_arguments_are_rejected_on_the_host():
@@ -57,6 +57,10 @@ def test_invalid_arguments_are_rejected_on_the_host():
     ws = lib.varq_quant_workspace_bytes(i64([2, 5, 3, 8]), 0b0011)
     assert ws >= 3 * 8 * 2 * 4 and ws % (3 * 8 * 4) == 0
     assert lib.varq_quant_workspace_bytes(i64([2, 5, 3, 7]), 0b0011) == 3 * 7 * 2 * 4
+    # the entry point without a workspace turns down what its static scratch cannot hold, on the host
+    assert lib.varq_quant_static_scratch_bytes() == 16 << 20
+    rc = lib.varq_quant_pack_static(fake, 0, i64([8, 4096, 16, 128]), 0b0001, 8, 0, 1e-12, fake, None, fake, None, None, None)
+    assert rc == -4 and b'static' in lib.varq_last_error()
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128,
                              1, 2, 2, None, 16, 16, 16, 96, None, 1.0, 0, None, 0, 0, None)
     assert rc == -1 and b'D must be' in lib.varq_last_error()

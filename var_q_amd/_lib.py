@@ -7,7 +7,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, 'libvarq_hip.so')
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 SYMBOLS = {
     'varq_abi_version': (c_int, []),
@@ -23,6 +23,9 @@ SYMBOLS = {
     'varq_quant_pack2': (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_int, c_float,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  POINTER(c_int64), c_void_p, c_size_t, c_void_p]),
+    'varq_quant_static_scratch_bytes': (c_size_t, []),
+    'varq_quant_pack_static': (c_int, [c_void_p, c_int, POINTER(c_int64), c_int, c_int, c_int, c_float,
+                                       c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_int64), c_void_p]),
     'varq_pack': (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     'varq_unpack': (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     'varq_dequant': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64),

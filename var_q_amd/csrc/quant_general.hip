@@ -11,6 +11,7 @@
 // in which partial results meet.  Channel counts that are not a multiple of 8 and
 // rows wider than 512 channels take scalar kernels with ordered-integer atomics.
 #include "varq_common.h"
+#include <mutex>
 
 namespace {
 
@@ -640,4 +641,58 @@ extern "C" int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, con
   VARQ_CHECK_ARG(x1, "quant_pack2: null second tensor");
   return quant_pack_impl(x0, x1, x_dtype, host_shape4, reduce_mask, bits, asym, eps, words0, codes0, scale0, zp0,
                          words1, codes1, scale1, zp1, host_out_map, workspace, workspace_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------
+// Its workspace is this array, which every device the library runs on holds from the load
+// of the code object to the end of the process.  Host code never uses the array's name as
+// an address: scratch_for_current_device() asks the runtime once per device where that
+// device's copy lives and hands out that pointer.
+static __device__ __align__(256) unsigned char scratch[VARQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_for_current_device(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return varq_set_error(VARQ_ERR_LAUNCH, "quant_pack_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return varq_set_error(VARQ_ERR_UNSUPPORTED, "quant_pack_static: device index %d beyond %d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return varq_set_error(VARQ_ERR_LAUNCH, "quant_pack_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return VARQ_OK;
+}
+}  // namespace
+
+extern "C" size_t varq_quant_static_scratch_bytes(void) { return (size_t)VARQ_STATIC_SCRATCH_BYTES; }
+
+extern "C" int varq_quant_pack_static(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
+                                      int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,
+                                      const int64_t *host_out_map, void *stream) {
+  VARQ_CHECK_ARG(host_shape4, "quant_pack_static: null shape");
+  VARQ_CHECK_ARG(reduce_mask >= 0 && reduce_mask < 16, "quant_pack_static: bad reduce mask");
+  const size_t need = varq_quant_workspace_bytes(host_shape4, reduce_mask);
+  if (need > (size_t)VARQ_STATIC_SCRATCH_BYTES)
+    return varq_set_error(VARQ_ERR_WORKSPACE,
+                          "quant_pack_static: this shape and grouping need %zu bytes of partial results, the static "
+                          "scratch holds %zu; use varq_quant_pack with a workspace of the caller's",
+                          need, (size_t)VARQ_STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  const int rc = scratch_for_current_device(&ws);
+  if (rc != VARQ_OK) return rc;
+  // every partial and parameter the kernels read is written earlier in the same call (plain
+  // stores, or the fill kernel of the scalar path), so what an earlier call left behind is
+  // never seen and nothing needs clearing here
+  return quant_pack_impl(x, nullptr, x_dtype, host_shape4, reduce_mask, bits, asym, eps, words, codes, scale, zp,
+                         nullptr, nullptr, nullptr, nullptr, host_out_map, ws, (size_t)VARQ_STATIC_SCRATCH_BYTES, stream);
 }
