@@ -3,8 +3,15 @@ reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar
 (G_TENSOR), and the affine per-head-per-dim variant of benchmark configuration 3 --
 against the oracle path quantize -> dequant -> bf16 SDPA and an fp64 evaluation of the same
 formula.  Tolerances as in test_gpu_attention.py (max-abs 2e-2 in range units, cosine >=
-0.9995); the codes handed to the kernel are the oracle's own, so the comparison isolates
-the attention."""
+0.9995), with a tighter bar on the distance from the fp64 value: 1.25e-2 of the range, on
+the data of the benchmark configurations (outlier channels x15) throughout.  The kernel
+scales the queries by the K table and rounds them to bf16 once per segment; chunks of
+channels with an outlier scale carry the rounding remainder through a second MFMA, which
+is what keeps that distance at 0.2-0.5 % (bf16 output rounding alone is up to 0.4 %); the
+first steps of a D=64 schedule that share one key tile are converted to the units of the
+step behind them and rounded to bf16 as the oracle rounds the whole cache, and stay at
+the oracle's own distance (up to 1.2 %).  The codes handed to the kernel are the oracle's
+own, so the comparison isolates the attention."""
 import math
 
 import pytest
@@ -16,6 +23,8 @@ from test_gpu_attention import _compare, _exact_fp64
 from var_q_amd import ops, schedules
 
 pytestmark = pytest.mark.gpu
+
+FP64_BAR = 1.25e-2   # kernel vs fp64, in units of the output range (the general bar is 2e-2)
 
 
 def _quantize_channel(x, bits, asym, dims=(0, 2)):
@@ -43,7 +52,7 @@ def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist=
                                  kv_limit=None if kv_limit is None else kv_limit.to(dev), splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, kd, vd, scale, bias)
-    _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what)
+    _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what, fp64_bar=FP64_BAR)
 
 
 @pytest.mark.parametrize('D', [64, 128])
@@ -152,7 +161,7 @@ def _stepwise(dev, B, H, D, steps, bits, asym, Lq, seed, masked=False, what='', 
                                  kv_limit=None if lim is None else lim.to(dev), seg_ends=ends, splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, deq[0], deq[1], scale, bias)
-    _compare(out, ref, _exact_fp64(q, deq[0], deq[1], scale, bias, dev), what)
+    _compare(out, ref, _exact_fp64(q, deq[0], deq[1], scale, bias, dev), what, fp64_bar=FP64_BAR)
 
 
 VAR_STEPS = [n * n for n in O.VAR_PATCH_NUMS]
@@ -166,12 +175,9 @@ def test_stepwise_cache_reference_default_rule(dev):
 
 @pytest.mark.parametrize('bits,asym', [(4, False), (2, True), (8, True)])
 def test_stepwise_cache_other_widths(dev, bits, asym):
-    """Eight steps of the Infinity schedule at D=128.  The 2-bit case runs on data without
-    the x15 outlier channels: with four levels over an outlier channel both the kernel and
-    the oracle sit at the edge of the 2e-2 bar there (measured 0.64 and 0.34 from the fp64
-    value at range 29; with one table, test_small_all_visible keeps the outlier data)."""
-    _stepwise(dev, 1, 2, 128, [1, 4, 16, 36, 64, 144, 256, 400], bits, asym, 400, seed=50 + bits, what='stepwise D128',
-              outlier_mul=1.0 if bits == 2 else 15.0)
+    """Eight steps of the Infinity schedule at D=128, on the data of the benchmark
+    configurations (outlier channels x15), 2-bit codes included."""
+    _stepwise(dev, 1, 2, 128, [1, 4, 16, 36, 64, 144, 256, 400], bits, asym, 400, seed=50 + bits, what='stepwise D128')
 
 
 def test_stepwise_cache_masked_queries(dev):

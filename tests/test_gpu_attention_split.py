@@ -44,13 +44,10 @@ def test_block_causal_mask(dev, splits):
 @pytest.mark.parametrize('bits,asym', [(8, False), (4, True)])
 def test_stepwise_tables(dev, splits, bits, asym):
     """A share may begin in the middle of the cache: it starts with the tables of its first
-    segment and crosses the later boundaries like the one-workgroup path.  (Data without the
-    x15 outlier channels: with them the rounding of the table-scaled queries to bf16 puts the
-    one-workgroup result itself near the bar, whatever the seed; the subject here is the sharing.)"""
-    _stepwise(dev, 2, 3, 64, VAR_STEPS, bits, asym, 256, seed=141 + splits, what='split stepwise', splits=splits,
-              outlier_mul=1.0)
+    segment and crosses the later boundaries like the one-workgroup path."""
+    _stepwise(dev, 2, 3, 64, VAR_STEPS, bits, asym, 256, seed=141 + splits, what='split stepwise', splits=splits)
     _stepwise(dev, 1, 2, 128, [1, 4, 16, 36, 64, 144, 256, 400], bits, asym, 400, seed=150 + splits,
-              what='split stepwise D128', splits=splits, outlier_mul=1.0)
+              what='split stepwise D128', splits=splits)
 
 
 def test_stepwise_masked(dev):
@@ -134,10 +131,10 @@ def test_many_heads_few_queries_stepwise_tables(dev, fmt_blhc):
     rule at a large batch), in both layouts."""
     B, H, D, bits = 40, 8, 64, 8
     steps = [1, 4, 9, 16, 25, 36]
-    _stepwise(dev, B, H, D, steps, bits, False, 36, seed=801, what='small workgroups stepwise', outlier_mul=1.0)
-    _stepwise(dev, B, H, D, steps, 4, True, 20, seed=802, what='small workgroups stepwise asym', outlier_mul=1.0, splits=1)
+    _stepwise(dev, B, H, D, steps, bits, False, 36, seed=801, what='small workgroups stepwise')
+    _stepwise(dev, B, H, D, steps, 4, True, 20, seed=802, what='small workgroups stepwise asym', splits=1)
     _stepwise(dev, B, H, D, steps + [49], 8, False, 100, seed=803, what='small workgroups stepwise, four wavefronts',
-              outlier_mul=1.0, splits=1)
+              splits=1)
     L, nseg = sum(steps), len(steps)
     ends = [sum(steps[:i + 1]) for i in range(nseg)]
     gen = torch.Generator(device=dev).manual_seed(9)

@@ -66,6 +66,8 @@ constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row ma
 
 constexpr int kMaxSegments = 16;
 constexpr int kChanTableRows = 5;   // LDS rows per segment of the per-channel tables
+constexpr int kMaxLoAny = 4;        // most remainder passes per key block (per-channel tables)
+constexpr float kLoRatio = 3.f;      // a chunk gets one when its largest K scale is this many times the head's mean
 
 struct AttnParams {
   const __bf16 *q;
@@ -260,7 +262,8 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 }
 
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
-template <int D, int BITS, int GK, int GV> struct AttnLds {
+// (CHAN: per-channel tables have no per-key K parameters, hence no rank-1 operands)
+template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
   static constexpr bool kFoldSv = (D / GV == 1);   // one V group: its scale rides inside the logits
@@ -271,7 +274,7 @@ template <int D, int BITS, int GK, int GV> struct AttnLds {
   static constexpr int kVp = kKx + 2 * 64 * KXS * 2;
   static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
   static constexpr int kKz = kVt + 2 * D * (64 + 8) * 2;          // rank-1 operands of S^T, 2 x 16 bytes per key and group
-  static constexpr int kWz = kKz + 3 * (D / GK) * 64 * 32;        // 8 rows per slot for the extra PV MFMA
+  static constexpr int kWz = kKz + (CHAN ? 0 : 3 * (D / GK) * 64 * 32);   // 8 rows per slot for the extra PV MFMA
   static constexpr int kPar = kWz + 3 * 8 * RSR * 2;
   static constexpr int kFlag = kPar + 3 * kParFloats * 4;
   static constexpr int kBytes = kFlag + 16;
@@ -302,7 +305,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
   constexpr int NDB = D / 32;               // 32-row blocks of O^T
   constexpr int VTS = BN + 8;               // V^T row stride (bf16 elements)
-  using L = AttnLds<D, BITS, GK, GV>;
+  using L = AttnLds<D, BITS, GK, GV, CHAN>;
 
   // Pipelined LDS buffers (one workgroup barrier per tile):
   //   packed V and the per-key parameters of tile t live in slot t % 3, the
@@ -325,6 +328,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // V scale, V zero-point (zeros where a table is absent) and the ratio of the V scales of the
   // previous segment and this one; filled once in the prologue
   float *const lds_tab = reinterpret_cast<float *>(lds_raw + (L::kBytes + 15) / 16 * 16);
+  // per segment two words: remainder slot + 1 of 16-channel contraction chunk ch in bits 4ch..4ch+2
+  // (0 = none); chunk of slot s in bits 4s..4s+2 and the number of slots in use from bit 16
+  u32 *const lds_clo = reinterpret_cast<u32 *>(lds_tab + kMaxSegments * kChanTableRows * D);
   constexpr int TR = kChanTableRows;   // rows per segment: K scale, K zero-point, V scale, V zero-point, sv(seg-1)/sv(seg)
   const bool k_affine = CHAN && p.k_chan_zp != nullptr, v_affine = CHAN && p.v_chan_zp != nullptr;   // (uniform)
   constexpr int KXS = L::KXS, RSV = L::RSV;
@@ -374,7 +380,23 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // the term, is dropped).  With a single V group, slots 0..2 of the upper half add
   // log2(vs)/ck (three pieces against 1.0), which makes exp2(logit) come out as
   // p * vs without a multiplication; the other upper slots are zero.
-  float qbias = 0.f;   // CHAN: -softmax_scale*log2(e) * sum_d q'[d] zk[d] of the current segment
+  // CHAN: per-query constant of the current segment's logits,
+  // -softmax_scale*log2(e) * (sum_d q'[d] zk[d] + kOff * sum_d q'[d]): the K zero-points and the
+  // offset of the code images (the token-mode kernels carry both on the rank-1 MFMA, whose key
+  // side is the same for every key here)
+  float qbias = 0.f;
+  // CHAN: q[d] * sk[d] is rounded to bf16 for the MFMA, the same rounding for every key of the
+  // segment, so its error does not average out over the keys the way the reference's rounding
+  // of the dequantized K does: on a channel whose scale is far above the others (an outlier
+  // channel) it tilts the softmax.  The 16-channel chunks whose largest scale is at least
+  // kLoRatio times the head's mean scale -- up to kMaxLo of them, the largest first -- get a
+  // second MFMA per key block with the rounding remainders as the Q operand (hi + lo carries 16
+  // significant bits) and the same A operand, the chunk's widened K.
+  // (D=64: four chunks in all, and registers are scarcer where the tables change along the keys)
+    constexpr int kMaxLo = D == 64 ? 2 : kMaxLoAny;
+  u32x4_t qlo[CHAN ? kMaxLo : 1];
+  // chunk of slot s in bits 4s..4s+2 (slots fill from 0), slots in use in bits 16..18 (wave-uniform)
+  u32 lo_info = 0u;
   // (called from two places: force the inlining, or its captures would live in memory)
   // (pre: the raw values were requested into qb earlier -- the prologue does, to overlap the
   // trip with its other loads)
@@ -382,6 +404,17 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     float qsum[NSK], zb = 0.f;
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
+    int slot_of[CHAN ? NCH : 1];   // remainder slot of chunk ch, or -1 (wave-uniform)
+    if constexpr (CHAN) {
+      // the segment's chunks with a remainder pass, chosen in the prologue
+      // (one 8-byte read: slot + 1 of chunk ch in bits 4ch..4ch+2 of the first word)
+      const uint2 info = *reinterpret_cast<const uint2 *>(&lds_clo[seg * 2]);
+      const u32 slots = __builtin_amdgcn_readfirstlane(info.x);
+      lo_info = __builtin_amdgcn_readfirstlane(info.y);
+#pragma unroll
+      for (int ch = 0; ch < NCH; ++ch) slot_of[ch] = (int)((slots >> (4 * ch)) & 7u) - 1;
+      qlo[0] = u32x4_t{0u, 0u, 0u, 0u};   // (slot 0 is multiplied whether in use or not)
+    }
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
       const int oct = k_octet<GK>(ch, half);
@@ -390,6 +423,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       if constexpr (KEEP_Q) raw = qraw[ch];
       else raw = decltype(pre)::value ? qb[ch] : *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
       float sk[8];
+      u32x4_t lo4 = {0u, 0u, 0u, 0u};
+      const bool with_lo = CHAN && slot_of[CHAN ? ch : 0] >= 0;   // (wave-uniform)
       if constexpr (CHAN) {
         const float *tk = lds_tab + (seg * TR + 0) * D + oct * 8;
         const float4 s0 = *reinterpret_cast<const float4 *>(tk), s1 = *reinterpret_cast<const float4 *>(tk + 4);
@@ -402,11 +437,23 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         const u32 lo = (raw[d0 >> 1] >> (16 * (d0 & 1))) << 16, hi = (raw[d1 >> 1] >> (16 * (d1 & 1))) << 16;
         u32 pair = (lo >> 16) | hi;
         if constexpr (CHAN) {
-          // q[d] * sk[d], rounded to bf16 like any MFMA operand
-          pair = pack_bf16_rne(u2f(lo) * sk[d0], u2f(hi) * sk[d1]);
+          // q[d] * sk[d], rounded to bf16 like any MFMA operand; what the rounding left behind
+          // (exact in fp32, then rounded to bf16 itself) is the operand of the remainder pass
+          const float f0 = u2f(lo) * sk[d0], f1 = u2f(hi) * sk[d1];
+          pair = pack_bf16_rne(f0, f1);
+          if (with_lo) lo4[j2] = pack_bf16_rne(f0 - u2f(pair << 16), f1 - u2f(pair & 0xffff0000u));
         }
         qb[ch][j2] = pair;
         qsum[ch / (GK / 16)] += u2f(pair << 16) + u2f(pair & 0xffff0000u);
+      }
+      if constexpr (CHAN) {
+        if (with_lo) {
+#pragma unroll
+          for (int sl = 0; sl < kMaxLo; ++sl)
+            if (slot_of[ch] == sl) qlo[sl] = lo4;
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) qsum[0] += u2f(lo4[j2] << 16) + u2f(lo4[j2] & 0xffff0000u);
+        }
       }
       if (k_affine) {   // the K zero-points against the rounded operands, for the segment's logit constant
         const float *tz = lds_tab + (seg * TR + 1) * D + oct * 8;
@@ -418,14 +465,21 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
           zb = __builtin_fmaf(u2f(pair << 16), zk[KCodec<BITS>::slot_d(2 * j2)], zb);
           zb = __builtin_fmaf(u2f(pair & 0xffff0000u), zk[KCodec<BITS>::slot_d(2 * j2 + 1)], zb);
         }
+        if (with_lo) {
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) {
+            zb = __builtin_fmaf(u2f(lo4[j2] << 16), zk[KCodec<BITS>::slot_d(2 * j2)], zb);
+            zb = __builtin_fmaf(u2f(lo4[j2] & 0xffff0000u), zk[KCodec<BITS>::slot_d(2 * j2 + 1)], zb);
+          }
+        }
       }
       if constexpr (CHAN) __builtin_amdgcn_sched_barrier(0);   // one chunk's table entries in registers at a time
     }
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
-    if constexpr (CHAN) qbias = -p.scale_log2e * (zb + __shfl_xor(zb, 32, 64));
+    if constexpr (CHAN) qbias = -p.scale_log2e * (zb + __shfl_xor(zb, 32, 64) + KCodec<BITS>::kOff * qsum[0]);
 #pragma unroll
-    for (int s = 0; s < NSK; ++s) {
+    for (int s = 0; s < (CHAN ? 0 : NSK); ++s) {
       u32 b0, b1, b2;
       split3_bf16(qsum[s], b0, b1, b2);
       if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
@@ -607,7 +661,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     };
     // keys of the merged run carry values, not code images: no image factor, no offset terms
     const bool merged = merged_tile(tile);
-    if (seg < NSK) {
+    if (!CHAN && seg < NSK) {   // (per-channel tables: one factor for all keys, no rank-1 term)
       par[P_CK + seg * BN + key] = merged ? p.scale_log2e : ck_of(ksc);
       u32 a0, a1, a2;
       split3_bf16(merged ? 0.f : -(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
@@ -617,7 +671,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     }
     if (vseg < NSV) {
       const int seg = vseg;
-      if (FOLD_SV) {
+      if (FOLD_SV && !CHAN) {
         u32 l0, l1, l2;
         split3_bf16(__builtin_amdgcn_logf(vsc) * __builtin_amdgcn_rcpf(ck_of(ksc0)), l0, l1, l2);
         lds_kz[(sl * NSK * BN + key) * 2 + 1] = u32x4_t{l0 | (l1 << 16), l2, 0u, 0u};
@@ -756,6 +810,58 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       lds_tab[(seg * TR + 4) * D + d] =
           seg ? lds_tab[((seg - 1) * TR + 2) * D + d] * __builtin_amdgcn_rcpf(lds_tab[(seg * TR + 2) * D + d]) : 1.f;
     }
+    // Chunks that get a remainder pass: largest K scale of the chunk's 16 channels (the two
+    // octets that the lane halves contract together) >= kLoRatio * mean K scale of the head; at
+    // most kMaxLo of them, the largest first.  2*NCH adjacent lanes per segment, one octet each
+    // (the last wavefronts', which have the least of the loop above).
+    {
+      constexpr int GL = 2 * NCH;                      // lanes per segment: (chunk, lane half)
+      const int rt = NT - 1 - tid;                     // (reversed: lane groups stay aligned, NT is a multiple of 64)
+      const int seg = rt / GL, gl = rt % GL;
+      if (seg < (p.nseg + 64 / GL - 1) / (64 / GL) * (64 / GL)) {   // whole wavefronts: the exchanges below need every lane
+        const int sg = min(seg, p.nseg - 1);
+        const float4 *tk = reinterpret_cast<const float4 *>(lds_tab + (sg * TR + 0) * D + k_octet<GK>(gl >> 1, gl & 1) * 8);
+        const float4 a = tk[0], b = tk[1];
+        const float e[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        float mx = 0.f, tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { mx = fmaxf(mx, __builtin_fabsf(e[j])); tot += __builtin_fabsf(e[j]); }
+        mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+#pragma unroll
+        for (int off = 1; off < GL; off <<= 1) tot += __shfl_xor(tot, off, 64);
+        float w[NCH];
+        const int base = (threadIdx.x & 63) / GL * GL;   // first lane of the group (in hardware lane order)
+        // (rt reverses the lane order inside a wavefront: chunk c sits at lanes base + GL-1-2c and -2c-1)
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) w[ch] = __shfl(mx, base + GL - 1 - 2 * ch, 64);
+        const float thr = kLoRatio * tot * (1.f / D);
+        int so[NCH], cl[kMaxLo], n = 0;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) so[ch] = -1;
+#pragma unroll
+        for (int sl = 0; sl < kMaxLo; ++sl) {
+          int best = -1;
+          float bw = 0.f;
+#pragma unroll
+          for (int ch = 0; ch < NCH; ++ch)
+            if (w[ch] >= thr && so[ch] < 0 && (best < 0 || w[ch] > bw)) { best = ch; bw = w[ch]; }
+#pragma unroll
+          for (int ch = 0; ch < NCH; ++ch)
+            if (ch == best) so[ch] = sl;
+          cl[sl] = best < 0 ? 0 : best;
+          n += best >= 0;
+        }
+        u32 slots = 0u, info = (u32)n << 16;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) slots |= (u32)(so[ch] + 1) << (4 * ch);
+#pragma unroll
+        for (int sl = 0; sl < kMaxLo; ++sl) info |= (u32)cl[sl] << (4 * sl);
+        if (gl == 0 && seg < p.nseg) {
+          lds_clo[seg * 2] = slots;
+          lds_clo[seg * 2 + 1] = info;
+        }
+      }
+    }
     __syncthreads();
   }
   load_q(max(cur_a.seg, p.nconv), std::true_type{});   // (the merged run is attended with the base segment's tables)
@@ -881,7 +987,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   };
   auto load_scales = [&](int kb) {
 #pragma unroll
-    for (int s = 0; s < (HOIST ? NSK : 0); ++s)
+    for (int s = 0; s < ((HOIST && !CHAN) ? NSK : 0); ++s)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
@@ -912,19 +1018,49 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
     for (int s = 0; s < NSK; ++s) {
-      // starts the accumulator with the zero-point term (see bq above)
       floatx16_t zero;
 #pragma unroll
       for (int j = 0; j < 16; ++j) zero[j] = 0.f;
-      sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
-                                                            __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+      if constexpr (CHAN) {
+        // The key side of the rank-1 term is a constant here and lives in qbias.  In its place:
+        // the remainder pass of the chunk with the largest outlier scale -- that chunk's K operand
+        // against q_lo.  Issued whether or not the segment has such a chunk (q_lo is zero then,
+        // and names chunk 0): a branch here would stand between the LDS requests of the chunk
+        // loop and their MFMAs.
+        const u32x4_t alo0 = *reinterpret_cast<const u32x4_t *>(&kx[krow_i * KXS + (half * NCH + (int)(lo_info & 7u)) * 8]);
+        sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, alo0),
+                                                              __builtin_bit_cast(bf16x8_t, qlo[0]), zero, 0, 0, 0);
+      } else {
+        // starts the accumulator with the zero-point term (see bq above)
+        sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
+                                                              __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+      }
     }
     const uint16_t *krow = &kx[krow_i * KXS];
+    // (the second slot's K operand is requested like the first: no branch ahead of the chunk loop)
+    u32x4_t alo1 = {0u, 0u, 0u, 0u};
+    if constexpr (CHAN) alo1 = *reinterpret_cast<const u32x4_t *>(&krow[(half * NCH + (int)((lo_info >> 4) & 7u)) * 8]);
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
       const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[k_octet<GK>(ch, half) * 8]);
       sacc[kb][ch / (GK / 16)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
           __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][ch / (GK / 16)], 0, 0, 0);
+    }
+    if constexpr (CHAN) {
+      // further remainder passes: more than one chunk with an outlier scale
+      const int nlo = (int)(lo_info >> 16);
+      if (nlo > 1) {
+        sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, alo1),
+                                                              __builtin_bit_cast(bf16x8_t, qlo[1]), sacc[kb][0], 0, 0, 0);
+#pragma unroll
+        for (int sl = 2; sl < kMaxLo; ++sl) {
+          if (sl >= nlo) break;
+          const int c = (int)((lo_info >> (4 * sl)) & 7u);
+          const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[(half * NCH + c) * 8]);
+          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                __builtin_bit_cast(bf16x8_t, qlo[sl]), sacc[kb][0], 0, 0, 0);
+        }
+      }
     }
     __builtin_amdgcn_s_setprio(0);
   };
@@ -932,13 +1068,15 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // logits -> P'^T operands of one block: online softmax against a lazily moved reference
   auto softmax = [&](int kb) {
     float z[16];
+    // CHAN: one factor for every key (keys of the merged run carry values, not code images)
+    const float ck_all = in_merged ? p.scale_log2e : p.scale_log2e * KCodec<BITS>::kMul;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       float v = CHAN ? (in_merged ? 0.f : qbias) - m_ref : -m_ref;
 #pragma unroll
       for (int s = 0; s < NSK; ++s) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        v = __builtin_fmaf(HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key], sacc[kb][s][i], v);
+        v = __builtin_fmaf(CHAN ? ck_all : HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key], sacc[kb][s][i], v);
       }
       z[i] = v;
     }
@@ -1152,7 +1290,7 @@ int device_cus();
 
 template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, bool SEGS>
 void launch_shape(const AttnParams &p, hipStream_t st) {
-  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * kChanTableRows * D * 4 : 0);
+  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV, CHAN>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * (kChanTableRows * D + 2) * 4 : 0);
   static_assert(lds_bytes <= 160 * 1024, "LDS budget");
   // above 64 KiB the limit has to be raised, once per device the process launches on
   static bool configured[64] = {false};
