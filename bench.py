@@ -6,11 +6,16 @@ and V [2,16,10521,128] bf16 to INT4 group-128 asymmetric, then fused dequant
 attention of the final scale's 4096 queries over all 10521 packed keys.  Inputs
 are resident in HBM before the timed region.  Prints ONE JSON line.
 
-After the timed region (and outside `value`) it also replays benchmark configuration 5,
-one image batch of the Infinity schedule through the pre-allocated mixed-bit
-cache (append + attend per scale), and reports its latency per image.
+Before the W warm-up steps the same step runs untimed until 150 ms of GPU work have
+passed, whatever W is: the first ~50 ms after idle run at lower clocks.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c5] [--no-c3] [--no-rule]
+After the timed region (and outside `value`): the quantize+pack kernel and the
+unpack+dequant kernel of configuration 4 timed as back-to-back launches between one
+event pair (kernel time without the dispatch gaps); the CPU baseline (1 thread and all
+threads, per stage, median of 3) with the parity check of the timed GPU results against
+it; and legs for configurations 2, 3 and 5 and for the shipped JSON rules.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c2] [--no-c3] [--no-c5] [--no-rule]
 """
 import argparse
 import json
@@ -42,28 +47,53 @@ def algorithmic_bytes():
     return quant_pack, kv_read, attn_flops
 
 
-def cpu_baseline(torch, O, k0, v0, q0, threads):
-    """The CPU oracle timed on this host: full-size quantize+pack of K and V,
-    unpack+dequant of both, and bf16 SDPA on a 512-query sample (scaled x8)."""
+def cpu_model():
+    try:
+        for line in open('/proc/cpuinfo'):
+            if line.lower().startswith('model name'):
+                return line.split(':', 1)[1].strip()
+    except OSError:
+        pass
+    return 'unknown'
+
+
+def _median(v):
+    v = sorted(v)
+    return v[len(v) // 2]
+
+
+def cpu_baseline(torch, O, k0, v0, q0, threads, reps=3):
+    """The CPU oracle timed on this host, per stage, median of `reps` runs, with all the
+    threads the box gives this process and with one thread: full-size quantize+pack of K and
+    V, unpack+dequant of both, bf16 attention of the 4096 queries (all of them with all
+    threads; a 512-query sample scaled x8 with one thread, to bound the run time)."""
+    scale = 1.0 / math.sqrt(D)
+    res, keep = {}, None
+    for label, nthreads, nq in (('all_threads', threads, LQ), ('one_thread', 1, 512)):
+        torch.set_num_threads(nthreads)
+        tq, td, ta = [], [], []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            kq, ks, kz = O.quant_groupwise(k0, GROUP, BITS, True)
+            kw, kmeta = O.pack_last_dim(kq, BITS)
+            vq, vs, vz = O.quant_groupwise(v0, GROUP, BITS, True)
+            vw, vmeta = O.pack_last_dim(vq, BITS)
+            t1 = time.perf_counter()
+            kd = O.dequant_groupwise(O.unpack_last_dim(kw, kmeta), ks, kz, GROUP)
+            vd = O.dequant_groupwise(O.unpack_last_dim(vw, vmeta), vs, vz, GROUP)
+            t2 = time.perf_counter()
+            ref = O.attention_ref(q0[:, :, :nq], kd, vd, scale)
+            t3 = time.perf_counter()
+            tq.append((t1 - t0) / 2)
+            td.append(t2 - t1)
+            ta.append((t3 - t2) * (LQ / nq))
+        res[label] = {'threads': nthreads, 'quant_pack_s_per_tensor': round(_median(tq), 4),
+                      'unpack_dequant_s_both': round(_median(td), 4), 'attention_s_4096_queries': round(_median(ta), 4),
+                      'attention_queries_timed': nq}
+        if keep is None:
+            keep = {'kw': kw, 'ks': ks, 'kz': kz, 'vw': vw, 'vs': vs, 'vz': vz, 'kd': kd, 'vd': vd, 'ref': ref}
     torch.set_num_threads(threads)
-    t0 = time.perf_counter()
-    kq, ks, kz = O.quant_groupwise(k0, GROUP, BITS, True)
-    kw, kmeta = O.pack_last_dim(kq, BITS)
-    t1 = time.perf_counter()
-    vq, vs, vz = O.quant_groupwise(v0, GROUP, BITS, True)
-    vw, vmeta = O.pack_last_dim(vq, BITS)
-    t2 = time.perf_counter()
-    kd = O.dequant_groupwise(O.unpack_last_dim(kw, kmeta), ks, kz, GROUP)
-    vd = O.dequant_groupwise(O.unpack_last_dim(vw, vmeta), vs, vz, GROUP)
-    t3 = time.perf_counter()
-    nq = 512
-    ref = O.attention_ref(q0[:, :, :nq], kd, vd, 1.0 / math.sqrt(D))
-    t4 = time.perf_counter()
-    t_quant = (t2 - t0) / 2
-    t_attn = (t3 - t2) + (t4 - t3) * (LQ / nq)
-    return {'kw': kw, 'ks': ks, 'kz': kz, 'vw': vw, 'ref': ref, 'nq': nq,
-            't_quant_pack_per_tensor_s': t_quant, 't_unpack_dequant_s': t3 - t2, 't_sdpa_sample_s': t4 - t3,
-            't_attn_equiv_s': t_attn}
+    return res, keep
 
 
 def c5_latency(torch, dev, passes=10, warm=3):
@@ -101,6 +131,69 @@ def c5_latency(torch, dev, passes=10, warm=3):
             'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes}
 
 
+def timed_launches(torch, fn, reps=20, warm=5, rounds=5):
+    """Seconds per call of fn: `reps` back-to-back launches between one event pair on the
+    current stream, median of `rounds` such measurements."""
+    for _ in range(warm):
+        fn()
+    ts = []
+    for _ in range(rounds):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1) / reps * 1e-3)
+    return _median(ts)
+
+
+def c2_rates(torch, dev):
+    """Config 2: VAR-d16 batch shape, K/V bf16 [64,16,680,64], INT4 asymmetric, K in groups of
+    32 channels, V in groups of 64 (per token), 8 codes per word; the final-scale 256 queries
+    over all 680 keys.  Two K and two V tensors are cycled (4 x 89 MB > the 256 MB Infinity
+    Cache) so that the quantizer reads HBM."""
+    import varq_oracle as O
+    from var_q_amd import ops
+    B2, H2, L2, D2, LQ2, bits = 64, 16, 680, 64, 256, 4
+    n_el = B2 * H2 * L2 * D2
+    ks_in = [O.synth_kv((B2, H2, L2, D2), 1002 + i, dtype=torch.bfloat16).to(dev) for i in range(2)]
+    vs_in = [O.synth_kv((B2, H2, L2, D2), 2002 + i, dtype=torch.bfloat16).to(dev) for i in range(2)]
+    q = torch.randn(B2, H2, LQ2, D2, device=dev, generator=torch.Generator(device=dev).manual_seed(3002)).bfloat16()
+    out = {'workload': 'config 2: VAR-d16 K/V bf16 [64,16,680,64] -> INT4 asymmetric, K group 32, V group 64; '
+                       'final-scale 256 queries over 680 keys'}
+    rowmap = [1, 1, B2 * H2 * L2, 0, 0, 1, 0, -1]
+    packed = {}
+    for name, xs, g in (('k_g32', ks_in, 32), ('v_g64', vs_in, 64)):
+        w, sc, zp = ops.quant_pack_rows(xs[0], g, bits, True)
+        packed[name] = (w, sc, zp)
+        i = [0]
+
+        def qfn():
+            i[0] ^= 1
+            ops.quant_pack_rows_into(xs[i[0]], g, bits, True, 1e-12, w, sc, zp, rowmap)
+        t_q = timed_launches(torch, qfn)
+        ops.quant_pack_rows_into(xs[0], g, bits, True, 1e-12, w, sc, zp, rowmap)     # (leave set 0 in the buffers)
+        groups = n_el // g
+        qbytes = n_el * 2 + n_el * bits // 8 + groups * 8
+        t_d = timed_launches(torch, lambda: ops.dequant(w, sc, zp, D2, bits, torch.bfloat16))
+        dbytes = n_el * bits // 8 + groups * 8 + n_el * 2
+        out[name] = {'quant_pack_us': round(t_q * 1e6, 1), 'quant_pack_GBps': round(qbytes / t_q / 1e9, 1),
+                     'quant_pack_frac_hbm_peak': round(qbytes / t_q / 1e9 / HBM_PEAK_GBPS, 4),
+                     'quant_pack_tokens_per_s': round(B2 * L2 / t_q, 1),
+                     'unpack_dequant_us': round(t_d * 1e6, 1), 'unpack_dequant_GBps': round(dbytes / t_d / 1e9, 1),
+                     'unpack_dequant_frac_hbm_peak': round(dbytes / t_d / 1e9 / HBM_PEAK_GBPS, 4)}
+    o = torch.empty_like(q)
+    (kw, ksc, kzp), (vw, vsc, vzp) = packed['k_g32'], packed['v_g64']
+    t_a = timed_launches(torch, lambda: ops.fused_attn(q, kw, ksc, kzp, vw, vsc, vzp, bits, bits, L2, 1.0 / math.sqrt(D2), out=o))
+    flops = 4 * B2 * H2 * LQ2 * L2 * D2
+    kv = sum(n_el * bits // 8 + (n_el // g) * 8 for g in (32, 64))
+    out['fused_attn'] = {'us': round(t_a * 1e6, 1), 'TFLOPs': round(flops / t_a / 1e12, 1),
+                         'frac_mfma_peak': round(flops / t_a / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                         'kv_read_GBps': round(kv / t_a / 1e9, 1), 'query_tokens_per_s': round(B2 * LQ2 / t_a, 1)}
+    return out
+
+
 def c3_rates(torch, dev, reps=20, warm=5):
     """Config 3: VAR-d30 shape, K/V bf16 [32,30,680,64], quantized per (head, channel) over
     batch and tokens: (i) INT2 asymmetric, (ii) INT8 symmetric (the reference's
@@ -112,16 +205,7 @@ def c3_rates(torch, dev, reps=20, warm=5):
     k, v = (torch.randn(B3, H3, L3, D3, device=dev, generator=gd).bfloat16() for _ in range(2))
     q = torch.randn(B3, H3, LQ3, D3, device=dev, generator=gd).bfloat16()
 
-    def timed(fn):
-        for _ in range(warm):
-            fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3
+    timed = lambda fn: timed_launches(torch, fn, reps, warm)
 
     out = {'workload': 'config 3: VAR-d30 K/V bf16 [32,30,680,64], one (scale, zp) per (head, channel); '
                        'final-scale 256 queries'}
@@ -197,12 +281,36 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
     return out
 
 
+def attention_check(torch, dev, out, q, kd, vd, ref, scale):
+    """The timed attention output against the oracle (cosine) and against an fp64 evaluation of
+    the same formula on the oracle's dequantized operands (max-abs in units of the output
+    range), as the parity tests do; the fp64 softmax runs through torch on the GPU, one head at
+    a time (checker plumbing)."""
+    got = out.double().cpu()
+    refd = ref.double()
+    exact = torch.empty_like(refd)
+    for b in range(q.shape[0]):
+        for h in range(q.shape[1]):
+            s = (q[b, h].double().to(dev) @ kd[b, h].double().to(dev).T) * scale
+            exact[b, h] = (torch.softmax(s, dim=-1) @ vd[b, h].double().to(dev)).cpu()
+    span = max(1.0, float(exact.abs().max()))
+    return {
+        'attn_cosine_vs_oracle': round(float(torch.nn.functional.cosine_similarity(got.flatten(), refd.flatten(), dim=0)), 6),
+        'attn_output_range': round(span, 3),
+        'attn_maxabs_vs_fp64_over_range': round(float((got - exact).abs().max()) / span, 5),
+        'oracle_maxabs_vs_fp64_over_range': round(float((refd - exact).abs().max()) / span, 5),
+        'attn_maxabs_vs_oracle_over_range': round(float((got - refd).abs().max()) / span, 5),
+        'queries_checked': int(q.shape[2]),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
+    ap.add_argument('--no-c2', action='store_true', help='skip the config-2 rates leg (profiling runs)')
     ap.add_argument('--no-c5', action='store_true', help='skip the config-5 latency leg (profiling runs)')
     ap.add_argument('--no-c3', action='store_true', help='skip the config-3 rates leg (profiling runs)')
     ap.add_argument('--single-launches', action='store_true', help='quantize K and V in two launches instead of one')
@@ -246,15 +354,19 @@ def main():
 
     PAIR = not args.single_launches
 
-    def step(i, ev=None):
+    def quantize(i):
         s, t = i % NBUF, outs[i % NBUF]
-        if ev: ev[0].record()
         if PAIR:   # K and V of the step in one launch, as the cache append does
             ops.quant_pack_rows_pair_into(ks_in[s], vs_in[s], GROUP, BITS, True, 1e-12, (t['kw'], t['ks'], t['kz']),
                                           (t['vw'], t['vs'], t['vz']), rowmap)
         else:
             ops.quant_pack_rows_into(ks_in[s], GROUP, BITS, True, 1e-12, t['kw'], t['ks'], t['kz'], rowmap)
             ops.quant_pack_rows_into(vs_in[s], GROUP, BITS, True, 1e-12, t['vw'], t['vs'], t['vz'], rowmap)
+
+    def step(i, ev=None):
+        t = outs[i % NBUF]
+        if ev: ev[0].record()
+        quantize(i)
         if ev: ev[1].record()
         ops.fused_attn(q, t['kw'], t['ks'], t['kz'], t['vw'], t['vs'], t['vz'], BITS, BITS, L, scale, out=o)
         if ev: ev[2].record()
@@ -267,6 +379,18 @@ def main():
         torch.cuda.synchronize()
         del ca, cb
 
+    # clocks: the same step, untimed, until 150 ms of GPU work have passed
+    prewarm_steps, e0 = 0, torch.cuda.Event(enable_timing=True)
+    e0.record()
+    while True:
+        for _ in range(20):
+            step(prewarm_steps)
+            prewarm_steps += 1
+        e1 = torch.cuda.Event(enable_timing=True)
+        e1.record()
+        torch.cuda.synchronize()
+        if e0.elapsed_time(e1) >= 150.0 or prewarm_steps >= 2000:
+            break
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -281,8 +405,32 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
 
     # events sit on the stream the kernels are launched on (torch's current stream)
-    t_quant = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps * 1e-3 / 2   # two launches (K, V) per step
+    t_quant_step = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps * 1e-3 / 2   # per tensor, dispatch gap included
     t_at = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps * 1e-3
+
+    # ---- the HBM-bound kernels of configuration 4 as back-to-back launches between one event pair:
+    #      kernel time without the gap between a recorded event and the next dispatch
+    cnt = [0]
+
+    def quantize_next():
+        quantize(cnt[0])
+        cnt[0] += 1
+    t_quant = timed_launches(torch, quantize_next, reps=40, warm=8) / 2          # per tensor
+    deq_out = torch.empty((B, H, L, D), dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    shape4, strides4 = _lib.i64arr([B, H, L, D]), _lib.i64arr([H * L, L, 1, 1])
+
+    def dequant_next():   # the C ABI directly: no allocation and no Python wrapper between the launches
+        t = outs[cnt[0] % NBUF]
+        cnt[0] += 1
+        _lib.check(lib.varq_dequant(t['kw'].data_ptr(), None, t['ks'].data_ptr(), t['kz'].data_ptr(), shape4, strides4,
+                                    GROUP, BITS, None, deq_out.data_ptr(), 1, stream), 'varq_dequant')
+    for i in range(NBUF):
+        quantize(i)
+    t_deq = timed_launches(torch, dequant_next, reps=40, warm=8)
+    n = B * H * L * D
+    deq_bytes = n * BITS // 8 + (n // GROUP) * 8 + n * 2           # packed codes + scale/zp in, bf16 out
 
     # ---- CPU baseline + parity of the timed results against it ------------------
     cpu = None
@@ -291,24 +439,32 @@ def main():
         threads = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
         step(0)
         torch.cuda.synchronize()
-        c = cpu_baseline(torch, O, k0, v0, q0, threads)
+        stages, c = cpu_baseline(torch, O, k0, v0, q0, threads)
         t = outs[0]
         words_ok = bool(torch.equal(t['kw'].cpu(), c['kw']) and torch.equal(t['vw'].cpu(), c['vw'])
-                        and torch.equal(t['ks'].cpu(), c['ks']) and torch.equal(t['kz'].cpu(), c['kz']))
-        got, ref = o[:, :, :c['nq']].double().cpu(), c['ref'].double()
-        cosine = float(torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0))
-        checked = {'packed_words_scales_zps_bit_exact': words_ok, 'attn_cosine_vs_oracle': round(cosine, 6)}
-        if not words_ok or cosine < 0.9995:
+                        and torch.equal(t['ks'].cpu(), c['ks']) and torch.equal(t['kz'].cpu(), c['kz'])
+                        and torch.equal(t['vs'].cpu(), c['vs']) and torch.equal(t['vz'].cpu(), c['vz']))
+        cnt[0] = 0            # input set 0 again: the one the CPU leg dequantized
+        dequant_next()
+        torch.cuda.synchronize()
+        deq_ok = bool(torch.equal(deq_out.cpu(), c['kd'].bfloat16()))
+        checked = {'packed_words_scales_zps_bit_exact': words_ok, 'unpack_dequant_bf16_bit_exact': deq_ok}
+        checked.update(attention_check(torch, dev, o, q0, c['kd'], c['vd'], c['ref'], scale))
+        bad = (not words_ok or not deq_ok or checked['attn_cosine_vs_oracle'] < 0.9995 or checked['attn_maxabs_vs_fp64_over_range'] > 2e-2
+               or checked['attn_maxabs_vs_oracle_over_range'] > 2e-2 + checked['oracle_maxabs_vs_fp64_over_range'])
+        if bad:
             print('bench.py: GPU results differ from the oracle: %r' % checked, file=sys.stderr)
             sys.exit(1)
+        a = stages['all_threads']
+        t_cpu_attn = a['unpack_dequant_s_both'] + a['attention_s_4096_queries']
         cpu = {
-            'value': round(kv_bytes / c['t_attn_equiv_s'] / 1e9, 4), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
-            'sample': ('torch-CPU oracle on this host: full-size INT4 g128 quantize+pack of K and V '
-                       '(%.3f s per tensor = %.2f GB/s), unpack+dequant of both (%.3f s), bf16 SDPA on 512 of the '
-                       '4096 queries (%.3f s, scaled x8); value = packed-KV bytes / (dequant + scaled SDPA)'
-                       % (c['t_quant_pack_per_tensor_s'], quant_bytes / c['t_quant_pack_per_tensor_s'] / 1e9,
-                          c['t_unpack_dequant_s'], c['t_sdpa_sample_s'])),
-            'pack_GBps': round(quant_bytes / c['t_quant_pack_per_tensor_s'] / 1e9, 3),
+            'value': round(kv_bytes / t_cpu_attn / 1e9, 4), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
+            'cpu_model': cpu_model(), 'os_cpu_count': os.cpu_count(),
+            'sample': ('torch-CPU oracle on this host, median of 3 runs per stage: full-size INT4 g128 quantize+pack of K and '
+                       'V, unpack+dequant of both, bf16 attention of all 4096 queries (one thread: 512 queries scaled x8); '
+                       'value = packed-KV bytes / (unpack+dequant + attention) with all threads'),
+            'pack_GBps': round(quant_bytes / a['quant_pack_s_per_tensor'] / 1e9, 3),
+            'stages': stages,
         }
 
     attn_tflops = attn_flops / t_at / 1e12
@@ -329,20 +485,34 @@ def main():
         'dtype': 'bf16', 'dtype_detail': 'bf16 MFMA operands holding exact int4 codes, fp32 scales and accumulation', 'data': 'synthetic',
         'config': {'workload': 'config 4: Infinity-2B KV [B=2,H=16,L=10521,D=128] bf16 -> INT4 group-128 asymmetric '
                                'quantize+pack of K and V, then fused dequant attention of the final 4096 queries',
-                   'B': B, 'H': H, 'L': L, 'D': D, 'Lq': LQ, 'bits': BITS, 'group': GROUP, 'input_sets_cycled': NBUF},
+                   'B': B, 'H': H, 'L': L, 'D': D, 'Lq': LQ, 'bits': BITS, 'group': GROUP, 'input_sets_cycled': NBUF,
+                   'prewarm_steps_untimed': prewarm_steps},
         'attn_kv_read_frac_hbm_peak': round(kv_gbps / HBM_PEAK_GBPS, 5),
         'attn_ms': round(t_at * 1e3, 4), 'attn_TFLOPs': round(attn_tflops, 2),
         'attn_query_tokens_per_s': round(B * LQ / t_at, 1),
         'pack_GBps': round(pack_gbps, 2), 'pack_frac_hbm_peak': round(pack_gbps / HBM_PEAK_GBPS, 4),
         'pack_us_per_tensor': round(t_quant * 1e6, 2), 'pack_tokens_per_s': round(B * L / t_quant, 1),
+        'pack_us_per_tensor_in_step': round(t_quant_step * 1e6, 2),
+        'unpack_dequant_GBps': round(deq_bytes / t_deq / 1e9, 2), 'unpack_dequant_frac_hbm_peak': round(deq_bytes / t_deq / 1e9 / HBM_PEAK_GBPS, 4),
+        'unpack_dequant_us_per_tensor': round(t_deq * 1e6, 2),
         'roofline': {'kernel': 'fused_attn_kernel<128,4,128,128,token scales>', 'bound': 'mfma', 'achieved': round(attn_tflops, 2),
                      'peak': MFMA_BF16_PEAK_TFLOPS, 'unit': 'TFLOP/s', 'frac': round(attn_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                     'traffic': None if not traffic else traffic.get('fused_attn')},
+                     'traffic': None if not traffic else traffic.get('fused_attn'),
+                     'timing': 'HIP events around each of the timed steps\' launches'},
         'roofline_pack': {'kernel': 'quant_pack_rows32_kernel<bf16,4,asym,4 lanes per group,dense>', 'bound': 'hbm', 'achieved': round(pack_gbps, 2),
                           'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(pack_gbps / HBM_PEAK_GBPS, 4),
                           'traffic': None if not traffic else traffic.get('quant_pack_rows', 0) // (1 if PAIR else 2) or None,
-                          'tensors_per_launch': 2 if PAIR else 1},
+                          'tensors_per_launch': 2 if PAIR else 1,
+                          'timing': '40 back-to-back launches over the %d cycled input sets between one HIP event pair, median '
+                                    'of 5 (inside the timed steps, one launch between its own events: '
+                                    'pack_us_per_tensor_in_step)' % NBUF},
+        'roofline_dequant': {'kernel': 'dequant_kernel<int4 words, group 128, bf16 out>', 'bound': 'hbm',
+                             'achieved': round(deq_bytes / t_deq / 1e9, 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                             'frac': round(deq_bytes / t_deq / 1e9 / HBM_PEAK_GBPS, 4),
+                             'traffic': None if not traffic else traffic.get('dequant'),
+                             'timing': '40 back-to-back launches through the C ABI between one HIP event pair, median of 5'},
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
+        'config2_rates': None if args.no_c2 else c2_rates(torch, dev),
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
         'shipped_rule_latency': None if args.no_rule else shipped_rule_latency(torch, dev),
