@@ -15,7 +15,7 @@ event pair (kernel time without the dispatch gaps); the CPU baseline (1 thread a
 threads, per stage, median of 3) with the parity check of the timed GPU results against
 it; and legs for configurations 2, 3 and 5 and for the shipped JSON rules.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c2] [--no-c3] [--no-c5] [--no-rule]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c2] [--no-c3] [--no-c5] [--no-prepare] [--no-rule]
 """
 import argparse
 import json
@@ -227,6 +227,37 @@ def c3_rates(torch, dev, reps=20, warm=5):
     return out
 
 
+def prepare_rates(torch, dev):
+    """Producer side in one pass (qkv_prepare_kernel): the qkv projection output of the last
+    Infinity scale, bf16 [B=2, L=4096, 3, H=16, c=128] -> q normalised, scaled per head and
+    rotated (bf16) and k, v normalised / rotated and quantized to INT4 group 128 into their cache
+    rows.  Four input sets are cycled (4 x 101 MB)."""
+    from var_q_amd import hooks, ops
+    Bp, Lp, Hp, cp, bits, g = 2, 4096, 16, 128, 4, 128
+    gd = torch.Generator(device=dev).manual_seed(6006)
+    xs = [torch.randn(Bp, Lp, 3, Hp, cp, device=dev, generator=gd).bfloat16() for _ in range(4)]
+    cos, sin = hooks.rope2d_tables(cp, [(64, 64)])
+    rope = (cos.to(dev), sin.to(dev))
+    mul = torch.rand(Hp, device=dev, generator=gd) + 1
+    Wp = cp * bits // 32
+    mk = lambda last, dt: torch.empty((Bp, Hp, Lp, last), dtype=dt, device=dev)
+    t = dict(q=mk(cp, torch.bfloat16), kw=mk(Wp, torch.int32), vw=mk(Wp, torch.int32), ks=mk(1, torch.float32),
+             kz=mk(1, torch.float32), vs=mk(1, torch.float32), vz=mk(1, torch.float32))
+    rowmap = [Bp, Lp, Hp, Hp * Lp, 1, Lp, 0, -1]
+    i = [0]
+
+    def fn():
+        i[0] += 1
+        ops.qkv_prepare_append(xs[i[0] % 4], t['q'], g, bits, True, 1e-12, t['kw'], t['ks'], t['kz'], t['vw'], t['vs'], t['vz'],
+                               rowmap, None, mul, True, 1e-12, rope, 0)
+    dt = timed_launches(torch, fn, reps=40, warm=10)
+    rows = Bp * Lp * Hp
+    nbytes = rows * (3 * cp * 2 + cp * 2 + 2 * cp * bits // 8 + 2 * (cp // g) * 8)    # qkv in, q out, packed k and v, scales and zps
+    return {'workload': 'qkv [2,4096,3,16,128] bf16 -> q bf16 (l2-norm, per-head scale, 2-D rotary) + k, v INT4 g128 into the cache',
+            'us': round(dt * 1e6, 1), 'GBps': round(nbytes / dt / 1e9, 1), 'frac_hbm_peak': round(nbytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
+            'tokens_per_s': round(Bp * Lp / dt, 1), 'algorithmic_MB': round(nbytes / 1e6, 2)}
+
+
 def shipped_rule_latency(torch, dev, passes=5, warm=2):
     """The rules of the shipped JSON files (G_SCALE_HEAD_DIM, 8 bits), one layer, per scale
     quantize + cache K and V with the drop-in quantizers, then attend:
@@ -315,6 +346,7 @@ def main():
     ap.add_argument('--no-c3', action='store_true', help='skip the config-3 rates leg (profiling runs)')
     ap.add_argument('--single-launches', action='store_true', help='quantize K and V in two launches instead of one')
     ap.add_argument('--no-rule', action='store_true', help='skip the shipped-rule latency leg (profiling runs)')
+    ap.add_argument('--no-prepare', action='store_true', help='skip the producer-side (qkv_prepare) leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -515,6 +547,7 @@ def main():
         'config2_rates': None if args.no_c2 else c2_rates(torch, dev),
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
+        'qkv_prepare_rates': None if args.no_prepare else prepare_rates(torch, dev),
         'shipped_rule_latency': None if args.no_rule else shipped_rule_latency(torch, dev),
     }
     print(json.dumps(line), flush=True)

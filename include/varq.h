@@ -105,6 +105,7 @@ int varq_quant_pack_rows2(const void *x0, const void *x1, int x_dtype, int64_t n
  *           len of a [B,H,cap,..] buffer is {n, cap - n, len}, a [B,n,H,c] step in
  *           a [B,cap,H,..] buffer {n*H, (cap - n)*H, len*H}.
  *   workspace  >= varq_quant_workspace_bytes(...) bytes, any contents
+ *   scale, zp and workspace are 16-byte aligned
  * bits in 2..8 when only codes are requested, {2,4,8} when words are.
  */
 size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask);

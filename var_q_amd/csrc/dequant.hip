@@ -60,19 +60,113 @@ template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t ele
   }
 }
 
-template <int ODT>
+// U items (octets) per lane, 256 lanes apart: all of a lane's loads are issued before the first
+// of them is used, so a wavefront keeps U times the bytes in flight and the launch has a U-th of
+// the wavefronts (with one item per lane the kernel is bound by wavefront turnover, not by
+// bandwidth: 54-61 % of the HBM peak on the benchmark shapes against 62-70 % with four).
+template <int ODT, int U>
 __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
-  // grid = (tiles of 256 octets, i1, i0): no division to find the block's place
+  // grid = (tiles of 256*U octets, i1, i0): no division to find the block's place
   const int64_t i0 = blockIdx.z, i1 = blockIdx.y;
-  const int o = blockIdx.x * 256 + threadIdx.x;          // octet inside the (i0, i1) pair, < 2^31
+  const int o0 = blockIdx.x * (256 * U) + threadIdx.x;   // first octet inside the (i0, i1) pair, < 2^31
+  const int64_t sbase0 = i0 * p.ss0 + i1 * p.ss1;
+  const int64_t in_base = i0 * p.in_map.os0 + i1 * p.in_map.os1 + p.in_map.off;
+  const int64_t out_base = (i0 * p.n1 + i1) * p.n2;
+  const bool words_ok = (p.c & 7) == 0 && p.words != nullptr &&
+                        (p.bits != 8 || (reinterpret_cast<uintptr_t>(p.words) & 7) == 0);   // (block-uniform)
+  // one scale per channel that does not depend on the token (a per-(head, channel) table), rows of
+  // a power-of-two number of octets: the lane's U items are the same octet column of U tokens
+  // and share one vector of 8 scales and 8 zero-points
+  const bool chan = words_ok && p.group == 1 && p.ss3 == 1 && p.ss2 == 0 && p.c8_shift >= 0 && p.c8 <= 256 &&
+                    ((sbase0 | (int64_t)(reinterpret_cast<uintptr_t>(p.scale) >> 2) |
+                      (int64_t)(reinterpret_cast<uintptr_t>(p.zp) >> 2)) & 3) == 0;
+  const bool fast = words_ok && (p.group & 7) == 0;
+  if (fast || chan) {
+    // packed words: one word (two for 8-bit codes) per item, and one scale and zero-point per
+    // item (groups of whole octets) or the lane's vectors (per-channel tables)
+    int w0[U], w1[U], i2v[U], colv[U];
+    float sv[U], zv[U];
+    bool live[U];
+    float cs[8], cz[8];
+    if (chan) {
+      const int col = o0 & (p.c8 - 1);
+      const float4 *sp = reinterpret_cast<const float4 *>(p.scale + sbase0 + col * 8);
+      const float4 sa = sp[0], sb = sp[1];
+      cs[0] = sa.x; cs[1] = sa.y; cs[2] = sa.z; cs[3] = sa.w; cs[4] = sb.x; cs[5] = sb.y; cs[6] = sb.z; cs[7] = sb.w;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) cz[j] = 0.f;
+      if (p.zp) {
+        const float4 *zq = reinterpret_cast<const float4 *>(p.zp + sbase0 + col * 8);
+        const float4 za = zq[0], zb = zq[1];
+        cz[0] = za.x; cz[1] = za.y; cz[2] = za.z; cz[3] = za.w; cz[4] = zb.x; cz[5] = zb.y; cz[6] = zb.z; cz[7] = zb.w;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int o = o0 + u * 256;
+      live[u] = o < p.octets_per_pair;
+      const int oc = live[u] ? o : 0;
+      int i2, col;
+      if (p.c8_shift >= 0) { i2 = oc >> p.c8_shift; col = oc & (p.c8 - 1); }
+      else { i2 = oc / p.c8; col = oc - i2 * p.c8; }
+      i2v[u] = i2; colv[u] = col;
+      const int32_t *src = p.words + (in_base + i2 * p.in_map.os2) * p.wpr;
+      if (p.bits == 4) { w0[u] = src[col]; w1[u] = 0; }
+      else if (p.bits == 8) { const int2 t = *reinterpret_cast<const int2 *>(src + col * 2); w0[u] = t.x; w1[u] = t.y; }
+      else { w0[u] = src[col >> 1]; w1[u] = 0; }
+      if (!chan) {
+        const int64_t g = sbase0 + i2 * p.ss2 + (col * 8 / p.group) * p.ss3;
+        sv[u] = p.scale[g];
+        zv[u] = p.zp ? p.zp[g] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live[u]) continue;
+      int q[8];
+      if (p.bits == 4) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_sbfe(w0[u], 4 * j, 4);
+      } else if (p.bits == 8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { q[j] = __builtin_amdgcn_sbfe(w0[u], 8 * j, 8); q[4 + j] = __builtin_amdgcn_sbfe(w1[u], 8 * j, 8); }
+      } else {
+        const int w = w0[u] >> ((colv[u] & 1) * 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_sbfe(w, 2 * j, 2);
+      }
+      float f[8];
+      if (chan) {
+        // (the same two operations as the scalar form below, so the results are the same bits)
+        if (p.zp) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) f[j] = ((float)q[j] - cz[j]) * cs[j];
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) f[j] = (float)q[j] * cs[j];
+        }
+      } else if (p.zp) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = ((float)q[j] - zv[u]) * sv[u];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (float)q[j] * sv[u];
+      }
+      store8<ODT>(p.out, (out_base + i2v[u]) * p.c + colv[u] * 8, f, 8);
+    }
+    return;
+  }
+#pragma unroll 1
+  for (int u = 0; u < U; ++u) {
+  const int o = o0 + u * 256;
   if (o >= p.octets_per_pair) return;
   int i2, col;
   if (p.c8_shift >= 0) { i2 = o >> p.c8_shift; col = o & (p.c8 - 1); }
   else { i2 = o / p.c8; col = o - i2 * p.c8; }
   const int ch0 = col * 8;
   const int n_valid = min(8, p.c - ch0);
-  const int64_t in_row = i0 * p.in_map.os0 + i1 * p.in_map.os1 + i2 * p.in_map.os2 + p.in_map.off;
-  const int64_t out_row = (i0 * p.n1 + i1) * p.n2 + i2;
+  const int64_t in_row = in_base + i2 * p.in_map.os2;
+  const int64_t out_row = out_base + i2;
 
   int q[8];
   if (p.codes) {
@@ -102,7 +196,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
     }
   }
 
-  const int64_t sbase = i0 * p.ss0 + i1 * p.ss1 + i2 * p.ss2;
+  const int64_t sbase = sbase0 + i2 * p.ss2;
   float f[8];
   if ((p.group & 7) == 0) {
     const int64_t g = sbase + (ch0 / p.group) * p.ss3;
@@ -140,6 +234,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
     }
   }
   store8<ODT>(p.out, out_row * p.c + ch0, f, ((p.c & 7) == 0) ? 8 : n_valid);
+  }
 }
 
 }  // namespace
@@ -179,14 +274,23 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
   p.c8_shift = -1;
   for (int sh = 0; sh < 20; ++sh)
     if ((1 << sh) == p.c8) p.c8_shift = sh;
-  const int64_t tiles = (p.octets_per_pair + 255) / 256;
+  // four items per lane where a pair has the work for it (the last block's idle lanes weigh less
+  // than the wavefront turnover they save), one otherwise
+  const int U = p.octets_per_pair >= 2048 ? 4 : 1;
+  const int64_t tiles = (p.octets_per_pair + 256 * U - 1) / (256 * U);
   // a pair with few rows wastes lanes of its last block only; pairs map to grid.y/z (limit 65535 each)
-  VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 256 && s[1] <= 65535 && s[0] <= 65535, "dequant: shape exceeds the grid limits");
+  VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 1024 && s[1] <= 65535 && s[0] <= 65535, "dequant: shape exceeds the grid limits");
   dim3 grid((unsigned)tiles, (unsigned)s[1], (unsigned)s[0]);
   hipStream_t st = (hipStream_t)stream;
-  if (out_dtype == VARQ_F32) hipLaunchKernelGGL(dequant_kernel<VARQ_F32>, grid, dim3(256), 0, st, p);
-  else if (out_dtype == VARQ_BF16) hipLaunchKernelGGL(dequant_kernel<VARQ_BF16>, grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL(dequant_kernel<VARQ_F16>, grid, dim3(256), 0, st, p);
+#define VARQ_DEQ(ODT_)                                                                       \
+  do {                                                                                       \
+    if (U == 4) hipLaunchKernelGGL((dequant_kernel<ODT_, 4>), grid, dim3(256), 0, st, p);    \
+    else hipLaunchKernelGGL((dequant_kernel<ODT_, 1>), grid, dim3(256), 0, st, p);           \
+  } while (0)
+  if (out_dtype == VARQ_F32) VARQ_DEQ(VARQ_F32);
+  else if (out_dtype == VARQ_BF16) VARQ_DEQ(VARQ_BF16);
+  else VARQ_DEQ(VARQ_F16);
+#undef VARQ_DEQ
   VARQ_CHECK_LAUNCH("dequant");
   return VARQ_OK;
 }

@@ -13,6 +13,16 @@
 #include "varq_common.h"
 #include <mutex>
 
+#ifndef VARQ_GEN_NRO_MIN
+#define VARQ_GEN_NRO_MIN 256
+#endif
+#ifndef VARQ_FIN_THREADS
+#define VARQ_FIN_THREADS 65536
+#endif
+#ifndef VARQ_GEN_BLOCKS
+#define VARQ_GEN_BLOCKS 2048
+#endif
+
 namespace {
 
 // Order-preserving float <-> uint map so that integer atomicMin/Max implement
@@ -131,23 +141,37 @@ __device__ __forceinline__ Lane decode(const Plan &pl) {
   return l;
 }
 
-// Calls body(row) for every row of this thread, in step order.
-template <typename F>
-__device__ __forceinline__ void for_rows(const Plan &pl, const Lane &l, F body) {
+// Calls body(row, v) for every row of this thread, in step order, with the row's 8 values of
+// this lane's octet.
+template <int DT, typename F>
+__device__ __forceinline__ void for_rows(const GenParams &p, const Plan &pl, const Lane &l, F body) {
   const int s0 = l.z * pl.steps_per_chunk, s1 = min(s0 + pl.steps_per_chunk, pl.steps);
   const int64_t base = (int64_t)l.ko * pl.ko_rs + l.q;
+  const int64_t col8 = l.col * 8;
+  // (one load in flight per lane: issuing two steps' loads before either is used, or the next
+  // row's load ahead of the current row's arithmetic, was measured 5-15 % slower on both phases)
   if (pl.fold_ro) {
     // d2 kept: a step is `sub` consecutive reduced positions
     for (int s = s0; s < s1; ++s) {
       const int ro = s * pl.sub + l.f;
-      if (ro < pl.nro) body(base + (int64_t)ro * pl.ro_rs);
+      if (ro < pl.nro) {
+        const int64_t r = base + (int64_t)ro * pl.ro_rs;
+        float v[8];
+        In8<DT>::load(p.x, r * p.c + col8, v);
+        body(r, v);
+      }
     }
   } else {
     // d2 reduced: a step is `sub` (= R) consecutive rows of one ro
     int ro = s0 / pl.T, t = s0 - ro * pl.T;
     for (int s = s0; s < s1; ++s) {
       const int ri = t * pl.sub + l.f;
-      if (ri < pl.RI) body(base + (int64_t)ro * pl.ro_rs + ri);
+      if (ri < pl.RI) {
+        const int64_t r = base + (int64_t)ro * pl.ro_rs + ri;
+        float v[8];
+        In8<DT>::load(p.x, r * p.c + col8, v);
+        body(r, v);
+      }
       if (++t == pl.T) { t = 0; ++ro; }
     }
   }
@@ -164,9 +188,7 @@ __global__ __launch_bounds__(256) void minmax_tiled_kernel(GenParams p, Plan pl,
 #pragma unroll
   for (int j = 0; j < NV; ++j) { mx[j] = ASYM ? -INFINITY : 0.f; mn[j] = INFINITY; }
   if (l.live) {
-    for_rows(pl, l, [&](int64_t row) {
-      float v[8];
-      In8<DT>::load(p.x, row * p.c + l.col * 8, v);
+    for_rows<DT>(p, pl, l, [&](int64_t, const float (&v)[8]) {
       if (KEEPC) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -189,22 +211,38 @@ __global__ __launch_bounds__(256) void minmax_tiled_kernel(GenParams p, Plan pl,
       if (ASYM) mn[0] = fminf(mn[0], __shfl_xor(mn[0], off, 64));
     }
   }
-  // fold the `sub` row lanes that share q (lane index = (f*lanesQ + lq)*c8p + col)
+  // fold the `sub` row lanes that share q (lane index = (f*lanesQ + lq)*c8p + col, so the
+  // positions f of one (q, col) lie `stride` lanes apart): inside a wavefront by lane exchanges
+  // when the stride is a power of two below 64, the rest -- at most one value per wavefront
+  // then -- through LDS.  (Idle lanes hold the identity of max / min.)
   if (pl.sub > 1) {
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      lds_mx[j * 256 + threadIdx.x] = mx[j];
-      if (ASYM) lds_mn[j * 256 + threadIdx.x] = mn[j];
-    }
-    __syncthreads();
-    if (l.f == 0) {
-      const int stride = pl.lanesQ * pl.c8p;
-      for (int f = 1; f < pl.sub; ++f)
+    const int stride = pl.lanesQ * pl.c8p;
+    int fstep = 1;                       // distance in f between the values still to fold
+    if (stride < 64 && (stride & (stride - 1)) == 0) {
+      for (int off = stride; off < 64; off <<= 1) {
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-          mx[j] = fmaxf(mx[j], lds_mx[j * 256 + threadIdx.x + f * stride]);
-          if (ASYM) mn[j] = fminf(mn[j], lds_mn[j * 256 + threadIdx.x + f * stride]);
+          mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, 64));
+          if (ASYM) mn[j] = fminf(mn[j], __shfl_xor(mn[j], off, 64));
         }
+      }
+      fstep = 64 / stride;
+    }
+    if (fstep < pl.sub) {
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        lds_mx[j * 256 + threadIdx.x] = mx[j];
+        if (ASYM) lds_mn[j * 256 + threadIdx.x] = mn[j];
+      }
+      __syncthreads();
+      if (l.f == 0) {
+        for (int f = fstep; f < pl.sub; f += fstep)
+#pragma unroll
+          for (int j = 0; j < NV; ++j) {
+            mx[j] = fmaxf(mx[j], lds_mx[j * 256 + threadIdx.x + f * stride]);
+            if (ASYM) mn[j] = fminf(mn[j], lds_mn[j * 256 + threadIdx.x + f * stride]);
+          }
+      }
     }
   }
   if (l.f != 0 || l.q >= pl.Q || l.col >= pl.c8 || (!KEEPC && l.col != 0)) return;
@@ -279,19 +317,32 @@ __global__ __launch_bounds__(256) void quant_tiled_kernel(GenParams p, Plan pl, 
   const int64_t g = (int64_t)l.ko * pl.ko_gs + (int64_t)(live ? l.q : 0) * pl.q_gs + (KEEPC ? (live ? l.col : 0) * 8 : 0);
   float s[NV], r[NV], z[NV];
   bool all_plain = true;
+  if constexpr (KEEPC) {
+    // the lane's eight groups are adjacent and start at a multiple of 8: 16-byte loads (the
+    // workspace and the outputs are 16-byte aligned; checked on the host)
+    auto ld8 = [&](const float *src, float (&dst)[NV]) {
+      const float4 a = reinterpret_cast<const float4 *>(src + g)[0], b = reinterpret_cast<const float4 *>(src + g)[1];
+      dst[0] = a.x; dst[1] = a.y; dst[2] = a.z; dst[3] = a.w; dst[4 % NV] = b.x; dst[5 % NV] = b.y; dst[6 % NV] = b.z; dst[7 % NV] = b.w;
+    };
+    ld8(p.scale, s);
+    ld8(rinv, r);
+    if (p.asym) ld8(p.zp, z);
+    else {
 #pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    s[j] = p.scale[g + j];
-    r[j] = rinv[g + j];
-    z[j] = p.asym ? p.zp[g + j] : 0.f;
-    all_plain = all_plain && plain[g + j] != 0u;
+      for (int j = 0; j < NV; ++j) z[j] = 0.f;
+    }
+    const uint4 pa = reinterpret_cast<const uint4 *>(plain + g)[0], pb = reinterpret_cast<const uint4 *>(plain + g)[1];
+    all_plain = (pa.x & pa.y & pa.z & pa.w & pb.x & pb.y & pb.z & pb.w) != 0u;
+  } else {
+    s[0] = p.scale[g];
+    r[0] = rinv[g];
+    z[0] = p.asym ? p.zp[g] : 0.f;
+    all_plain = plain[g] != 0u;
   }
   const float qmin = (float)p.qmin, qmax = (float)p.qmax;
   const u32 mask = (1u << p.bits) - 1u;
   if (!live) return;   // (only the 2-bit path shuffles, and there c8 is even: partners are live together)
-  for_rows(pl, l, [&](int64_t row) {
-    float v[8];
-    In8<DT>::load(p.x, row * p.c + l.col * 8, v);
+  for_rows<DT>(p, pl, l, [&](int64_t row, const float (&v)[8]) {
     int q[8];
     if (all_plain) {
 #pragma unroll
@@ -435,6 +486,15 @@ bool make_plan(const int64_t *sh, int reduce_mask, int64_t n_groups, Plan &pl) {
   }
   pl.nko = (int)nko; pl.nro = (int)nro; pl.Q = (int)Q; pl.RI = (int)RI;
   pl.lanesQ = (int)(Q < pl.R ? Q : pl.R);
+  if (RI == 1 && nro >= VARQ_GEN_NRO_MIN) {
+    // Groups indexed by the innermost leading dim, many reduced rows each (the reference's default
+    // method in layout BLHc): few row lanes on q -- rows of at least 128 channels per wavefront
+    // segment -- and the others on consecutive reduced rows, which fold inside the workgroup.  More
+    // tiles over q, hence fewer chunks and fewer partials for the finalize kernel to fold.
+    int cap = 1;
+    while (cap * 2 * c <= 128) cap *= 2;
+    if (pl.lanesQ > cap) pl.lanesQ = cap;
+  }
   pl.sub = pl.R / pl.lanesQ;
   pl.tilesQ = (int)((Q + pl.lanesQ - 1) / pl.lanesQ);
   pl.fold_ro = (RI == 1);
@@ -442,7 +502,7 @@ bool make_plan(const int64_t *sh, int reduce_mask, int64_t n_groups, Plan &pl) {
   if (pl.fold_ro) { pl.T = 1; steps = (nro + pl.sub - 1) / pl.sub; }
   else { pl.T = (int)((RI + pl.sub - 1) / pl.sub); steps = nro * pl.T; }
   const int64_t kept_blocks = nko * pl.tilesQ;
-  int64_t Z = (4096 + kept_blocks - 1) / kept_blocks;
+  int64_t Z = (VARQ_GEN_BLOCKS + kept_blocks - 1) / kept_blocks;
   const int64_t zcap = (8ll << 20) / (n_groups > 0 ? n_groups : 1);   // partials stay below 64 MiB
   if (Z > zcap) Z = zcap;
   // ... and below a sixteenth of the input: with few kept blocks (groups indexed by the
@@ -482,19 +542,15 @@ int run_tiled(GenParams &p, const Plan &pl, void *workspace, hipStream_t st) {
   }
   // z-lanes per group in the finalize kernel: enough threads in total, no more lanes than partials
   int ZL = 1;
-  while (ZL < 256 && ZL < pl.Z && ng * ZL < 65536) ZL <<= 1;
+  while (ZL < 256 && ZL < pl.Z && ng * ZL < VARQ_FIN_THREADS) ZL <<= 1;
   dim3 fgrid((unsigned)((ng + 256 / ZL - 1) / (256 / ZL)), nt);
   if (p.asym)
     hipLaunchKernelGGL((finalize_tiled_kernel<true>), fgrid, dim3(256), 0, st, p, pl.Z, ZL, part_max, part_min, rinv, plain);
   else
     hipLaunchKernelGGL((finalize_tiled_kernel<false>), fgrid, dim3(256), 0, st, p, pl.Z, ZL, part_max, part_min, rinv, plain);
-  // phase B has no partials to keep apart: longer chunks amortize the per-thread parameter loads
-  Plan pb = pl;
-  constexpr int min_spc = 16;   // measured on [32,30,680,64] and [2,16,10521,128]: 12..24 steps per thread are best
-  if (pb.steps_per_chunk < min_spc) {
-    pb.steps_per_chunk = min_spc < pb.steps ? min_spc : pb.steps;
-    pb.Z = (pb.steps + pb.steps_per_chunk - 1) / pb.steps_per_chunk;
-  }
+  // phase B walks the same chunks (its per-thread parameters are eight 16-byte loads; chunks of 4 to 8 steps
+  // per thread measured alike, longer ones slower)
+  const Plan &pb = pl;
   dim3 bgrid((unsigned)((int64_t)pb.nko * pb.tilesQ * pb.Z), nt);
   if (p.keepc) hipLaunchKernelGGL((quant_tiled_kernel<DT, true>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
   else hipLaunchKernelGGL((quant_tiled_kernel<DT, false>), bgrid, dim3(256), 0, st, p, pb, rinv, plain);
@@ -575,6 +631,8 @@ int quant_pack_impl(const void *x, const void *x1, int x_dtype, const int64_t *h
   if (workspace_bytes < need)
     return varq_set_error(VARQ_ERR_WORKSPACE, "quant_pack: workspace %zu < %zu bytes", workspace_bytes, need);
   VARQ_CHECK_ARG(rows * s[3] < (1ll << 40), "quant_pack: tensor too large");
+  VARQ_CHECK_ARG((((uintptr_t)workspace | (uintptr_t)scale | (uintptr_t)zp | (uintptr_t)scale1 | (uintptr_t)zp1) & 15) == 0,
+                 "quant_pack: scale, zp and workspace must be 16-byte aligned");
 
   GenParams p;
   p.x = x;
