@@ -35,6 +35,7 @@ struct PrepParams {
   int B, L, H, c, c8, c8_shift;
   int token_start, l2norm, nseg;
   float norm_eps, eps;
+  bool slow_levels;            // eps so small that (max - min) / levels must be a true division
   int64_t rows;                // B*L*H
 };
 
@@ -58,11 +59,80 @@ __device__ __forceinline__ bool plain_divisor(float d) {
   return d > 0x1p-96f && d < 0x1p96f && (f2u(d) & 0x7fffffu) != 0x7fffffu;
 }
 
-// group-wise quantize + pack of one octet held by each of LG adjacent lanes
-template <int BITS, bool ASYM, int LG>
-__device__ __forceinline__ void quant_octet(const float (&v)[8], float eps, float &s_out, float &zp_out, u32 &w0, u32 &w1) {
+// (max - min) / levels as IEEE division rounds it.  The divisor is a constant whose significand
+// is not all ones, so the quotient shortcut applies whenever its residual cannot underflow:
+// range >= 2^-90.  Below that the true quotient is below 2^-91 and any eps >= 2^-80 replaces it;
+// smaller eps values take the division (`slow`, uniform for the launch).
+template <int BITS> __device__ __forceinline__ float range_over_levels(float range, bool slow) {
+  constexpr float kLv = (float)QRange<BITS>::kLevels;
+  // (a range that overflowed to infinity takes the division too; the branch is wave-uniform)
+  if (slow || __builtin_amdgcn_ballot_w64(!(range < 0x1p126f)) != 0) return range / kLv;
+  return exact_div(range, kLv, 1.0f / kLv);
+}
+
+// Scale, reciprocal and the shortcut flag of one group from its max and min.
+template <int BITS, bool ASYM>
+__device__ __forceinline__ void group_scale(float mx, float mn, float eps, bool slow, float &s, float &r, bool &plain) {
+  constexpr float kMax = (float)QRange<BITS>::kMax;
+  s = ASYM ? fmaxf(range_over_levels<BITS>(mx - mn, slow), eps) : fmaxf(mx / kMax, eps);
+  r = 1.0f / s;
+  plain = plain_divisor(s);
+}
+// ... and its zero-point (wave_plain: every lane of the wavefront may take the shortcut)
+template <int BITS, bool ASYM>
+__device__ __forceinline__ float group_zp(float mn, float s, float r, bool wave_plain) {
+  if (!ASYM) return 0.f;
+  return (float)QRange<BITS>::kMin - rintf(wave_plain ? exact_div(mn, s, r) : mn / s);
+}
+
+// codes of one octet from the group's parameters, packed.
+// fast (wave-uniform: every lane may take the quotient shortcut and no zero-point exceeds 2^22):
+// clamp(rint(t) + zp, qmin, qmax) = rint(clamp(t, qmin - zp, qmax - zp)) + zp since the bounds
+// are integers; adding 1.5 * 2^23 rounds the clamped quotient to nearest-even and leaves the
+// integer in the low mantissa bits, and the zero-point is added to all fields of the finished
+// word at once, modulo the field width (the sum is known to fit the field).
+template <int BITS, bool ASYM>
+__device__ __forceinline__ void pack_octet(const float (&v)[8], float s, float r, float zp, bool fast, u32 &w0, u32 &w1) {
   constexpr float kMin = (float)QRange<BITS>::kMin, kMax = (float)QRange<BITS>::kMax;
-  float mx, mn = 0.f;
+  u32 acc = 0;
+  w0 = 0; w1 = 0;
+  if (fast) {
+    const float lo = kMin - zp, hi = kMax - zp;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const u32 q = f2u(__builtin_amdgcn_fmed3f(exact_div(v[j], s, r), lo, hi) + 12582912.f);
+      acc = __builtin_amdgcn_alignbit(q, acc, BITS);
+      if (BITS == 8 && j == 3) { w0 = acc; acc = 0; }
+    }
+    if (BITS == 8) w1 = acc;
+    else if (BITS == 4) w0 = acc;
+    else w0 = acc >> 16;
+    if (ASYM) {
+      constexpr u32 kFieldHi = BITS == 8 ? 0x80808080u : BITS == 4 ? 0x88888888u : 0xaaaaaaaau;
+      constexpr u32 kFieldLsb = BITS == 8 ? 0x01010101u : BITS == 4 ? 0x11111111u : 0x55555555u;
+      const u32 zrep = ((u32)(int)zp & ((1u << BITS) - 1u)) * kFieldLsb;
+      const u32 zlo = zrep & ~kFieldHi, zhi = zrep & kFieldHi;
+      w0 = ((w0 & ~kFieldHi) + zlo) ^ (w0 & kFieldHi) ^ zhi;
+      if (BITS == 8) w1 = ((w1 & ~kFieldHi) + zlo) ^ (w1 & kFieldHi) ^ zhi;
+      if (BITS == 2) w0 &= 0xffffu;
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float n = rintf(v[j] / s);
+    const int q = (int)__builtin_amdgcn_fmed3f(ASYM ? n + zp : n, kMin, kMax);
+    acc = __builtin_amdgcn_alignbit((u32)q, acc, BITS);
+    if (BITS == 8 && j == 3) { w0 = acc; acc = 0; }
+  }
+  if (BITS == 8) w1 = acc;
+  else if (BITS == 4) w0 = acc;
+  else w0 = acc >> 16;
+}
+
+template <bool ASYM, int LG>
+__device__ __forceinline__ void octet_minmax(const float (&v)[8], float &mx, float &mn) {
+  mn = 0.f;
   if (ASYM) {
     mx = v[0]; mn = v[0];
 #pragma unroll
@@ -75,58 +145,36 @@ __device__ __forceinline__ void quant_octet(const float (&v)[8], float eps, floa
     for (int j = 0; j < 8; ++j) mx = fmaxf(mx, fabsf(v[j]));
     mx = group_allreduce<LG, true>(mx);
   }
-  const float s = ASYM ? fmaxf((mx - mn) / (float)QRange<BITS>::kLevels, eps) : fmaxf(mx / kMax, eps);
-  const float r = 1.0f / s;
-  const bool plain = plain_divisor(s);
-  // the shortcut or the division for the whole wavefront: no per-element branches
-  const bool wave_plain = __builtin_amdgcn_ballot_w64(!plain) == 0;
-  const float zp = ASYM ? kMin - rintf(wave_plain ? exact_div(mn, s, r) : mn / s) : 0.f;
-  float t[8];
-  if (wave_plain) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) t[j] = exact_div(v[j], s, r);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) t[j] = v[j] / s;
-  }
-  u32 acc = 0;
-  w0 = 0; w1 = 0;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float n = rintf(t[j]);
-    const int q = (int)__builtin_amdgcn_fmed3f(ASYM ? n + zp : n, kMin, kMax);
-    acc = __builtin_amdgcn_alignbit((u32)q, acc, BITS);
-    if (BITS == 8 && j == 3) { w0 = acc; acc = 0; }
-  }
-  if (BITS == 8) w1 = acc;
-  else if (BITS == 4) w0 = acc;
-  else w0 = acc >> 16;
-  s_out = s; zp_out = zp;
 }
+
+// the other lane of an aligned lane pair
+__device__ __forceinline__ float pair_swap(float v) { return dpp_f<0xB1>(v); }
 
 // One lane = 8 channels of one (b, l, h); LR = c/8 lanes form the row, LG = group/8 a group.
 template <int DT, int BITS, bool ASYM, int LR, int LG>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
-  // Lanes walk the (b, h, l) order of the outputs, so the prepared q, the packed words and
-  // the scales of a wavefront are contiguous; the reads are whole 16*LR-byte rows either way.
-  const u32 o = blockIdx.x * 256u + threadIdx.x;      // < 2^31 (checked on the host)
-  const u32 r = o / LR;
-  const int col = (int)(o - r * LR);
-  const bool live = r < (u32)p.rows;
-  const u32 rc = live ? r : (u32)p.rows - 1u;         // idle lanes recompute the last row, never store
-  const int l = (int)(rc % (u32)p.L);
-  const u32 bh = rc / (u32)p.L;
-  const int h = (int)(bh % (u32)p.H);
-  const int b = (int)(bh / (u32)p.H);
+  // grid = (tiles of 256/LR tokens, B*H): lanes walk the (b, h, l) order of the outputs, so the
+  // prepared q, the packed words and the scales of a wavefront are contiguous; the reads are
+  // whole 16*LR-byte rows either way.  (b, h) is uniform for the workgroup: no vector divisions.
+  const int bh = blockIdx.y;
+  const int h = bh % p.H, b = bh / p.H;
+  const int o = blockIdx.x * 256 + threadIdx.x;
+  const int lt = o / LR;                              // (LR is a power of two)
+  const int col = o - lt * LR;
+  const bool live = lt < p.L;
+  const int l = live ? lt : p.L - 1;                  // idle lanes recompute the last token, never store
   const int c = p.c;
-  const int64_t bl = (int64_t)b * p.L + l;
-  const int64_t base = (bl * 3) * (int64_t)p.H * c + (int64_t)h * c + col * 8;
-  const int64_t tstride = (int64_t)p.H * c;
+  // element offsets: the (b, h) part is uniform for the workgroup, the lane's part fits 32 bits
+  // (L * 3 * H * c < 2^31, checked on the host)
+  const int64_t base_bh = ((int64_t)b * p.L * 3) * (int64_t)p.H * c + (int64_t)h * c;
+  const int tstride = p.H * c;
+  const int lane_off = l * 3 * tstride + col * 8;
+  const bool odd = col & 1;
 
   float q[8], k[8], v[8];
-  In8<DT>::load(p.qkv, base, q);
-  In8<DT>::load(p.qkv, base + tstride, k);
-  In8<DT>::load(p.qkv, base + 2 * tstride, v);
+  In8<DT>::load(p.qkv, base_bh + lane_off, q);
+  In8<DT>::load(p.qkv, base_bh + lane_off + tstride, k);
+  In8<DT>::load(p.qkv, base_bh + lane_off + 2 * tstride, v);
 
   if (p.l2norm) {
     float sq = q[0] * q[0], sk = k[0] * k[0];
@@ -134,11 +182,17 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     for (int j = 1; j < 8; ++j) { sq = sq + q[j] * q[j]; sk = sk + k[j] * k[j]; }
     sq = group_allsum<LR>(sq);
     sk = group_allsum<LR>(sk);
-    const float dq = fmaxf(__builtin_sqrtf(sq), p.norm_eps), dk = fmaxf(__builtin_sqrtf(sk), p.norm_eps);
-    const float rq = 1.0f / dq, rk = 1.0f / dk;
-    const bool pq = plain_divisor(dq), pk = plain_divisor(dk);
+    // the two norms of a row are two jobs of one instruction stream: even lanes take q's, odd
+    // lanes k's (square root, clamp, reciprocal, shortcut test), then the lanes of a pair swap
+    const float ssum = odd ? sk : sq;
+    const float dmine = fmaxf(__builtin_sqrtf(ssum), p.norm_eps);
+    const float rmine = 1.0f / dmine;
+    const bool pmine = plain_divisor(dmine);
+    const float dother = pair_swap(dmine), rother = pair_swap(rmine);
+    const float dq = odd ? dother : dmine, dk = odd ? dmine : dother;
+    const float rq = odd ? rother : rmine, rk = odd ? rmine : rother;
     const float mul = p.scale_mul ? p.scale_mul[h] : 1.f;
-    if (__builtin_amdgcn_ballot_w64(!(pq && pk)) == 0) {
+    if (__builtin_amdgcn_ballot_w64(!pmine) == 0) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) { q[j] = exact_div(q[j], dq, rq); k[j] = exact_div(k[j], dk, rk); }
     } else {
@@ -151,7 +205,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     }
   }
   if (p.cos) {
-    const int64_t t = (int64_t)(p.token_start + l) * (c / 2) + col * 4;
+    const int t = (p.token_start + l) * (c / 2) + col * 4;     // (fits 32 bits: checked on the host)
     const float4 cs = *reinterpret_cast<const float4 *>(p.cos + t);
     const float4 sn = *reinterpret_cast<const float4 *>(p.sin + t);
     const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
@@ -165,10 +219,36 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     }
   }
 
-  float ks, kz, vs, vz;
+  // group-wise quantizer of k and v
+  float kmx, kmn, vmx, vmn;
+  octet_minmax<ASYM, LG>(k, kmx, kmn);
+  octet_minmax<ASYM, LG>(v, vmx, vmn);
+  float ks, kr, kz, vs, vr, vz;
+  bool wave_plain;   // the shortcut or the division for the whole wavefront: no per-element branches
+  if constexpr (LG >= 2) {
+    // a lane pair lies inside one group: the even lane derives k's parameters, the odd lane v's,
+    // in one instruction stream, and the pair swaps
+    float s, r;
+    bool pl;
+    const float mn = odd ? vmn : kmn;
+    group_scale<BITS, ASYM>(odd ? vmx : kmx, mn, p.eps, p.slow_levels, s, r, pl);
+    wave_plain = __builtin_amdgcn_ballot_w64(!pl) == 0;
+    const float z = group_zp<BITS, ASYM>(mn, s, r, wave_plain);
+    const float so = pair_swap(s), ro = pair_swap(r), zo = pair_swap(z);
+    ks = odd ? so : s; kr = odd ? ro : r; kz = odd ? zo : z;
+    vs = odd ? s : so; vr = odd ? r : ro; vz = odd ? z : zo;
+  } else {
+    bool kplain, vplain;
+    group_scale<BITS, ASYM>(kmx, kmn, p.eps, p.slow_levels, ks, kr, kplain);
+    group_scale<BITS, ASYM>(vmx, vmn, p.eps, p.slow_levels, vs, vr, vplain);
+    wave_plain = __builtin_amdgcn_ballot_w64(!(kplain && vplain)) == 0;
+    kz = group_zp<BITS, ASYM>(kmn, ks, kr, wave_plain);
+    vz = group_zp<BITS, ASYM>(vmn, vs, vr, wave_plain);
+  }
   u32 kw0, kw1, vw0, vw1;
-  quant_octet<BITS, ASYM, LG>(k, p.eps, ks, kz, kw0, kw1);
-  quant_octet<BITS, ASYM, LG>(v, p.eps, vs, vz, vw0, vw1);
+  const bool fast = wave_plain && __builtin_amdgcn_ballot_w64(!(fabsf(kz) <= 0x1p22f && fabsf(vz) <= 0x1p22f)) == 0;
+  pack_octet<BITS, ASYM>(k, ks, kr, kz, fast, kw0, kw1);
+  pack_octet<BITS, ASYM>(v, vs, vr, vz, fast, vw0, vw1);
 
   // cache row of (b, l, h)
   int64_t s0 = b, s1 = l, s2 = h;
@@ -185,12 +265,17 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     kw0 |= ko << 16; vw0 |= vo << 16;
   }
   if (live) {
-    __bf16 *qo = reinterpret_cast<__bf16 *>(p.q_out) + (((int64_t)b * p.H + h) * p.L + l) * c + col * 8;
-    uint16_t hq[8];
+    __bf16 *qo = reinterpret_cast<__bf16 *>(p.q_out) + (int64_t)bh * p.L * c + (l * c + col * 8);
+    // hardware round-to-nearest-even conversion, two values per instruction
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    u32 w[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) hq[j] = f32_to_bf16_rne(q[j]);
-    *reinterpret_cast<uint4 *>(qo) = make_uint4(hq[0] | ((u32)hq[1] << 16), hq[2] | ((u32)hq[3] << 16),
-                                                hq[4] | ((u32)hq[5] << 16), hq[6] | ((u32)hq[7] << 16));
+    for (int j = 0; j < 4; ++j) {
+      const f2 t = {q[2 * j], q[2 * j + 1]};
+      w[j] = __builtin_bit_cast(u32, __builtin_convertvector(t, bf2));
+    }
+    *reinterpret_cast<uint4 *>(qo) = make_uint4(w[0], w[1], w[2], w[3]);
   }
   if (!stored) return;
   if (BITS == 8) {
@@ -264,7 +349,8 @@ extern "C" int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int 
   VARQ_CHECK_ARG(qkv && q_out && k_words && v_words && k_scale && v_scale && (!asym || (k_zp && v_zp)) && host_rowmap,
                  "qkv_prepare: null pointer");
   VARQ_CHECK_ARG(((uintptr_t)qkv & 15) == 0 && ((uintptr_t)q_out & 15) == 0, "qkv_prepare: qkv and q_out must be 16-byte aligned");
-  VARQ_CHECK_ARG(rows * (c / 8) < (1ll << 31) - 256, "qkv_prepare: tensor too large");
+  VARQ_CHECK_ARG(rows * (c / 8) < (1ll << 31) - 256 && (int64_t)L * 3 * H * c < (1ll << 31) &&
+                     ((int64_t)token_start + L) * (c / 2) < (1ll << 31), "qkv_prepare: tensor too large");
 
   PrepParams p;
   p.qkv = qkv; p.scale_mul = q_scale_mul; p.cos = rope_cos; p.sin = rope_sin; p.q_out = q_out;
@@ -276,9 +362,10 @@ extern "C" int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int 
   p.B = B; p.L = L; p.H = H; p.c = c; p.c8 = c / 8; p.c8_shift = 0;
   p.token_start = token_start; p.l2norm = l2norm ? 1 : 0; p.nseg = c / group;
   p.norm_eps = norm_eps; p.eps = eps; p.rows = rows;
-  const int64_t blocks = (rows * p.c8 + 255) / 256;
-  VARQ_CHECK_ARG(blocks < (1ll << 31), "qkv_prepare: too many blocks");
-  dim3 grid((unsigned)blocks);
+  p.slow_levels = !(eps >= 0x1p-80f);
+  const int64_t tiles = ((int64_t)L * p.c8 + 255) / 256;
+  VARQ_CHECK_ARG(tiles < (1ll << 31) && (int64_t)B * H <= 65535, "qkv_prepare: B*H must not exceed 65535");
+  dim3 grid((unsigned)tiles, (unsigned)(B * H));
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (x_dtype == VARQ_F32) rc = launch_dt<VARQ_F32>(p, bits, asym, p.c8, group / 8, grid, st);
