@@ -262,11 +262,13 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 }
 
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
-// (CHAN: per-channel tables have no per-key K parameters, hence no rank-1 operands)
+// (CHAN: per-channel tables have no per-key K parameters, hence no rank-1 operands; kDeq: more than
+// one K or V group per key -- those kernels dequantize when a tile is widened, see the kernel)
 template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
+  static constexpr bool kDeq = !CHAN && (D / GK > 1 || D / GV > 1);
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
-  static constexpr bool kFoldSv = (D / GV == 1);   // one V group: its scale rides inside the logits
+  static constexpr bool kFoldSv = !kDeq && (D / GV == 1);   // one V group: its scale rides inside the logits
   static constexpr int kParFloats = ((D / GK) + (kFoldSv ? 1 : 2) * (D / GV)) * 64;
   static constexpr int RSR = 64 + 8;        // stride (bf16) of the rows feeding the extra PV MFMA
   static constexpr int KXS = D + 8;         // stride (bf16) of a widened K row: 16-byte rows, bank spread
@@ -274,7 +276,7 @@ template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
   static constexpr int kVp = kKx + 2 * 64 * KXS * 2;
   static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
   static constexpr int kKz = kVt + 2 * D * (64 + 8) * 2;          // rank-1 operands of S^T, 2 x 16 bytes per key and group
-  static constexpr int kWz = kKz + (CHAN ? 0 : 3 * (D / GK) * 64 * 32);   // 8 rows per slot for the extra PV MFMA
+  static constexpr int kWz = kKz + ((CHAN || kDeq) ? 0 : 3 * (D / GK) * 64 * 32);   // 8 rows per slot for the extra PV MFMA
   static constexpr int kPar = kWz + 3 * 8 * RSR * 2;
   static constexpr int kFlag = kPar + 3 * kParFloats * 4;
   static constexpr int kBytes = kFlag + 16;
@@ -300,6 +302,15 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
+  // DEQ: several K or V groups per key.  Carrying exact codes through the MFMAs would need one
+  // logit accumulator and one rank-1 MFMA per K group and one set of weights and one extra MFMA
+  // per V group (19 -> 28 MFMAs per key block at four groups, and registers that do not exist).
+  // These kernels dequantize instead when a tile is widened -- (code - zp) * scale in fp32,
+  // rounded to bf16, the very values the reference's attention sees after its dequantize and
+  // downcast (VAR_Q/quant.py:216-224, VAR/models/basic_var.py:158) -- and then run like a plain
+  // bf16 flash attention: one accumulator, one set of weights, whatever the group count.
+  constexpr bool DEQ = AttnLds<D, BITS, GK, GV, CHAN>::kDeq;
+  constexpr int NSKA = DEQ ? 1 : NSK, NSVA = DEQ ? 1 : NSV;   // accumulators / weight sets
   static_assert(NW >= NSK && NW >= NSV && NW >= 2, "one wavefront per K group and per V group stages the parameters");
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
@@ -338,6 +349,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   constexpr bool FOLD_SV = L::kFoldSv;
   constexpr int RSR = L::RSR;
   constexpr int P_CK = 0, P_VR = NSK * BN, P_SV = P_VR + NSV * BN;
+  constexpr int P_VZ = P_VR;   // DEQ: per (V group, key) the zero-point image; P_SV holds the scale image
 
   // XCD-aware decode: consecutive workgroup ids go to different XCDs (8 of
   // them), so ids congruent mod 8 share an L2.  All query tiles of one
@@ -479,7 +491,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
     if constexpr (CHAN) qbias = -p.scale_log2e * (zb + __shfl_xor(zb, 32, 64) + KCodec<BITS>::kOff * qsum[0]);
 #pragma unroll
-    for (int s = 0; s < (CHAN ? 0 : NSK); ++s) {
+    for (int s = 0; s < ((CHAN || DEQ) ? 0 : NSK); ++s) {
       u32 b0, b1, b2;
       split3_bf16(qsum[s], b0, b1, b2);
       if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
@@ -579,9 +591,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int j = 0; j < 16; ++j) racc[j] = 0.f;
   float m_ref = 0.f;                 // softmax reference (log2 domain)
-  float r_run[NSV];                  // sum_l p' * vzp_r, only fed on tiles with a remainder
+  float r_run[NSVA];                 // sum_l p' * vzp_r, only fed on tiles with a remainder
 #pragma unroll
-  for (int s = 0; s < NSV; ++s) r_run[s] = 0.f;
+  for (int s = 0; s < NSVA; ++s) r_run[s] = 0.f;
 
   const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
   const int64_t kv_ts = p.kv_ts;
@@ -592,6 +604,11 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   constexpr int LPT = (QUADS + NT - 1) / NT;          // pieces per thread
   u32x4_t kreg[LPT], vreg[LPT];
   float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
+  // DEQ: scale and zero-point of the K groups that the thread's 16-byte pieces hold (a piece is
+  // 128 / BITS channels of one key: one group, or two for 2-bit codes in groups of 32)
+  constexpr int CPP = 128 / BITS;                       // channels per piece
+  constexpr int GPP = (DEQ && CPP > GK) ? CPP / GK : 1; // groups per piece
+  float kgs[DEQ ? LPT * GPP : 1], kgz[DEQ ? LPT * GPP : 1];
 
   auto prefetch_k = [&](int) {   // the next tile of the K stream
     const int t0 = cur_k.start;
@@ -602,6 +619,15 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
         kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + key * kv_ts * WPR + (piece % (WPR / 4)) * 4);
+        if constexpr (DEQ) {
+          const int g0 = (piece % (WPR / 4)) * CPP / GK;   // first group of the piece
+#pragma unroll
+          for (int j = 0; j < GPP; ++j) {
+            const int64_t g = (kv_row0 + key * kv_ts) * NSK + g0 + j;
+            kgs[i * GPP + j] = p.k_scale[g];
+            kgz[i * GPP + j] = p.k_zp ? p.k_zp[g] : 0.f;
+          }
+        }
       }
     }
   };
@@ -623,7 +649,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       ksc = 1.f; kzp = 0.f; vsc = 1.f; vzp = 0.f; ksc0 = 1.f;   // unit per-key parameters
     } else {
       const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = NW - 1 - seg;
-      if (seg < NSK) {
+      if (!DEQ && seg < NSK) {
         const int64_t g = (kv_row0 + key * kv_ts) * NSK + seg;
         ksc = p.k_scale[g];
         kzp = p.k_zp ? p.k_zp[g] : 0.f;
@@ -661,7 +687,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     };
     // keys of the merged run carry values, not code images: no image factor, no offset terms
     const bool merged = merged_tile(tile);
-    if (!CHAN && seg < NSK) {   // (per-channel tables: one factor for all keys, no rank-1 term)
+    if (!CHAN && !DEQ && seg < NSK) {   // (per-channel tables: one factor for all keys, no rank-1 term)
       par[P_CK + seg * BN + key] = merged ? p.scale_log2e : ck_of(ksc);
       u32 a0, a1, a2;
       split3_bf16(merged ? 0.f : -(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
@@ -669,7 +695,14 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       dst[0] = u32x4_t{a0 | (a0 << 16), a0 | (a1 << 16), a1 | (a1 << 16), a2 | (a2 << 16)};
       if (!(FOLD_SV && seg == 0)) dst[1] = u32x4_t{0u, 0u, 0u, 0u};
     }
-    if (vseg < NSV) {
+    if (DEQ) {
+      // (code - zp) * vs = (raw - (zp + kOff) / kMul) * (kMul * vs) for the code image `raw` the
+      // widening step produces; both factors are exact rescalings by powers of two
+      if (vseg < NSV) {
+        par[P_VZ + vseg * BN + key] = (vzp + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+        par[P_SV + vseg * BN + key] = vsc * VCodec<BITS>::kMul;
+      }
+    } else if (vseg < NSV) {
       const int seg = vseg;
       if (FOLD_SV && !CHAN) {
         u32 l0, l1, l2;
@@ -699,9 +732,11 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   asm volatile("" : "+v"(kmask));   // keep the mask in a vector register (see KCodec::expand)
 
   // row of the extra PV block this lane feeds in the MFMA of V group s (as element offset)
-  int rowsel[NSV];
+  int rowsel[NSVA];
 #pragma unroll
-  for (int s = 0; s < NSV; ++s) rowsel[s] = ((col == s) ? s : (s == 0 && col >= 4 && col < 7) ? col : 7) * RSR;
+  for (int s = 0; s < NSVA; ++s) rowsel[s] = ((col == s) ? s : (s == 0 && col >= 4 && col < 7) ? col : 7) * RSR;
+  // DEQ: row 0 of the extra block is a row of ones (the softmax denominator), the others zero
+  const u32 ones_a = (DEQ && col == 0) ? 0x3f803f80u : 0u;
 
   // packed V of `tile` -> V^T bf16: a work item is 2 adjacent keys x 8 channels (one
   // packed word of each key), written as 8 dwords of the transposed tile
@@ -732,6 +767,14 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         }
       } else {
         VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
+        if constexpr (DEQ) {
+          // code images -> values of the two keys, (raw - z') * s' in fp32, rounded to bf16
+          const float *pt = lds_par + (tile % 3) * L::kParFloats + (oct * 8 / GV) * BN + kp2 * 2;
+          const float2 z2 = *reinterpret_cast<const float2 *>(pt + P_VZ), s2 = *reinterpret_cast<const float2 *>(pt + P_SV);
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            pr[j] = pack_bf16_rne((u2f(pr[j] << 16) - z2.x) * s2.x, (u2f(pr[j] & 0xffff0000u) - z2.y) * s2.y);
+        }
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * VTS + kp2 * 2]) = pr[j];
@@ -777,6 +820,15 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         for (int j = 0; j < OPQ; ++j) {
           u32 a[4];
           KCodec<BITS>::expand(q4, j, kmask, a);
+          if constexpr (DEQ) {
+            // code images -> values: (raw - (zp + kOff) / kMul) * (kMul * ks), the reference's
+            // (code - zp) * scale with both factors rescaled exactly, rounded to bf16
+            const int gl = (j * 8) / GK < GPP ? (j * 8) / GK : GPP - 1;   // group of octet j inside the piece
+            const float zk = (kgz[i * GPP + gl] + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul);
+            const float sk = kgs[i * GPP + gl] * KCodec<BITS>::kMul;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((u2f(a[m] << 16) - zk) * sk, (u2f(a[m] & 0xffff0000u) - zk) * sk);
+          }
           *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
         }
       }
@@ -888,17 +940,17 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // ---- the three phases of one 32-key block, as lambdas over per-tile state --------
   // LDS operands are requested ahead of their use where the registers allow it (the
   // scheduling fences keep the requests where they are written).
-  constexpr bool HOIST = (NSK == 1 && NSV == 1);
+  constexpr bool HOIST = (NSKA == 1 && NSVA == 1);
   int t0 = 0;
   const uint16_t *kx = nullptr, *vt = nullptr, *wz = nullptr;
   const float *par = nullptr;
   const u32x4_t *kz = nullptr;
   bool tile_rem = false, first = true;
   // register i of this lane <-> key kb*32 + 16*(i/8) + 8*half + i%8 of the tile
-  floatx16_t sacc[2][NSK];
-  u32 pop[2][NSV][2][4];          // P'^T operands: p * vs as bf16, [block][V group][16-key chunk][dword]
-  float ckv[2][NSK][16], svv[2][NSV][16];
-  u32x4_t vta[NDB], wza[NSV];
+  floatx16_t sacc[2][NSKA];
+  u32 pop[2][NSVA][2][4];          // P'^T operands: p * vs as bf16, [block][V group][16-key chunk][dword]
+  float ckv[2][NSKA][16], svv[2][NSVA][16];
+  u32x4_t vta[NDB], wza[NSVA];
 
   // per-channel tables: segment of the tile being attended, end of the tile's keys, and the
   // softmax denominator as it was when the current segment began
@@ -987,7 +1039,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   };
   auto load_scales = [&](int kb) {
 #pragma unroll
-    for (int s = 0; s < ((HOIST && !CHAN) ? NSK : 0); ++s)
+    for (int s = 0; s < ((HOIST && !CHAN && !DEQ) ? NSK : 0); ++s)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
@@ -995,7 +1047,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         ckv[kb][s][4 * i4] = t.x; ckv[kb][s][4 * i4 + 1] = t.y; ckv[kb][s][4 * i4 + 2] = t.z; ckv[kb][s][4 * i4 + 3] = t.w;
       }
 #pragma unroll
-    for (int s = 0; s < ((HOIST && !FOLD_SV) ? NSV : 0); ++s)
+    for (int s = 0; s < ((HOIST && !FOLD_SV && !DEQ) ? NSV : 0); ++s)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
@@ -1008,8 +1060,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int d = 0; d < NDB; ++d)
       vta[d] = *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * VTS + (kb * 2 + c) * 16 + half * 8]);
 #pragma unroll
-    for (int s = 0; s < NSV; ++s)
+    for (int s = 0; s < (DEQ ? 0 : NSV); ++s)
       wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
+    if constexpr (DEQ) wza[0] = u32x4_t{ones_a, ones_a, ones_a, ones_a};
   };
 
   // S^T = K Q^T for one 32-key block; the A operands are the widened K rows in LDS
@@ -1017,11 +1070,13 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     __builtin_amdgcn_s_setprio(1);
     const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
-    for (int s = 0; s < NSK; ++s) {
+    for (int s = 0; s < NSKA; ++s) {
       floatx16_t zero;
 #pragma unroll
       for (int j = 0; j < 16; ++j) zero[j] = 0.f;
-      if constexpr (CHAN) {
+      if constexpr (DEQ) {
+        sacc[kb][s] = zero;   // (dequantized operands: no zero-point term)
+      } else if constexpr (CHAN) {
         // The key side of the rank-1 term is a constant here and lives in qbias.  In its place:
         // the remainder pass of the chunk with the largest outlier scale -- that chunk's K operand
         // against q_lo.  Issued whether or not the segment has such a chunk (q_lo is zero then,
@@ -1043,8 +1098,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
       const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[k_octet<GK>(ch, half) * 8]);
-      sacc[kb][ch / (GK / 16)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-          __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][ch / (GK / 16)], 0, 0, 0);
+      constexpr int kAcc = DEQ ? 0 : 1;
+      sacc[kb][kAcc * (ch / (GK / 16))] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][kAcc * (ch / (GK / 16))], 0, 0, 0);
     }
     if constexpr (CHAN) {
       // further remainder passes: more than one chunk with an outlier scale
@@ -1074,9 +1130,10 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int i = 0; i < 16; ++i) {
       float v = CHAN ? (in_merged ? 0.f : qbias) - m_ref : -m_ref;
 #pragma unroll
-      for (int s = 0; s < NSK; ++s) {
+      for (int s = 0; s < NSKA; ++s) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        v = __builtin_fmaf(CHAN ? ck_all : HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key], sacc[kb][s][i], v);
+        v = __builtin_fmaf(DEQ ? p.scale_log2e : CHAN ? ck_all : HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key],
+                           sacc[kb][s][i], v);
       }
       z[i] = v;
     }
@@ -1114,7 +1171,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) racc[j] *= alpha;
 #pragma unroll
-      for (int s = 0; s < NSV; ++s) r_run[s] *= alpha;
+      for (int s = 0; s < NSVA; ++s) r_run[s] *= alpha;
       if constexpr (CHAN) l_prev *= alpha;
     }
     first = false;
@@ -1122,22 +1179,22 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
 #pragma unroll
-    for (int s = 0; s < NSV; ++s)
+    for (int s = 0; s < NSVA; ++s)
 #pragma unroll
       for (int i2 = 0; i2 < 8; ++i2) {
         const int i = 2 * i2;
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        if constexpr (FOLD_SV) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
+        if constexpr (FOLD_SV || DEQ) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
         else if constexpr (HOIST)
           pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[kb][s][i], pv[i + 1] * svv[kb][s][i + 1]);
         else
           pop[kb][s][i >> 3][(i & 7) >> 1] =
               pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
       }
-    if (tile_rem) {
+    if (!DEQ && tile_rem) {
       // the remainder term must see the same bf16-rounded weights as the MFMA
 #pragma unroll
-      for (int s = 0; s < NSV; ++s)
+      for (int s = 0; s < NSVA; ++s)
 #pragma unroll
         for (int i2 = 0; i2 < 8; ++i2) {
           const int i = 2 * i2;
@@ -1156,12 +1213,12 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-      u32x4_t av[NDB], aw[NSV];
+      u32x4_t av[NDB], aw[NSVA];
       if (!(preloaded && c == 0) && !(HOIST && c == 1)) load_v_operands(kb, c);
 #pragma unroll
       for (int d = 0; d < NDB; ++d) av[d] = vta[d];
 #pragma unroll
-      for (int s = 0; s < NSV; ++s) aw[s] = wza[s];
+      for (int s = 0; s < NSVA; ++s) aw[s] = wza[s];
       if (HOIST && c == 0) {
         load_v_operands(kb, 1);   // in flight under this chunk's MFMAs
         __builtin_amdgcn_sched_barrier(0);
@@ -1169,13 +1226,13 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
       for (int d = 0; d < NDB; ++d) {
         constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
-        const int s = d / DBS;
+        const int s = DEQ ? 0 : d / DBS;
         u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
         oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[d]),
                                                           __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
       }
 #pragma unroll
-      for (int s = 0; s < NSV; ++s) {
+      for (int s = 0; s < NSVA; ++s) {
         u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
         racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
                                                        __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
@@ -1207,13 +1264,14 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   // ---- epilogue -------------------------------------------------------------------
 #pragma unroll
-  for (int s = 0; s < NSV; ++s) r_run[s] += __shfl_xor(r_run[s], 32, 64);
+  for (int s = 0; s < NSVA; ++s) r_run[s] += __shfl_xor(r_run[s], 32, 64);
   // rows 4..6 of racc are registers 0..2 of the upper lane half, rows 0..3 registers 0..3 of the lower
-  const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
+  // (DEQ: the denominator is row 0, the sum of the weights against the row of ones)
+  const float l_sum = DEQ ? __shfl(racc[0], col, 64) : __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
   const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
-  float rq[NSV];
+  float rq[NSVA];
 #pragma unroll
-  for (int s = 0; s < NSV; ++s) rq[s] = __shfl(racc[s], col, 64) + r_run[s];
+  for (int s = 0; s < NSVA; ++s) rq[s] = DEQ ? 0.f : __shfl(racc[s], col, 64) + r_run[s];
   if (q_live) {
     __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D;
     // with the keys shared out: the normalized fp32 output and (reference, denominator) of
@@ -1225,8 +1283,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 #pragma unroll
     for (int d = 0; d < NDB; ++d) {
       constexpr int DBS = GV / 32;
-      const float r = rq[d / DBS];
-      constexpr float VM = VCodec<BITS>::kMul;
+      const float r = rq[DEQ ? 0 : d / DBS];
+      constexpr float VM = DEQ ? 1.f : VCodec<BITS>::kMul;   // (DEQ: the accumulators hold values already)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
