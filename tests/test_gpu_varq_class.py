@@ -228,3 +228,19 @@ def test_reserve_tokens_keeps_the_buffers_in_place(dev):
     assert len(ptrs) == 1 and a._c_item.buf.shape[2] < 1000
     assert torch.equal(a.cached_item, b.cached_item) and torch.equal(a.cached_scale, b.cached_scale)
     assert a.cached_item.shape[2] == total
+
+
+def test_layout_change_with_cached_steps_is_refused(dev):
+    """qkv_format may be re-assigned before the first step (Infinity's attention assigns it every
+    forward, basic.py:309,314); with steps cached in the other layout the next step raises instead
+    of continuing on a truncated cache."""
+    note('VAR_Q layout change')
+    q = VAR_Q(8, 'BLHc', 'G_SCALE_HEAD_DIM')
+    q.qkv_format = 'BHLc'
+    x = torch.randn(2, 3, 4, 64, device=dev)
+    assert q.use_var_q(x).shape == x.shape
+    q.qkv_format = 'BHLc'                                   # the same layout again: nothing happens
+    assert q.use_var_q(x).shape == (2, 3, 8, 64)
+    q.qkv_format = 'BLHc'
+    with pytest.raises(ValueError, match='qkv_format was changed'):
+        q.use_var_q(x)

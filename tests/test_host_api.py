@@ -35,7 +35,7 @@ def test_constructor_contract_matches_reference():
 def test_qkv_format_assignment_rederives_layout():
     q = VAR_Q(8, 'BLHc')
     q.qkv_format = 'BHLc'                      # what Infinity's attention does every forward
-    assert q.dim_cat == 2 and q.dim_map['G_SCALE_HEAD_DIM'] == (0, 2)
+    assert q.dim_cat == 2 and q.dim_map == VAR_Q(8, 'BHLc').dim_map
 
 
 def test_cpu_tensors_are_refused():
@@ -46,6 +46,12 @@ def test_cpu_tensors_are_refused():
         PU.pack_last_dim_to_int32_triton(torch.zeros(2, 8, dtype=torch.int8), 4)
     with pytest.raises(AssertionError):
         PU.unpack_last_dim_from_int32_triton(torch.zeros(2, 1, dtype=torch.int32),
+                                             {'orig_c': 8, 'vals_per_word': 8, 'pad_len': 0, 'bits': 4})
+    # the reference's _python pair takes CPU tensors; this drop-in says why it does not
+    with pytest.raises(VarqError, match='no CPU fallback'):
+        PU.pack_last_dim_to_int32_python(torch.zeros(2, 8, dtype=torch.int8), 4)
+    with pytest.raises(VarqError, match='no CPU fallback'):
+        PU.unpack_last_dim_from_int32_python(torch.zeros(2, 1, dtype=torch.int32),
                                              {'orig_c': 8, 'vals_per_word': 8, 'pad_len': 0, 'bits': 4})
 
 

@@ -366,7 +366,13 @@ class VAR_Q:
         s_cur = self._expand_scale_like_L(q_cur, self.scale)
         z_cur = None if self.zp is None else self._expand_scale_like_L(q_cur, self.zp)
         if m in ('G_SCALE_HEAD_DIM', 'G_SCALE', 'G_TOKEN', 'G_TOKEN_HEAD', 'G_TENSOR', 'G_GROUP', 'G_HEAD'):
-            if self._c_item.dim != self.dim_cat:   # layout was re-assigned before the first step
+            if self._c_item.dim != self.dim_cat:
+                # the layout was re-assigned: fine before the first step, an error once steps are
+                # cached (their tokens lie along the other dim; dropping them silently would leave
+                # the generation running on a truncated cache)
+                if self._c_item.len > 0:
+                    raise ValueError('VAR_Q: qkv_format was changed to %s with %d tokens cached in the other layout'
+                                     % (self.qkv_format, self._c_item.len))
                 self._reset_cache()
             st, self._staged = self._staged, None
             if st is not None and st[0] is self._c_item.buf and st[1] == self._c_item.len and st[2] is q_cur:
