@@ -5,22 +5,23 @@ same dequantized operands.
 
 How the tolerance is applied, and why.  Two kinds of kernels are tested here.
 
-The kernels for more than one scale group per key (group 64 or 32 at head dim 128, group
-32 at head dim 64) dequantize K and V to bf16 when a tile enters LDS, which is what the
+The kernels that dequantize -- more than one scale group per key (group 64 or 32 at head
+dim 128, group 32 at head dim 64) and the per-(head, channel) tables of the reference's
+shipped rule -- turn K and V into bf16 values when a tile enters LDS, which is what the
 reference's attention sees; they meet the literal bar: max|out - oracle| <= 2e-2 in units
-of the output range, usually one bf16 step.
+of the output range.  The per-channel-table tests ask for half of that
+(`oracle_bar=1e-2`): the arithmetic in front of the softmax is the reference's own.
 
-The single-group kernels (and the per-channel-table kernels) multiply the integer codes
-exactly and apply scales/zero-points in fp32; the oracle first rounds the dequantized K
-and V to bf16 (as the reference's attention backends do).  On unit-range data the two
-agree to well inside 2e-2.  On the heavy-tailed Infinity-2B benchmark data
-(configuration 4) (outputs up to ~95, where one bf16 ulp is 0.5) the oracle's operand
-rounding alone moves ITS output by up to ~4 from the fp64 value, while the kernel stays
-within ~0.3 of it.  So a result passes when
+The single-group token kernels multiply the integer codes exactly and apply scales and
+zero-points in fp32; the oracle first rounds the dequantized K and V to bf16 (as the
+reference's attention backends do).  On unit-range data the two agree to well inside 2e-2.
+On the heavy-tailed Infinity-2B benchmark data (configuration 4) (outputs up to ~95, where
+one bf16 ulp is 0.5) the oracle's operand rounding alone moves ITS output by up to ~4 from
+the fp64 value, while the kernel stays within ~0.3 of it.  So a result passes when
     cosine(out, oracle) >= 0.9995                                    (always)
 and either
-    max|out - oracle| <= 2e-2 * max(1, max|oracle|)                  (the literal bar)
-or
+    max|out - oracle| <= oracle_bar * max(1, max|oracle|)            (the literal bar, or tighter)
+or (only where oracle_bar is the general 2e-2)
     max|out - fp64|   <= 2e-2 * max(1, max|fp64|)                    (range units)
     max|out - oracle| <= 2e-2 * max(1, max|oracle|) + max|oracle - fp64|
 i.e. the kernel is within tolerance of the true value, and no further from the oracle
@@ -51,7 +52,7 @@ def _exact_fp64(q, kd, vd, scale, bias, dev):
                              None if bias is None else bias.to(dev)).cpu()
 
 
-def _compare(out, ref, exact, what='', fp64_bar=2e-2):
+def _compare(out, ref, exact, what='', oracle_bar=2e-2):
     out, ref = out.double().cpu(), ref.double()
     span = max(1.0, float(ref.abs().max()))
     err = float((out - ref).abs().max())
@@ -61,9 +62,10 @@ def _compare(out, ref, exact, what='', fp64_bar=2e-2):
           f'oracle-fp64 {e_ref:.4g}  cosine {cos:.6f}', flush=True)
     assert not bool(torch.isnan(out).any())
     assert cos >= 0.9995, f'{what}: cosine {cos}'
-    if fp64_bar >= 2e-2 and err <= 2e-2 * span:
-        return            # the literal bar: within 2e-2 (range units) of the reference path
-    assert e_out <= fp64_bar * span, f'{what}: kernel is {e_out} from the fp64 value (range {span}, bar {fp64_bar})'
+    if err <= oracle_bar * span:
+        return            # the literal bar (or a tighter one): within range units of the reference path
+    assert oracle_bar >= 2e-2, f'{what}: max-abs {err} vs oracle, bar {oracle_bar} x range {span}'
+    assert e_out <= 2e-2 * span, f'{what}: kernel is {e_out} from the fp64 value (range {span})'
     assert err <= 2e-2 * span + e_ref, f'{what}: max-abs {err} vs oracle (oracle itself {e_ref} from fp64, range {span})'
 
 

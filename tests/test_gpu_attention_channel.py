@@ -2,16 +2,14 @@
 reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
 (G_TENSOR), and the affine per-head-per-dim variant of benchmark configuration 3 --
 against the oracle path quantize -> dequant -> bf16 SDPA and an fp64 evaluation of the same
-formula.  Tolerances as in test_gpu_attention.py (max-abs 2e-2 in range units, cosine >=
-0.9995), with a tighter bar on the distance from the fp64 value: 1.25e-2 of the range, on
-the data of the benchmark configurations (outlier channels x15) throughout.  The kernel
-scales the queries by the K table and rounds them to bf16 once per segment; chunks of
-channels with an outlier scale carry the rounding remainder through a second MFMA, which
-is what keeps that distance at 0.2-0.5 % (bf16 output rounding alone is up to 0.4 %); the
-first steps of a D=64 schedule that share one key tile are converted to the units of the
-step behind them and rounded to bf16 as the oracle rounds the whole cache, and stay at
-the oracle's own distance (up to 1.2 %).  The codes handed to the kernel are the oracle's
-own, so the comparison isolates the attention."""
+formula, on the data of the benchmark configurations (outlier channels x15) throughout.
+The kernel dequantizes K and V with the tables of each key's segment when a tile is widened
+-- (code - zp) * scale in fp32, rounded to bf16, the oracle's own operands -- so the bar here
+is half the general one: max|out - oracle| <= 1e-2 in units of the output range (cosine >=
+0.9995 as everywhere); what is left is the bf16 rounding of the weights and of the output
+(one bf16 step of an output near the top of the range is 0.4e-2 to 0.8e-2 of it).  The distance of both from the fp64 value is printed beside it (up to ~2 % of
+the range on this data, the same for kernel and oracle).  The codes handed to the kernel are
+the oracle's own, so the comparison isolates the attention."""
 import math
 
 import pytest
@@ -24,7 +22,7 @@ from var_q_amd import ops, schedules
 
 pytestmark = pytest.mark.gpu
 
-FP64_BAR = 1.25e-2   # kernel vs fp64, in units of the output range (the general bar is 2e-2)
+ORACLE_BAR = 1e-2   # kernel vs oracle, in units of the output range: half the general bar (one bf16 step of the output is up to 0.8e-2)
 
 
 def _quantize_channel(x, bits, asym, dims=(0, 2)):
@@ -36,7 +34,8 @@ def _quantize_channel(x, bits, asym, dims=(0, 2)):
     return O.pack_last_dim(q, bits)[0], table(s), table(z), deq
 
 
-def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist='normal', dims=(0, 2), what='', splits=0):
+def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist='normal', dims=(0, 2), what='', splits=0,
+         drop_k_zp=False):
     g = torch.Generator().manual_seed(seed)
     k = O.synth_kv((B, H, Lk, D), seed + 1, dist).bfloat16()
     v = O.synth_kv((B, H, Lk, D), seed + 2, dist).bfloat16()
@@ -45,20 +44,26 @@ def _run(dev, B, H, Lq, Lk, D, bits, asym, seed, kv_limit=None, bias=None, dist=
     vw, vs, vz, vd = _quantize_channel(v, bits, asym, dims)
     scale = 1.0 / math.sqrt(D)
     note('fused_attn_channel', what, (B, H, Lq, Lk, D), bits, asym, 'splits', splits)
-    # one table: the zero-point of K cancels, so it is passed in one case of two only
-    kz_arg = None if (kz is None or seed % 2) else kz.to(dev)
+    # one table: the zero-point of K shifts all logits of a query alike and may be left out; the
+    # dequantized K is then offset per channel and rounds differently from the oracle's
+    kz_arg = None if (kz is None or drop_k_zp) else kz.to(dev)
     out = ops.fused_attn_channel(q.to(dev), kw.to(dev), ks.to(dev), kz_arg, vw.to(dev), vs.to(dev),
                                  None if vz is None else vz.to(dev), bits, Lk, scale,
                                  kv_limit=None if kv_limit is None else kv_limit.to(dev), splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, kd, vd, scale, bias)
-    _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what, fp64_bar=FP64_BAR)
+    _compare(out, ref, _exact_fp64(q, kd, vd, scale, bias, dev), what, oracle_bar=2e-2 if drop_k_zp else ORACLE_BAR)
 
 
 @pytest.mark.parametrize('D', [64, 128])
 @pytest.mark.parametrize('bits,asym', [(8, False), (4, False), (2, True), (4, True), (8, True)])
 def test_small_all_visible(dev, D, bits, asym):
     _run(dev, 2, 3, 200, 333, D, bits, asym, seed=bits * 10 + D + asym, what='channel small')
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+def test_k_zero_point_left_out(dev, bits):
+    _run(dev, 2, 3, 200, 333, 64, bits, True, seed=bits * 10 + 5, what='channel, no K zero-point', drop_k_zp=True)
 
 
 @pytest.mark.parametrize('Lq,Lk', [(1, 1), (4, 5), (33, 64), (129, 127), (7, 300)])
@@ -161,7 +166,7 @@ def _stepwise(dev, B, H, D, steps, bits, asym, Lq, seed, masked=False, what='', 
                                  kv_limit=None if lim is None else lim.to(dev), seg_ends=ends, splits=splits)
     torch.cuda.synchronize()
     ref = O.attention_ref(q, deq[0], deq[1], scale, bias)
-    _compare(out, ref, _exact_fp64(q, deq[0], deq[1], scale, bias, dev), what, fp64_bar=FP64_BAR)
+    _compare(out, ref, _exact_fp64(q, deq[0], deq[1], scale, bias, dev), what, oracle_bar=ORACLE_BAR)
 
 
 VAR_STEPS = [n * n for n in O.VAR_PATCH_NUMS]

@@ -65,9 +65,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
 
 constexpr int kMaxSegments = 16;
-constexpr int kChanTableRows = 5;   // LDS rows per segment of the per-channel tables
-constexpr int kMaxLoAny = 4;        // most remainder passes per key block (per-channel tables)
-constexpr float kLoRatio = 3.f;      // a chunk gets one when its largest K scale is this many times the head's mean
+constexpr int kChanTableRows = 4;   // LDS rows per segment of the per-channel tables
 
 struct AttnParams {
   const __bf16 *q;
@@ -81,11 +79,6 @@ struct AttnParams {
   // (fp32 [nseg, Hkv, D]); this is a cache that was quantized step by step
   int nseg;
   int seg_end[kMaxSegments];
-  // The first nconv segments (tiny first steps of a schedule, together at most one key tile)
-  // are attended in the units of segment nconv: their codes are turned into values relative
-  // to that segment's tables when the tile is widened (rounded to bf16, as the reference rounds
-  // the dequantized cache), so they share key tiles and cost no change of tables.
-  int nconv;
   const int32_t *head_map;
   const int32_t *kv_limit;
   int B, Hq, Hkv, Lq, Lk, Lstride;
@@ -162,6 +155,27 @@ template <> struct VCodec<8> {
     }
   }
 };
+// The kernels that dequantize want the images as fp32 numbers: f0[j], f1[j] = raw of channel j of
+// the octet in the two rows.  Bytes are converted once; the narrower fields come out of `pairs`.
+template <int BITS>
+__device__ __forceinline__ void v_pair_values(const u32 *row0, const u32 *row1, int oct, u32 M, float (&f0)[8], float (&f1)[8]) {
+  if constexpr (BITS == 8) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int w0 = (int)row0[2 * oct + h], w1 = (int)row1[2 * oct + h];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f0[4 * h + j] = (float)(int)__builtin_amdgcn_sbfe(w0, 8 * j, 8);
+        f1[4 * h + j] = (float)(int)__builtin_amdgcn_sbfe(w1, 8 * j, 8);
+      }
+    }
+  } else {
+    u32 pr[8];
+    VCodec<BITS>::pairs(row0, row1, oct, M, pr);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { f0[j] = __builtin_bit_cast(float, pr[j] << 16); f1[j] = __builtin_bit_cast(float, pr[j] & 0xffff0000u); }
+  }
+}
 
 __device__ __forceinline__ u32 pack_bf16_rne(float lo, float hi) {
   typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
@@ -253,6 +267,23 @@ template <> struct KCodec<8> {
   }
 };
 
+// The kernels that dequantize want the images as fp32 numbers, in the operand's slot order.
+template <int BITS> __device__ __forceinline__ void k_values(const u32 *q4, int oct, u32 M, float (&f)[8]) {
+  if constexpr (BITS == 8) {
+    const u32 w0 = q4[2 * oct], w1 = q4[2 * oct + 1];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[j] = (float)(int)__builtin_amdgcn_sbfe((int)w0, 8 * j, 8);
+      f[4 + j] = (float)(int)__builtin_amdgcn_sbfe((int)w1, 8 * j, 8);
+    }
+  } else {
+    u32 a[4];
+    KCodec<BITS>::expand(q4, oct, M, a);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) { f[2 * m] = __builtin_bit_cast(float, a[m] << 16); f[2 * m + 1] = __builtin_bit_cast(float, a[m] & 0xffff0000u); }
+  }
+}
+
 // octet (8-channel unit) of K that lane-half h contracts in 16-channel chunk ch;
 // chunks never straddle a scale group of `G` channels.
 template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
@@ -262,10 +293,10 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 }
 
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
-// (CHAN: per-channel tables have no per-key K parameters, hence no rank-1 operands; kDeq: more than
-// one K or V group per key -- those kernels dequantize when a tile is widened, see the kernel)
+// (kDeq: per-channel tables, or more than one K or V group per key -- those kernels dequantize when
+// a tile is widened, see the kernel, and have no rank-1 operands)
 template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
-  static constexpr bool kDeq = !CHAN && (D / GK > 1 || D / GV > 1);
+  static constexpr bool kDeq = CHAN || (D / GK > 1 || D / GV > 1);
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
   static constexpr bool kFoldSv = !kDeq && (D / GV == 1);   // one V group: its scale rides inside the logits
@@ -276,29 +307,24 @@ template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
   static constexpr int kVp = kKx + 2 * 64 * KXS * 2;
   static constexpr int kVt = (kVp + 3 * 64 * RSV * 4 + 15) / 16 * 16;
   static constexpr int kKz = kVt + 2 * D * (64 + 8) * 2;          // rank-1 operands of S^T, 2 x 16 bytes per key and group
-  static constexpr int kWz = kKz + ((CHAN || kDeq) ? 0 : 3 * (D / GK) * 64 * 32);   // 8 rows per slot for the extra PV MFMA
+  static constexpr int kWz = kKz + (kDeq ? 0 : 3 * (D / GK) * 64 * 32);   // 8 rows per slot for the extra PV MFMA
   static constexpr int kPar = kWz + 3 * 8 * RSR * 2;
   static constexpr int kFlag = kPar + 3 * kParFloats * 4;
   static constexpr int kBytes = kFlag + 16;
 };
 
-// CHAN: scales and zero-points per (head, channel) instead of per (key, channel group).
-// Then K[l,d] = sk[d] * (code[l,d] - zk[d]) and q.K[l] = sum_d (q[d] sk[d]) code[l,d] minus
-// a term that does not depend on the key, which the softmax cancels: the kernel attends
-// the raw codes with q scaled per channel.  With one table that term can be left out; when
-// the tables change along the keys it differs from segment to segment and is added to the
-// logits as a per-query constant of the segment.
-// Likewise out[d] = sv[d] * (sum_l p[l] code[l,d] - zv[d]) because the weights sum to one:
-// V runs with unit scale and the affine map is applied to the normalized output.
-// When the tables change along the keys (segments), key tiles never straddle a segment:
-// at a boundary the Q operands are rebuilt with the new K table and the output
-// accumulators are re-expressed in units of the new V table.
-// SEGS: the tables change along the keys (more than one segment).  A single table needs none
-// of what makes boundaries cheap (kept query registers, merged first steps), and is compiled
-// without it.
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8, bool SEGS = false>
-__global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
-  static_assert(CHAN || !SEGS, "segments belong to the per-channel tables");
+// CHAN: scales and zero-points per (head, channel) instead of per (key, channel group), in up
+// to 16 tables that change along the keys (a cache quantized step by step has one per step).
+// Such a kernel dequantizes when a tile is widened, like the kernels for several groups per key
+// (DEQ below): K[l,d] = (code[l,d] - zk_s[d]) * sk_s[d] with s the segment of key l, rounded to
+// bf16 -- what the reference's attention sees -- and likewise V.  The tables of the head sit in
+// LDS; a tile inside one segment reads that segment's rows, a tile that straddles segments
+// looks the segment up per key.  Everything behind the widening is a plain bf16 flash attention
+// that knows nothing of tables or segments.
+// WPS: wavefronts per SIMD the register allocation aims at (2, or 4: two 8-wavefront workgroups
+// per compute unit at 128 registers, which the D=64 kernels that dequantize afford)
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8, int WPS = 2>
+__global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p) {
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
@@ -335,15 +361,13 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   uint16_t *const lds_wz = reinterpret_cast<uint16_t *>(lds_raw + L::kWz);
   float *const lds_par = reinterpret_cast<float *>(lds_raw + L::kPar);    // [3][L::kParFloats]
   int *const lds_flag = reinterpret_cast<int *>(lds_raw + L::kFlag);      // [3] tile+1 if that tile has a zero-point remainder
-  // CHAN: the tables of this head for every segment, [nseg][5][D] fp32: K scale, K zero-point,
-  // V scale, V zero-point (zeros where a table is absent) and the ratio of the V scales of the
-  // previous segment and this one; filled once in the prologue
+  // CHAN: the tables of this head for every segment, [nseg][4][D] fp32, filled once in the
+  // prologue, as the widening steps use them: row 0 = kMul * sk and row 1 = (zk + kOff) / kMul in
+  // the slot order of the K operand octets, row 2 = kMul * sv and row 3 = (zv + kOff) / kMul by
+  // channel ((code - z) * s = (raw - z') * s' for the code image raw = (code + kOff) / kMul, both
+  // rescalings exact)
   float *const lds_tab = reinterpret_cast<float *>(lds_raw + (L::kBytes + 15) / 16 * 16);
-  // per segment two words: remainder slot + 1 of 16-channel contraction chunk ch in bits 4ch..4ch+2
-  // (0 = none); chunk of slot s in bits 4s..4s+2 and the number of slots in use from bit 16
-  u32 *const lds_clo = reinterpret_cast<u32 *>(lds_tab + kMaxSegments * kChanTableRows * D);
-  constexpr int TR = kChanTableRows;   // rows per segment: K scale, K zero-point, V scale, V zero-point, sv(seg-1)/sv(seg)
-  const bool k_affine = CHAN && p.k_chan_zp != nullptr, v_affine = CHAN && p.v_chan_zp != nullptr;   // (uniform)
+  constexpr int TR = kChanTableRows;
   constexpr int KXS = L::KXS, RSV = L::RSV;
   // parameter block of one tile: ck [NSK][BN]; vr [NSV][BN]; sv [NSV][BN] unless folded
   constexpr bool FOLD_SV = L::kFoldSv;
@@ -380,10 +404,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // Q^T operands, gathered in the slot order of the K codec
   u32x4_t qb[NCH];
   u32x4_t bq[NSK];
-  // per-channel tables at D=64: the query values as loaded stay in registers (16 of them), so
-  // that a segment boundary rebuilds the operands without going back to memory
-  constexpr bool KEEP_Q = SEGS && D == 64;
-  u32x4_t qraw[KEEP_Q ? NCH : 1];
   // The K zero-point term -(kzp+kOff)/kMul * sum(q) is a rank-1 update of S^T and
   // rides on one more MFMA per key block and group.  Both factors are split into
   // three bf16 pieces (a0+a1+a2, b0+b1+b2, exact) and the 9 products are laid on
@@ -392,106 +412,29 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // the term, is dropped).  With a single V group, slots 0..2 of the upper half add
   // log2(vs)/ck (three pieces against 1.0), which makes exp2(logit) come out as
   // p * vs without a multiplication; the other upper slots are zero.
-  // CHAN: per-query constant of the current segment's logits,
-  // -softmax_scale*log2(e) * (sum_d q'[d] zk[d] + kOff * sum_d q'[d]): the K zero-points and the
-  // offset of the code images (the token-mode kernels carry both on the rank-1 MFMA, whose key
-  // side is the same for every key here)
-  float qbias = 0.f;
-  // CHAN: q[d] * sk[d] is rounded to bf16 for the MFMA, the same rounding for every key of the
-  // segment, so its error does not average out over the keys the way the reference's rounding
-  // of the dequantized K does: on a channel whose scale is far above the others (an outlier
-  // channel) it tilts the softmax.  The 16-channel chunks whose largest scale is at least
-  // kLoRatio times the head's mean scale -- up to kMaxLo of them, the largest first -- get a
-  // second MFMA per key block with the rounding remainders as the Q operand (hi + lo carries 16
-  // significant bits) and the same A operand, the chunk's widened K.
-  // (D=64: four chunks in all, and registers are scarcer where the tables change along the keys)
-    constexpr int kMaxLo = D == 64 ? 2 : kMaxLoAny;
-  u32x4_t qlo[CHAN ? kMaxLo : 1];
-  // chunk of slot s in bits 4s..4s+2 (slots fill from 0), slots in use in bits 16..18 (wave-uniform)
-  u32 lo_info = 0u;
-  // (called from two places: force the inlining, or its captures would live in memory)
-  // (pre: the raw values were requested into qb earlier -- the prologue does, to overlap the
-  // trip with its other loads)
-  auto load_q = [&](int seg, auto pre) __attribute__((always_inline)) {
-    float qsum[NSK], zb = 0.f;
+  // (the raw values were requested into qb earlier -- the prologue does, to overlap the trip
+  // with its other loads)
+  auto load_q = [&]() {
+    float qsum[NSK];
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] = 0.f;
-    int slot_of[CHAN ? NCH : 1];   // remainder slot of chunk ch, or -1 (wave-uniform)
-    if constexpr (CHAN) {
-      // the segment's chunks with a remainder pass, chosen in the prologue
-      // (one 8-byte read: slot + 1 of chunk ch in bits 4ch..4ch+2 of the first word)
-      const uint2 info = *reinterpret_cast<const uint2 *>(&lds_clo[seg * 2]);
-      const u32 slots = __builtin_amdgcn_readfirstlane(info.x);
-      lo_info = __builtin_amdgcn_readfirstlane(info.y);
-#pragma unroll
-      for (int ch = 0; ch < NCH; ++ch) slot_of[ch] = (int)((slots >> (4 * ch)) & 7u) - 1;
-      qlo[0] = u32x4_t{0u, 0u, 0u, 0u};   // (slot 0 is multiplied whether in use or not)
-    }
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
-      const int oct = k_octet<GK>(ch, half);
-      // the octet's eight channels in one 16-byte load, then into the codec's slot order
-      u32x4_t raw;
-      if constexpr (KEEP_Q) raw = qraw[ch];
-      else raw = decltype(pre)::value ? qb[ch] : *reinterpret_cast<const u32x4_t *>(qptr + oct * 8);
-      float sk[8];
-      u32x4_t lo4 = {0u, 0u, 0u, 0u};
-      const bool with_lo = CHAN && slot_of[CHAN ? ch : 0] >= 0;   // (wave-uniform)
-      if constexpr (CHAN) {
-        const float *tk = lds_tab + (seg * TR + 0) * D + oct * 8;
-        const float4 s0 = *reinterpret_cast<const float4 *>(tk), s1 = *reinterpret_cast<const float4 *>(tk + 4);
-        sk[0] = s0.x; sk[1] = s0.y; sk[2] = s0.z; sk[3] = s0.w; sk[4] = s1.x; sk[5] = s1.y; sk[6] = s1.z; sk[7] = s1.w;
-      }
+      // the octet's eight channels, loaded in one 16-byte piece, into the codec's slot order
+      const u32x4_t raw = qb[ch];
 #pragma unroll
       for (int j2 = 0; j2 < 4; ++j2) {
         // operand slots 2*j2 and 2*j2+1, one dword
         const int d0 = KCodec<BITS>::slot_d(2 * j2), d1 = KCodec<BITS>::slot_d(2 * j2 + 1);   // channels within the octet
         const u32 lo = (raw[d0 >> 1] >> (16 * (d0 & 1))) << 16, hi = (raw[d1 >> 1] >> (16 * (d1 & 1))) << 16;
-        u32 pair = (lo >> 16) | hi;
-        if constexpr (CHAN) {
-          // q[d] * sk[d], rounded to bf16 like any MFMA operand; what the rounding left behind
-          // (exact in fp32, then rounded to bf16 itself) is the operand of the remainder pass
-          const float f0 = u2f(lo) * sk[d0], f1 = u2f(hi) * sk[d1];
-          pair = pack_bf16_rne(f0, f1);
-          if (with_lo) lo4[j2] = pack_bf16_rne(f0 - u2f(pair << 16), f1 - u2f(pair & 0xffff0000u));
-        }
-        qb[ch][j2] = pair;
-        qsum[ch / (GK / 16)] += u2f(pair << 16) + u2f(pair & 0xffff0000u);
+        qb[ch][j2] = (lo >> 16) | hi;
+        qsum[ch / (GK / 16)] += u2f(lo) + u2f(hi);
       }
-      if constexpr (CHAN) {
-        if (with_lo) {
-#pragma unroll
-          for (int sl = 0; sl < kMaxLo; ++sl)
-            if (slot_of[ch] == sl) qlo[sl] = lo4;
-#pragma unroll
-          for (int j2 = 0; j2 < 4; ++j2) qsum[0] += u2f(lo4[j2] << 16) + u2f(lo4[j2] & 0xffff0000u);
-        }
-      }
-      if (k_affine) {   // the K zero-points against the rounded operands, for the segment's logit constant
-        const float *tz = lds_tab + (seg * TR + 1) * D + oct * 8;
-        const float4 z0 = *reinterpret_cast<const float4 *>(tz), z1 = *reinterpret_cast<const float4 *>(tz + 4);
-        const float zk[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
-#pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) {
-          const u32 pair = qb[ch][j2];
-          zb = __builtin_fmaf(u2f(pair << 16), zk[KCodec<BITS>::slot_d(2 * j2)], zb);
-          zb = __builtin_fmaf(u2f(pair & 0xffff0000u), zk[KCodec<BITS>::slot_d(2 * j2 + 1)], zb);
-        }
-        if (with_lo) {
-#pragma unroll
-          for (int j2 = 0; j2 < 4; ++j2) {
-            zb = __builtin_fmaf(u2f(lo4[j2] << 16), zk[KCodec<BITS>::slot_d(2 * j2)], zb);
-            zb = __builtin_fmaf(u2f(lo4[j2] & 0xffff0000u), zk[KCodec<BITS>::slot_d(2 * j2 + 1)], zb);
-          }
-        }
-      }
-      if constexpr (CHAN) __builtin_amdgcn_sched_barrier(0);   // one chunk's table entries in registers at a time
     }
 #pragma unroll
     for (int s = 0; s < NSK; ++s) qsum[s] += __shfl_xor(qsum[s], 32, 64);
-    if constexpr (CHAN) qbias = -p.scale_log2e * (zb + __shfl_xor(zb, 32, 64) + KCodec<BITS>::kOff * qsum[0]);
 #pragma unroll
-    for (int s = 0; s < ((CHAN || DEQ) ? 0 : NSK); ++s) {
+    for (int s = 0; s < (DEQ ? 0 : NSK); ++s) {
       u32 b0, b1, b2;
       split3_bf16(qsum[s], b0, b1, b2);
       if (half == 0) bq[s] = u32x4_t{b0 | (b1 << 16), b2 | (b0 << 16), b1 | (b2 << 16), b0 | (b1 << 16)};
@@ -511,72 +454,31 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   }
   int n_tiles = (kv_end + BN - 1) / BN;
   // segment ends in LDS: indexing the kernel arguments with a run-time index would move
-  // the whole argument block to scratch memory
+  // the whole argument block to scratch memory (literal indices only, for the same reason)
   __shared__ int lds_seg_end[kMaxSegments];
   if constexpr (CHAN) {
-    // key tiles never straddle a segment of the tables: count them segment by segment
-    // (literal indices only: a loop index would be a run-time index at the time the
-    // argument block is split into registers)
-    n_tiles = 0;
-    int beg = 0;
-#define VARQ_SEG(S)                                                                            \
-  {                                                                                            \
-    const int e = p.seg_end[S];                                                                \
-    if (tid == 0) lds_seg_end[S] = e;                                                          \
-    if (S + 1 >= p.nconv) { /* (a merged segment is counted with the last one of its run) */   \
-      if (S < p.nseg && beg < kv_end) n_tiles += (min(e, kv_end) - beg + BN - 1) / BN;         \
-      beg = e;                                                                                 \
-    }                                                                                          \
-  }
-    VARQ_SEG(0) VARQ_SEG(1) VARQ_SEG(2) VARQ_SEG(3) VARQ_SEG(4) VARQ_SEG(5) VARQ_SEG(6) VARQ_SEG(7)
-    VARQ_SEG(8) VARQ_SEG(9) VARQ_SEG(10) VARQ_SEG(11) VARQ_SEG(12) VARQ_SEG(13) VARQ_SEG(14) VARQ_SEG(15)
+    if (p.nseg > 1 && tid == 0) {
+#define VARQ_SEG(S) lds_seg_end[S] = p.seg_end[S];
+      VARQ_SEG(0) VARQ_SEG(1) VARQ_SEG(2) VARQ_SEG(3) VARQ_SEG(4) VARQ_SEG(5) VARQ_SEG(6) VARQ_SEG(7)
+      VARQ_SEG(8) VARQ_SEG(9) VARQ_SEG(10) VARQ_SEG(11) VARQ_SEG(12) VARQ_SEG(13) VARQ_SEG(14) VARQ_SEG(15)
 #undef VARQ_SEG
-    static_assert(kMaxSegments == 16, "the list above names every segment");
-    __syncthreads();
-  }
-  // Position of a stream of consecutive tiles (the K prefetch, the V prefetch and the
-  // attention itself each walk the tiles in order).  Without segments tile t starts at
-  // key t * BN; with segments a tile ends where its segment ends.
-  struct TileCursor { int seg, start; };
-  auto cursor_advance = [&](TileCursor &c) __attribute__((always_inline)) {
-    if constexpr (CHAN) {
-      c.start += BN;
-      const int e = __builtin_amdgcn_readfirstlane(lds_seg_end[c.seg]);
-      if (c.start >= e && c.seg + 1 < p.nseg) { c.start = e; ++c.seg; }
-    } else {
-      c.start += BN;
+      static_assert(kMaxSegments == 16, "the list above names every segment");
     }
-  };
-  TileCursor cur_k{(CHAN && p.nconv > 0) ? p.nconv - 1 : 0, 0};   // (the merged run walks as one segment)
+    // (read behind the prologue's first barrier)
+  }
   int tbase = 0;   // index of this workgroup's first tile in the block's tile sequence
   if (p.nsplit > 1) {
     // this workgroup's share of the tiles: [t_begin, t_end) of the block's tile sequence
     const int t_begin = n_tiles * split / p.nsplit, t_end = n_tiles * (split + 1) / p.nsplit;
     tbase = t_begin;
-    if constexpr (CHAN) {
-      for (int i = 0; i < t_begin; ++i) cursor_advance(cur_k);
-    } else {
-      cur_k.start = t_begin * BN;
-    }
     n_tiles = t_end - t_begin;
   }
-  TileCursor cur_v = cur_k, cur_a = cur_k;
-  const int tile_base = cur_k.start;   // first key of this workgroup's tiles
-  // tiles of the merged run: the first npre of the sequence, dense from key 0
-  int npre = 0;
-  if constexpr (CHAN) {
-    if (p.nconv > 0) npre = (min(__builtin_amdgcn_readfirstlane(lds_seg_end[p.nconv - 1]), kv_end) + BN - 1) / BN;
-  }
-  // (at D=128 the conversion code costs registers that the main loop has not got: the host
-  // merges nothing there, and the code is left out)
-  constexpr bool MERGE = SEGS && D == 64;
-  auto merged_tile = [&](int tile) { return MERGE && tbase + tile < npre; };
-  // segment (< nconv) of a key of the merged run
-  auto merged_segment = [&](int key) {
-    int sgm = 0;
-    while (sgm + 1 < p.nconv && key >= lds_seg_end[sgm]) ++sgm;
-    return sgm;
-  };
+  const int tile_base = tbase * BN;   // first key of this workgroup's tiles
+  // The K prefetch, the V prefetch and the widening each walk the tiles in order.
+  int pk_tile = 0, pv_tile = 0;
+  // CHAN: segment of the first key of the next tile to be widened, and where that segment ends
+  // (wave-uniform; the tiles are widened in order, K and V of a tile one after the other)
+  int wseg = 0, wseg_end = p.Lk;
   int wave_minlim = q_live ? limit : p.Lk;
   for (int off = 1; off < 64; off <<= 1) wave_minlim = min(wave_minlim, __shfl_xor(wave_minlim, off, 64));
 
@@ -608,18 +510,19 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // 128 / BITS channels of one key: one group, or two for 2-bit codes in groups of 32)
   constexpr int CPP = 128 / BITS;                       // channels per piece
   constexpr int GPP = (DEQ && CPP > GK) ? CPP / GK : 1; // groups per piece
-  float kgs[DEQ ? LPT * GPP : 1], kgz[DEQ ? LPT * GPP : 1];
+  constexpr bool KGP = DEQ && !CHAN;                    // K group parameters travel with the pieces
+  float kgs[KGP ? LPT * GPP : 1], kgz[KGP ? LPT * GPP : 1];
 
   auto prefetch_k = [&](int) {   // the next tile of the K stream
-    const int t0 = cur_k.start;
-    cursor_advance(cur_k);
+    const int t0 = tile_base + pk_tile * BN;
+    ++pk_tile;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
       if (LPT * NT == QUADS || piece < QUADS) {
         const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
         kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + key * kv_ts * WPR + (piece % (WPR / 4)) * 4);
-        if constexpr (DEQ) {
+        if constexpr (KGP) {
           const int g0 = (piece % (WPR / 4)) * CPP / GK;   // first group of the piece
 #pragma unroll
           for (int j = 0; j < GPP; ++j) {
@@ -632,8 +535,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     }
   };
   auto prefetch = [&](int) {   // the next tile of the V stream
-    const int t0 = cur_v.start;
-    cursor_advance(cur_v);
+    const int t0 = tile_base + pv_tile * BN;
+    ++pv_tile;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
@@ -645,9 +548,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     // scales: thread t handles key t % 64; wavefront w takes K group w and V group
     // 3 - w, which puts the K and the V arithmetic of the single-group case on
     // different wavefronts
-    if constexpr (CHAN) {
-      ksc = 1.f; kzp = 0.f; vsc = 1.f; vzp = 0.f; ksc0 = 1.f;   // unit per-key parameters
-    } else {
+    if constexpr (!CHAN) {   // (per-channel tables: no per-key parameters)
       const int key = min(t0 + (tid & 63), p.Lk - 1), seg = tid >> 6, vseg = NW - 1 - seg;
       if (!DEQ && seg < NSK) {
         const int64_t g = (kv_row0 + key * kv_ts) * NSK + seg;
@@ -685,17 +586,17 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       const float c = ks * p.scale_log2e * KCodec<BITS>::kMul;
       return __builtin_fabsf(c) < 1e-30f ? 1e-30f : c;
     };
-    // keys of the merged run carry values, not code images: no image factor, no offset terms
-    const bool merged = merged_tile(tile);
-    if (!CHAN && !DEQ && seg < NSK) {   // (per-channel tables: one factor for all keys, no rank-1 term)
-      par[P_CK + seg * BN + key] = merged ? p.scale_log2e : ck_of(ksc);
+    if (!DEQ && seg < NSK) {
+      par[P_CK + seg * BN + key] = ck_of(ksc);
       u32 a0, a1, a2;
-      split3_bf16(merged ? 0.f : -(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
+      split3_bf16(-(kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), a0, a1, a2);
       u32x4_t *dst = &lds_kz[((sl * NSK + seg) * BN + key) * 2];
       dst[0] = u32x4_t{a0 | (a0 << 16), a0 | (a1 << 16), a1 | (a1 << 16), a2 | (a2 << 16)};
       if (!(FOLD_SV && seg == 0)) dst[1] = u32x4_t{0u, 0u, 0u, 0u};
     }
-    if (DEQ) {
+    if (CHAN) {
+      // (the tables are in LDS already)
+    } else if (DEQ) {
       // (code - zp) * vs = (raw - (zp + kOff) / kMul) * (kMul * vs) for the code image `raw` the
       // widening step produces; both factors are exact rescalings by powers of two
       if (vseg < NSV) {
@@ -704,7 +605,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       }
     } else if (vseg < NSV) {
       const int seg = vseg;
-      if (FOLD_SV && !CHAN) {
+      if (FOLD_SV) {
         u32 l0, l1, l2;
         split3_bf16(__builtin_amdgcn_logf(vsc) * __builtin_amdgcn_rcpf(ck_of(ksc0)), l0, l1, l2);
         lds_kz[(sl * NSK * BN + key) * 2 + 1] = u32x4_t{l0 | (l1 << 16), l2, 0u, 0u};
@@ -716,7 +617,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       if (!FOLD_SV) par[P_SV + seg * BN + key] = vsc;
       par[P_VR + seg * BN + key] = zr;
       uint16_t *rows = lds_wz + sl * 8 * RSR;
-      rows[seg * RSR + key] = merged ? (uint16_t)0 : (uint16_t)(f2u(zc + VCodec<BITS>::kOff) >> 16);
+      rows[seg * RSR + key] = (uint16_t)(f2u(zc + VCodec<BITS>::kOff) >> 16);
       if (seg == 0) {
         u32 i0, i1, i2;
         split3_bf16(__builtin_amdgcn_rcpf(vsc), i0, i1, i2);
@@ -738,43 +639,65 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // DEQ: row 0 of the extra block is a row of ones (the softmax denominator), the others zero
   const u32 ones_a = (DEQ && col == 0) ? 0x3f803f80u : 0u;
 
+  // CHAN: the widening of `tile` begins: (wseg, wseg_end) follow the tile's first key
+  auto widen_cursor = [&](int tile) {
+    if constexpr (CHAN) {
+      const int t0w = tile_base + tile * BN;
+      while (wseg + 1 < p.nseg && t0w >= wseg_end) {
+        ++wseg;
+        wseg_end = __builtin_amdgcn_readfirstlane(lds_seg_end[wseg]);
+      }
+    }
+  };
+  // CHAN: segment of a key of the tile being widened, searched upwards from the tile's first
+  auto key_segment = [&](int key) {
+    int sg = wseg;
+    while (sg + 1 < p.nseg && key >= lds_seg_end[sg]) ++sg;
+    return sg;
+  };
+  // CHAN: all keys of the tile being widened belong to segment wseg (wave-uniform)
+  auto tile_in_one_segment = [&](int tile) { return wseg + 1 >= p.nseg || tile_base + tile * BN + BN <= wseg_end; };
+
   // packed V of `tile` -> V^T bf16: a work item is 2 adjacent keys x 8 channels (one
   // packed word of each key), written as 8 dwords of the transposed tile
-  // (first: the call may meet the tile of the merged run, which is always the first of the
-  // sequence -- only the prologue's calls carry the conversion code, the loop's stay lean)
-  auto widen_v = [&](int tile, auto first) {
+  auto widen_v = [&](int tile) {
     const u32 *vp = lds_vp + (tile % 3) * BN * RSV;
     uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
-    const bool merged = decltype(first)::value && merged_tile(tile);
+    widen_cursor(tile);
+    const bool one_seg = !CHAN || tile_in_one_segment(tile);
     for (int item = tid; item < (BN / 2) * (D / 8); item += NT) {
       const int kp2 = item & (BN / 2 - 1), oct = item / (BN / 2);
       const u32 *row = &vp[kp2 * 2 * RSV];
       u32 pr[8];
-      if (merged) {
-        if constexpr (MERGE && decltype(first)::value) {
-          // values of the two keys in the V units of the base segment: (code - zv) * sv / sv_base,
-          // divided by the image factor that the epilogue multiplies back
-          const int k0 = min((tbase + tile) * BN + 2 * kp2, p.Lk - 1), k1 = min(k0 + 1, p.Lk - 1);
-          const float *tb = lds_tab + (p.nconv * TR + 2) * D + oct * 8;
-          const float *t0s = lds_tab + (merged_segment(k0) * TR + 2) * D + oct * 8, *t1s = lds_tab + (merged_segment(k1) * TR + 2) * D + oct * 8;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int off = (oct * 8 + j) * BITS;
-            const float rb = __builtin_amdgcn_rcpf(tb[j]) * (1.f / VCodec<BITS>::kMul);
-            const float c0 = staged_code<BITS>(row[off >> 5], off & 31), c1 = staged_code<BITS>(row[RSV + (off >> 5)], off & 31);
-            pr[j] = pack_bf16_rne((c0 - t0s[D + j]) * t0s[j] * rb, (c1 - t1s[D + j]) * t1s[j] * rb);
-          }
+      float f0[8], f1[8];
+      if constexpr (DEQ) v_pair_values<BITS>(row, row + RSV, oct, kmask, f0, f1);
+      else VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
+      if constexpr (CHAN) {
+        // code images -> values, (raw - z') * s' per channel in fp32, rounded to bf16
+        int sg0 = wseg, sg1 = wseg;
+        if (!one_seg) {
+          const int k0 = min(tile_base + tile * BN + 2 * kp2, p.Lk - 1);
+          sg0 = key_segment(k0);
+          sg1 = key_segment(min(k0 + 1, p.Lk - 1));
         }
-      } else {
-        VCodec<BITS>::pairs(row, row + RSV, oct, kmask, pr);
-        if constexpr (DEQ) {
-          // code images -> values of the two keys, (raw - z') * s' in fp32, rounded to bf16
-          const float *pt = lds_par + (tile % 3) * L::kParFloats + (oct * 8 / GV) * BN + kp2 * 2;
-          const float2 z2 = *reinterpret_cast<const float2 *>(pt + P_VZ), s2 = *reinterpret_cast<const float2 *>(pt + P_SV);
+        const float *t0s = lds_tab + (sg0 * TR + 2) * D + oct * 8;
+        const float4 sa = *reinterpret_cast<const float4 *>(t0s), sb = *reinterpret_cast<const float4 *>(t0s + 4);
+        const float4 za = *reinterpret_cast<const float4 *>(t0s + D), zb = *reinterpret_cast<const float4 *>(t0s + D + 4);
+        const float s0[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w}, z0[8] = {za.x, za.y, za.z, za.w, zb.x, zb.y, zb.z, zb.w};
+        if (one_seg || sg1 == sg0) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            pr[j] = pack_bf16_rne((u2f(pr[j] << 16) - z2.x) * s2.x, (u2f(pr[j] & 0xffff0000u) - z2.y) * s2.y);
+          for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z0[j]) * s0[j], (f1[j] - z0[j]) * s0[j]);
+        } else {
+          const float *t1s = lds_tab + (sg1 * TR + 2) * D + oct * 8;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z0[j]) * s0[j], (f1[j] - t1s[D + j]) * t1s[j]);
         }
+      } else if constexpr (DEQ) {
+        // code images -> values of the two keys, (raw - z') * s' in fp32, rounded to bf16
+        const float *pt = lds_par + (tile % 3) * L::kParFloats + (oct * 8 / GV) * BN + kp2 * 2;
+        const float2 z2 = *reinterpret_cast<const float2 *>(pt + P_VZ), s2 = *reinterpret_cast<const float2 *>(pt + P_SV);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * VTS + kp2 * 2]) = pr[j];
@@ -783,9 +706,11 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   // packed K of `tile` (in kreg) -> widened bf16 rows: each 16-byte piece holds OPQ octets
   // of one key, every octet becomes one 16-byte MFMA A operand
-  auto widen_k = [&](int tile, auto first) {
+  auto widen_k = [&](int tile) {
     uint16_t *kx = lds_kx + (tile & 1) * BN * KXS;
     constexpr int OPQ = 16 / BITS;            // octets per 16-byte piece
+    widen_cursor(tile);
+    const bool one_seg = !CHAN || tile_in_one_segment(tile);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const int piece = tid + i * NT;
@@ -793,41 +718,34 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         const int key = piece / (WPR / 4), oct0 = (piece % (WPR / 4)) * OPQ;
         constexpr u32 KX = KCodec<BITS>::kStageXor;
         const u32 q4[4] = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
-        if (decltype(first)::value && merged_tile(tile)) {
-          if constexpr (MERGE && decltype(first)::value) {
-            // the key's values in the K units of the base segment, (code - zk) * sk / sk_base, in
-            // the operand's slot order
-            const int kabs = min((tbase + tile) * BN + key, p.Lk - 1);
-            const float *ts = lds_tab + (merged_segment(kabs) * TR + 0) * D, *tb = lds_tab + (p.nconv * TR + 0) * D;
-#pragma unroll
-            for (int j = 0; j < OPQ; ++j) {
-              float val[8];
-#pragma unroll
-              for (int c = 0; c < 8; ++c) {
-                const int off = (j * 8 + c) * BITS, d = (oct0 + j) * 8 + c;
-                val[c] = (staged_code<BITS>(q4[off >> 5], off & 31) - ts[D + d]) * ts[d] * __builtin_amdgcn_rcpf(tb[d]);
-              }
-              u32 a[4];
-#pragma unroll
-              for (int j2 = 0; j2 < 4; ++j2)
-                a[j2] = pack_bf16_rne(val[KCodec<BITS>::slot_d(2 * j2)], val[KCodec<BITS>::slot_d(2 * j2 + 1)]);
-              *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
-            }
-          }
-          continue;
+        int sg = wseg;
+        if constexpr (CHAN) {
+          if (!one_seg) sg = key_segment(min(tile_base + tile * BN + key, p.Lk - 1));
         }
 #pragma unroll
         for (int j = 0; j < OPQ; ++j) {
           u32 a[4];
-          KCodec<BITS>::expand(q4, j, kmask, a);
-          if constexpr (DEQ) {
+          float f[8];
+          if constexpr (DEQ) k_values<BITS>(q4, j, kmask, f);
+          else KCodec<BITS>::expand(q4, j, kmask, a);
+          if constexpr (CHAN) {
+            // code images -> values: (raw - z') * s' per channel (rows 0 and 1 of the segment's
+            // tables, in the operand's slot order), the reference's (code - zp) * scale, rounded to bf16
+            const float *tk = lds_tab + sg * TR * D + (oct0 + j) * 8;
+            const float4 sa = *reinterpret_cast<const float4 *>(tk), sb = *reinterpret_cast<const float4 *>(tk + 4);
+            const float4 za = *reinterpret_cast<const float4 *>(tk + D), zb = *reinterpret_cast<const float4 *>(tk + D + 4);
+            const float sc[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w}, zc[8] = {za.x, za.y, za.z, za.w, zb.x, zb.y, zb.z, zb.w};
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+              a[m] = pack_bf16_rne((f[2 * m] - zc[2 * m]) * sc[2 * m], (f[2 * m + 1] - zc[2 * m + 1]) * sc[2 * m + 1]);
+          } else if constexpr (DEQ) {
             // code images -> values: (raw - (zp + kOff) / kMul) * (kMul * ks), the reference's
             // (code - zp) * scale with both factors rescaled exactly, rounded to bf16
             const int gl = (j * 8) / GK < GPP ? (j * 8) / GK : GPP - 1;   // group of octet j inside the piece
             const float zk = (kgz[i * GPP + gl] + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul);
             const float sk = kgs[i * GPP + gl] * KCodec<BITS>::kMul;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((u2f(a[m] << 16) - zk) * sk, (u2f(a[m] & 0xffff0000u) - zk) * sk);
+            for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((f[2 * m] - zk) * sk, (f[2 * m + 1] - zk) * sk);
           }
           *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
         }
@@ -839,88 +757,36 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   //      of tile 2 in registers ------------------------------------------------------------
   if (tid < 3) lds_flag[tid] = 0;
   for (int i = tid; i < 3 * RSR; i += NT) lds_wz[((i / RSR) * 8 + 7) * RSR + i % RSR] = 0;   // the all-zero row of each slot
-  __syncthreads();
   if (n_tiles > 0) { prefetch_k(0); prefetch(0); }
   // the query values, behind the first tile's requests and ahead of the table loads: one
   // round trip for all three
 #pragma unroll
-  for (int ch = 0; ch < NCH; ++ch) {
-    if constexpr (KEEP_Q) qraw[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
-    else qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
-  }
+  for (int ch = 0; ch < NCH; ++ch) qb[ch] = *reinterpret_cast<const u32x4_t *>(qptr + k_octet<GK>(ch, half) * 8);
   if constexpr (CHAN) {
-    for (int i = tid; i < p.nseg * 4 * D; i += NT) {
-      const int seg = i / (4 * D), which = (i / D) & 3, d = i % D;
+    // the head's tables, as the widening steps use them (see lds_tab above)
+    for (int i = tid; i < p.nseg * TR * D; i += NT) {
+      const int seg = i / (TR * D), which = (i / D) % TR, d = i % D;
+      const bool is_k = which < 2, is_zp = which & 1;
       const float *src = which == 0 ? p.k_chan_scale : which == 1 ? p.k_chan_zp : which == 2 ? p.v_chan_scale : p.v_chan_zp;
-      lds_tab[(seg * TR + which) * D + d] = src ? src[((int64_t)seg * p.Hkv + hs) * D + d] : 0.f;
+      const int c = is_k ? (d & ~7) + KCodec<BITS>::slot_d(d & 7) : d;   // K rows: the operand's slot order inside an octet
+      const float x = src ? src[((int64_t)seg * p.Hkv + hs) * D + c] : 0.f;
+      const float mul = is_k ? KCodec<BITS>::kMul : VCodec<BITS>::kMul, off = is_k ? KCodec<BITS>::kOff : VCodec<BITS>::kOff;
+      lds_tab[i] = is_zp ? (x + off) * (1.f / mul) : x * mul;
     }
-    __syncthreads();
-    // change of V units at the entry of a segment, per channel (the hardware reciprocal is
-    // accurate to an ulp, which is all a change of units needs)
-    for (int i = tid; i < p.nseg * D; i += NT) {
-      const int seg = i / D, d = i % D;
-      lds_tab[(seg * TR + 4) * D + d] =
-          seg ? lds_tab[((seg - 1) * TR + 2) * D + d] * __builtin_amdgcn_rcpf(lds_tab[(seg * TR + 2) * D + d]) : 1.f;
-    }
-    // Chunks that get a remainder pass: largest K scale of the chunk's 16 channels (the two
-    // octets that the lane halves contract together) >= kLoRatio * mean K scale of the head; at
-    // most kMaxLo of them, the largest first.  2*NCH adjacent lanes per segment, one octet each
-    // (the last wavefronts', which have the least of the loop above).
-    {
-      constexpr int GL = 2 * NCH;                      // lanes per segment: (chunk, lane half)
-      const int rt = NT - 1 - tid;                     // (reversed: lane groups stay aligned, NT is a multiple of 64)
-      const int seg = rt / GL, gl = rt % GL;
-      if (seg < (p.nseg + 64 / GL - 1) / (64 / GL) * (64 / GL)) {   // whole wavefronts: the exchanges below need every lane
-        const int sg = min(seg, p.nseg - 1);
-        const float4 *tk = reinterpret_cast<const float4 *>(lds_tab + (sg * TR + 0) * D + k_octet<GK>(gl >> 1, gl & 1) * 8);
-        const float4 a = tk[0], b = tk[1];
-        const float e[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        float mx = 0.f, tot = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { mx = fmaxf(mx, __builtin_fabsf(e[j])); tot += __builtin_fabsf(e[j]); }
-        mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-#pragma unroll
-        for (int off = 1; off < GL; off <<= 1) tot += __shfl_xor(tot, off, 64);
-        float w[NCH];
-        const int base = (threadIdx.x & 63) / GL * GL;   // first lane of the group (in hardware lane order)
-        // (rt reverses the lane order inside a wavefront: chunk c sits at lanes base + GL-1-2c and -2c-1)
-#pragma unroll
-        for (int ch = 0; ch < NCH; ++ch) w[ch] = __shfl(mx, base + GL - 1 - 2 * ch, 64);
-        const float thr = kLoRatio * tot * (1.f / D);
-        int so[NCH], cl[kMaxLo], n = 0;
-#pragma unroll
-        for (int ch = 0; ch < NCH; ++ch) so[ch] = -1;
-#pragma unroll
-        for (int sl = 0; sl < kMaxLo; ++sl) {
-          int best = -1;
-          float bw = 0.f;
-#pragma unroll
-          for (int ch = 0; ch < NCH; ++ch)
-            if (w[ch] >= thr && so[ch] < 0 && (best < 0 || w[ch] > bw)) { best = ch; bw = w[ch]; }
-#pragma unroll
-          for (int ch = 0; ch < NCH; ++ch)
-            if (ch == best) so[ch] = sl;
-          cl[sl] = best < 0 ? 0 : best;
-          n += best >= 0;
-        }
-        u32 slots = 0u, info = (u32)n << 16;
-#pragma unroll
-        for (int ch = 0; ch < NCH; ++ch) slots |= (u32)(so[ch] + 1) << (4 * ch);
-#pragma unroll
-        for (int sl = 0; sl < kMaxLo; ++sl) info |= (u32)cl[sl] << (4 * sl);
-        if (gl == 0 && seg < p.nseg) {
-          lds_clo[seg * 2] = slots;
-          lds_clo[seg * 2 + 1] = info;
-        }
-      }
-    }
-    __syncthreads();
   }
-  load_q(max(cur_a.seg, p.nconv), std::true_type{});   // (the merged run is attended with the base segment's tables)
-  if (n_tiles > 0) { stage(0); widen_k(0, std::true_type{}); }
+  __syncthreads();
+  if constexpr (CHAN) {
+    if (p.nseg > 1) {
+      // the segment of this workgroup's first key (a share of the keys may begin mid-cache)
+      wseg_end = __builtin_amdgcn_readfirstlane(lds_seg_end[0]);
+      widen_cursor(0);
+    }
+  }
+  load_q();
+  if (n_tiles > 0) { stage(0); widen_k(0); }
   if (n_tiles > 1) { prefetch_k(1); prefetch(1); stage(1); }
   __syncthreads();
-  if (n_tiles > 0) widen_v(0, std::true_type{});
+  if (n_tiles > 0) widen_v(0);
   if (n_tiles > 2) prefetch(2);
   __syncthreads();
 
@@ -930,7 +796,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
     for (int tile = 0; tile < n_tiles; ++tile) {
       if (tile + 2 < n_tiles) stage(tile + 2);
       if (tile + 3 < n_tiles) prefetch(tile + 3);
-      if (tile + 1 < n_tiles) { widen_v(tile + 1, std::false_type{}); widen_k(tile + 1, std::false_type{}); }
+      if (tile + 1 < n_tiles) { widen_v(tile + 1); widen_k(tile + 1); }
       if (tile + 2 < n_tiles) prefetch_k(tile + 2);
       __syncthreads();
     }
@@ -952,73 +818,8 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   float ckv[2][NSKA][16], svv[2][NSVA][16];
   u32x4_t vta[NDB], wza[NSVA];
 
-  // per-channel tables: segment of the tile being attended, end of the tile's keys, and the
-  // softmax denominator as it was when the current segment began
-  int seg_a = max(cur_a.seg, p.nconv), tile_end = 0;
-  bool in_merged = false;   // the tile being attended belongs to the merged run
-  float l_prev = 0.f;
-  // A new segment begins.  The true (unnormalized) output is, per channel,
-  //   sv * (kMul * oacc - rq - zv * (l_sum - l_prev))
-  // with rq, l_sum the readings of the extra block; the accumulators are re-expressed so that
-  // the same formula holds with the new tables and l_prev = l_sum, and the Q operands are
-  // rebuilt with the new K table.
-  auto segment_boundary = [&](int seg_new) __attribute__((always_inline)) {
-    if constexpr (CHAN) {
-      // (the Q operands first: with the accumulator arithmetic in front of it the register
-      // allocator spills, and spills here cost scratch traffic at every boundary)
-      // the Q operands with the new K table: from the kept registers at D=64, reloaded at D=128
-      load_q(seg_new, std::false_type{});
-      __builtin_amdgcn_sched_barrier(0);
-      const float l_sum = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
-      const float rq = __shfl(racc[0], col, 64) + r_run[0];
-      const float dl = l_sum - l_prev;
-      constexpr float VM = VCodec<BITS>::kMul;
-      // segments follow one another, so the ratio sv_old / sv_new is the new segment's entry row;
-      // with t = rq / VM and u = (rq + zv_old * dl) / VM the update is ro * (oacc - u) + t
-      const float *zv_old = lds_tab + (seg_a * TR + 3) * D, *ratio = lds_tab + (seg_new * TR + 4) * D;
-      const float t = rq * (1.f / VM), dlm = dl * (1.f / VM);
-#pragma unroll
-      for (int d = 0; d < NDB; ++d)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const int c0 = d * 32 + 8 * g4 + 4 * half;
-          const float4 r4 = *reinterpret_cast<const float4 *>(ratio + c0);
-          const float ro[4] = {r4.x, r4.y, r4.z, r4.w};
-          if (v_affine) {
-            const float4 zo = *reinterpret_cast<const float4 *>(zv_old + c0);
-            const float zz[4] = {zo.x, zo.y, zo.z, zo.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              oacc[d][4 * g4 + j] = __builtin_fmaf(ro[j], oacc[d][4 * g4 + j] - __builtin_fmaf(zz[j], dlm, t), t);
-          } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) oacc[d][4 * g4 + j] = __builtin_fmaf(ro[j], oacc[d][4 * g4 + j] - t, t);
-          }
-          __builtin_amdgcn_sched_barrier(0);   // one slice's registers at a time
-        }
-      l_prev = l_sum;
-      seg_a = seg_new;
-    }
-  };
-
   auto begin_tile = [&](int tile) {
-    if constexpr (CHAN) {
-      t0 = cur_a.start;
-      tile_end = min(t0 + BN, __builtin_amdgcn_readfirstlane(lds_seg_end[cur_a.seg]));
-      const int seg_t = max(cur_a.seg, p.nconv);
-      const bool was_merged = in_merged;
-      in_merged = merged_tile(tile);
-      if (__builtin_expect(seg_t != seg_a, 0)) {
-        segment_boundary(seg_t);
-      } else if (was_merged && !in_merged) {
-        // from the merged run into its base segment: same tables, but the zero-point term of
-        // the output belongs to the weights from here on only
-        l_prev = __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
-      }
-      cursor_advance(cur_a);
-    } else {
-      t0 = tile_base + tile * BN;
-    }
+    t0 = tile_base + tile * BN;
     kx = lds_kx + (tile & 1) * BN * KXS;
     par = lds_par + (tile % 3) * L::kParFloats;
     vt = lds_vt + (tile & 1) * D * VTS;
@@ -1032,14 +833,14 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
   // with the PV MFMAs of a block in flight: widen the next tile's K and V into the other slots
   auto widen_next = [&](int tile) {
     if (tile + 1 < n_tiles) {
-      widen_v(tile + 1, std::false_type{});
-      widen_k(tile + 1, std::false_type{});
+      widen_v(tile + 1);
+      widen_k(tile + 1);
       if (tile + 2 < n_tiles) prefetch_k(tile + 2);
     }
   };
   auto load_scales = [&](int kb) {
 #pragma unroll
-    for (int s = 0; s < ((HOIST && !CHAN && !DEQ) ? NSK : 0); ++s)
+    for (int s = 0; s < ((HOIST && !DEQ) ? NSK : 0); ++s)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int key = kb * 32 + 16 * (i4 >> 1) + 8 * half + 4 * (i4 & 1);
@@ -1076,15 +877,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       for (int j = 0; j < 16; ++j) zero[j] = 0.f;
       if constexpr (DEQ) {
         sacc[kb][s] = zero;   // (dequantized operands: no zero-point term)
-      } else if constexpr (CHAN) {
-        // The key side of the rank-1 term is a constant here and lives in qbias.  In its place:
-        // the remainder pass of the chunk with the largest outlier scale -- that chunk's K operand
-        // against q_lo.  Issued whether or not the segment has such a chunk (q_lo is zero then,
-        // and names chunk 0): a branch here would stand between the LDS requests of the chunk
-        // loop and their MFMAs.
-        const u32x4_t alo0 = *reinterpret_cast<const u32x4_t *>(&kx[krow_i * KXS + (half * NCH + (int)(lo_info & 7u)) * 8]);
-        sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, alo0),
-                                                              __builtin_bit_cast(bf16x8_t, qlo[0]), zero, 0, 0, 0);
       } else {
         // starts the accumulator with the zero-point term (see bq above)
         sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
@@ -1092,9 +884,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       }
     }
     const uint16_t *krow = &kx[krow_i * KXS];
-    // (the second slot's K operand is requested like the first: no branch ahead of the chunk loop)
-    u32x4_t alo1 = {0u, 0u, 0u, 0u};
-    if constexpr (CHAN) alo1 = *reinterpret_cast<const u32x4_t *>(&krow[(half * NCH + (int)((lo_info >> 4) & 7u)) * 8]);
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
       const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[k_octet<GK>(ch, half) * 8]);
@@ -1102,45 +891,26 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       sacc[kb][kAcc * (ch / (GK / 16))] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
           __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][kAcc * (ch / (GK / 16))], 0, 0, 0);
     }
-    if constexpr (CHAN) {
-      // further remainder passes: more than one chunk with an outlier scale
-      const int nlo = (int)(lo_info >> 16);
-      if (nlo > 1) {
-        sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, alo1),
-                                                              __builtin_bit_cast(bf16x8_t, qlo[1]), sacc[kb][0], 0, 0, 0);
-#pragma unroll
-        for (int sl = 2; sl < kMaxLo; ++sl) {
-          if (sl >= nlo) break;
-          const int c = (int)((lo_info >> (4 * sl)) & 7u);
-          const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[(half * NCH + c) * 8]);
-          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                __builtin_bit_cast(bf16x8_t, qlo[sl]), sacc[kb][0], 0, 0, 0);
-        }
-      }
-    }
     __builtin_amdgcn_s_setprio(0);
   };
 
   // logits -> P'^T operands of one block: online softmax against a lazily moved reference
   auto softmax = [&](int kb) {
     float z[16];
-    // CHAN: one factor for every key (keys of the merged run carry values, not code images)
-    const float ck_all = in_merged ? p.scale_log2e : p.scale_log2e * KCodec<BITS>::kMul;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      float v = CHAN ? (in_merged ? 0.f : qbias) - m_ref : -m_ref;
+      float v = -m_ref;
 #pragma unroll
       for (int s = 0; s < NSKA; ++s) {
         const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        v = __builtin_fmaf(DEQ ? p.scale_log2e : CHAN ? ck_all : HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key],
+        v = __builtin_fmaf(DEQ ? p.scale_log2e : HOIST ? ckv[kb][s][i] : par[P_CK + s * BN + key],
                            sacc[kb][s][i], v);
       }
       z[i] = v;
     }
-    // mask: block-causal key limit, the ragged last tile, and (per-channel tables) the
-    // keys of the next segment behind a short tile
-    const int lim_t = CHAN ? min(limit, tile_end) : limit;
-    if (t0 + BN > (CHAN ? min(wave_minlim, tile_end) : wave_minlim)) {
+    // mask: block-causal key limit and the ragged last tile
+    const int lim_t = limit;
+    if (t0 + BN > wave_minlim) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = t0 + kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
@@ -1172,7 +942,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
       for (int j = 0; j < 16; ++j) racc[j] *= alpha;
 #pragma unroll
       for (int s = 0; s < NSVA; ++s) r_run[s] *= alpha;
-      if constexpr (CHAN) l_prev *= alpha;
     }
     first = false;
     float pv[16];
@@ -1243,9 +1012,9 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
 
   for (int tile = 0; tile < n_tiles; ++tile) {
     begin_tile(tile);
-    // a tile with at most 32 keys (the end of a segment or of the cache) has nothing for
-    // the second key block: every weight there would be exp2(-inf) = 0
-    const bool half_tile = (CHAN ? min(kv_end, tile_end) : kv_end) - t0 <= 32;
+    // a tile with at most 32 keys (the end of the cache) has nothing for the second key
+    // block: every weight there would be exp2(-inf) = 0
+    const bool half_tile = kv_end - t0 <= 32;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       if (kb == 1 && half_tile) continue;
@@ -1290,17 +1059,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void fused_attn_kernel(AttnParams p) {
         // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
         float o0 = (VM * oacc[d][4 * g4 + 0] - r) * inv, o1 = (VM * oacc[d][4 * g4 + 1] - r) * inv;
         float o2 = (VM * oacc[d][4 * g4 + 2] - r) * inv, o3 = (VM * oacc[d][4 * g4 + 3] - r) * inv;
-        if constexpr (CHAN) {
-          // weighted mean of the codes -> values: sv * (mean - zv * share) per channel, share
-          // = the part of the weights that belongs to the current segment (1 without segments)
-          const int c0 = d * 32 + 8 * g4 + 4 * half;
-          const float4 sv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 2) * D + c0);
-          const float4 zv = *reinterpret_cast<const float4 *>(lds_tab + (seg_a * TR + 3) * D + c0);
-          // (a share that ended inside the merged run has no weight in the current segment)
-          const float share = in_merged ? 0.f : (l_sum - l_prev) * inv;   // inv = 0 for a query that sees no key
-          o0 = sv.x * (o0 - zv.x * share); o1 = sv.y * (o1 - zv.y * share);
-          o2 = sv.z * (o2 - zv.z * share); o3 = sv.w * (o3 - zv.w * share);
-        }
         if (shared_out) {
           *reinterpret_cast<float4 *>(wptr + d * 32 + 8 * g4 + 4 * half) = make_float4(o0, o1, o2, o3);
         } else {
@@ -1346,51 +1104,52 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
 
 int device_cus();
 
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, bool SEGS>
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, int WPS = 2>
 void launch_shape(const AttnParams &p, hipStream_t st) {
-  constexpr int lds_bytes = (AttnLds<D, BITS, GK, GV, CHAN>::kBytes + 15) / 16 * 16 + (CHAN ? kMaxSegments * (kChanTableRows * D + 2) * 4 : 0);
-  static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+  // (the per-channel tables take LDS by the number of segments of the launch)
+  constexpr int lds_base = (AttnLds<D, BITS, GK, GV, CHAN>::kBytes + 15) / 16 * 16, lds_seg = CHAN ? kChanTableRows * D * 4 : 0;
+  constexpr int lds_max = lds_base + kMaxSegments * lds_seg;
+  static_assert(lds_max <= 160 * 1024, "LDS budget");
+  const int lds_bytes = lds_base + p.nseg * lds_seg;
   // above 64 KiB the limit has to be raised, once per device the process launches on
   static bool configured[64] = {false};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !configured[dev]) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, SEGS>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);
     if (dev >= 0) configured[dev] = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, SEGS>), grid, dim3(NWV * 64), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS>), grid, dim3(NWV * 64), lds_bytes, st, p);
   if (p.nsplit > 1) {
     const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
     hipLaunchKernelGGL((combine_splits_kernel<D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
   }
 }
 
-template <int D, int BITS, int GK, int GV, bool CHAN, bool SEGS>
-void launch_nw(const AttnParams &p, hipStream_t st) {
+template <int D, int BITS, int GK, int GV, bool CHAN = false>
+void launch(const AttnParams &p, hipStream_t st) {
   if constexpr (D == 64) {
     // more (batch, head) pairs than compute units, at most four wavefronts of queries each:
     // small workgroups, two to a compute unit (same arithmetic, same results)
     if (p.Lq <= 128 && p.bh_total > device_cus()) {
-      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2, SEGS>(p, st);
-      else launch_shape<D, BITS, GK, GV, CHAN, 4, SEGS>(p, st);
+      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2>(p, st);
+      else launch_shape<D, BITS, GK, GV, CHAN, 4>(p, st);
       return;
     }
   }
-  launch_shape<D, BITS, GK, GV, CHAN, 8, SEGS>(p, st);
-}
-
-template <int D, int BITS, int GK, int GV, bool CHAN = false>
-void launch(const AttnParams &p, hipStream_t st) {
-  if constexpr (CHAN && D == 64) {   // (at D=128 the two kinds are the same code)
-    if (p.nseg > 1) {
-      launch_nw<D, BITS, GK, GV, true, true>(p, st);
+  if constexpr (D == 64 && AttnLds<D, BITS, GK, GV, CHAN>::kDeq) {
+    // The dequantizing kernels at D=64 fit 128 registers at the price of 36-96 bytes of spills,
+    // and two resident workgroups per compute unit hide each other's prologue and barriers:
+    // 5-13 % faster, except for one table of 8-bit codes (8 % slower: the most widening work).
+    if (!(CHAN && BITS == 8 && p.nseg == 1)) {
+      launch_shape<D, BITS, GK, GV, CHAN, 8, 4>(p, st);
       return;
     }
   }
-  launch_nw<D, BITS, GK, GV, CHAN, false>(p, st);
+  launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
 }
 
 template <int D, int BITS>
@@ -1486,7 +1245,8 @@ int set_splits(AttnParams &p, int D, int tiles, int splits, void *workspace, siz
 extern "C" size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk, int D, int nseg, int splits) {
   if (B <= 0 || Hkv <= 0 || Lq <= 0 || Lk <= 0 || (D != 64 && D != 128) || splits < 0 || splits > kMaxSplits) return 0;
   const int64_t rows = (int64_t)B * Hkv * Lq;
-  const int tiles = (Lk + BN - 1) / BN + (nseg > 1 ? nseg - 1 : 0);
+  (void)nseg;   // (the tile count does not depend on the tables)
+  const int tiles = (Lk + BN - 1) / BN;
   const int n = splits ? splits : choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), tiles, rows, D);
   return split_workspace_bytes(n, rows, D);
 }
@@ -1521,7 +1281,6 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.k_scale = k_scale; p.k_zp = k_zp; p.v_scale = v_scale; p.v_zp = v_zp;
   p.k_chan_scale = nullptr; p.k_chan_zp = nullptr; p.v_chan_scale = nullptr; p.v_chan_zp = nullptr;
   p.nseg = 1;
-  p.nconv = 0;
   for (int s = 0; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
   p.head_map = head_map; p.kv_limit = kv_limit;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
@@ -1591,17 +1350,13 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
     prev = e;
   }
   for (int s = nseg; s < kMaxSegments; ++s) p.seg_end[s] = Lk;
-  // leading segments that together fit one key tile are merged into the segment behind them
-  p.nconv = 0;
-  // (one tile: the kernel converts codes to values in its prologue only)
-  while (D == 64 && p.nconv + 1 < nseg && p.seg_end[p.nconv] <= BN) ++p.nconv;
   p.head_map = head_map; p.kv_limit = kv_limit;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
   if (int e = set_layout(p, layout, "fused_attn_channel")) return e;
-  if (int e = set_splits(p, D, (Lk + BN - 1) / BN + nseg - 1, splits, workspace, workspace_bytes, "fused_attn_channel"))
+  if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn_channel"))
     return e;
   hipStream_t st = (hipStream_t)stream;
   if (D == 128) {
