@@ -229,6 +229,10 @@ int varq_fused_attn(const void *q, void *out,
  *                        fp32 [nseg, Hkv, D]; zero-points NULL = symmetric.  With one
  *                        segment k_chan_zp may be NULL for an affine K as well: it shifts
  *                        every logit of a query by the same amount, which the softmax cancels
+ *                        (K is then offset per channel before it is rounded to bf16)
+ * K and V are dequantized with the tables of each key's segment as tiles enter LDS,
+ * (code - zp) * scale in fp32 rounded to bf16: the operands of the reference's attention
+ * after dequant_all (VAR_Q/quant.py:216-224) and its bf16 attention call.
  *   nseg, host_seg_end   1..16 segments; host int32 [nseg] (may be NULL when nseg == 1)
  *   everything else as in varq_fused_attn; one bit-width for K and V.
  */
