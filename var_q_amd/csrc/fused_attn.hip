@@ -293,10 +293,12 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 }
 
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
-// (kDeq: per-channel tables, or more than one K or V group per key -- those kernels dequantize when
-// a tile is widened, see the kernel, and have no rank-1 operands)
+// kDeq: the kernel dequantizes when a tile is widened (see the kernel) and has no rank-1 operands:
+// per-channel tables, more than one K or V group per key, and -- by measurement -- every kernel
+// at D=64 and the 8-bit kernels at D=128.  Exact codes in the MFMA operands remain where they are
+// the faster form: one group per key of 4- or 2-bit codes at D=128 (configuration 4).
 template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
-  static constexpr bool kDeq = CHAN || (D / GK > 1 || D / GV > 1);
+  static constexpr bool kDeq = CHAN || (D / GK > 1 || D / GV > 1) || D == 64 || BITS == 8;
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
   static constexpr bool kFoldSv = !kDeq && (D / GV == 1);   // one V group: its scale rides inside the logits
@@ -328,13 +330,15 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
-  // DEQ: several K or V groups per key.  Carrying exact codes through the MFMAs would need one
-  // logit accumulator and one rank-1 MFMA per K group and one set of weights and one extra MFMA
-  // per V group (19 -> 28 MFMAs per key block at four groups, and registers that do not exist).
-  // These kernels dequantize instead when a tile is widened -- (code - zp) * scale in fp32,
-  // rounded to bf16, the very values the reference's attention sees after its dequantize and
-  // downcast (VAR_Q/quant.py:216-224, VAR/models/basic_var.py:158) -- and then run like a plain
-  // bf16 flash attention: one accumulator, one set of weights, whatever the group count.
+  // DEQ: the kernel dequantizes when a tile is widened -- (code - zp) * scale in fp32, rounded to
+  // bf16, the very values the reference's attention sees after its dequantize and downcast
+  // (VAR_Q/quant.py:216-224, VAR/models/basic_var.py:158) -- and then runs like a plain bf16 flash
+  // attention: one accumulator, one set of weights, whatever the group count, no rank-1 MFMA and
+  // no extra O^T block (the softmax denominator is summed on the vector ALU).  With several K or
+  // V groups per key, exact codes in the MFMAs would need one logit accumulator and one rank-1
+  // MFMA per K group and one set of weights and one extra MFMA per V group (19 -> 28 MFMAs per
+  // key block at four groups, and registers that do not exist); where there is one group, which
+  // form is faster was measured (see AttnLds::kDeq).
   constexpr bool DEQ = AttnLds<D, BITS, GK, GV, CHAN>::kDeq;
   constexpr int NSKA = DEQ ? 1 : NSK, NSVA = DEQ ? 1 : NSV;   // accumulators / weight sets
   static_assert(NW >= NSK && NW >= NSV && NW >= 2, "one wavefront per K group and per V group stages the parameters");
@@ -492,6 +496,9 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   floatx16_t racc;
 #pragma unroll
   for (int j = 0; j < 16; ++j) racc[j] = 0.f;
+  // DEQ: no extra block; the softmax denominator is summed on the vector ALU from the weights as
+  // rounded for the MFMA (this lane's keys; the two lane halves are added in the epilogue)
+  float l_part = 0.f;
   float m_ref = 0.f;                 // softmax reference (log2 domain)
   float r_run[NSVA];                 // sum_l p' * vzp_r, only fed on tiles with a remainder
 #pragma unroll
@@ -636,8 +643,6 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   int rowsel[NSVA];
 #pragma unroll
   for (int s = 0; s < NSVA; ++s) rowsel[s] = ((col == s) ? s : (s == 0 && col >= 4 && col < 7) ? col : 7) * RSR;
-  // DEQ: row 0 of the extra block is a row of ones (the softmax denominator), the others zero
-  const u32 ones_a = (DEQ && col == 0) ? 0x3f803f80u : 0u;
 
   // CHAN: the widening of `tile` begins: (wseg, wseg_end) follow the tile's first key
   auto widen_cursor = [&](int tile) {
@@ -863,7 +868,6 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 #pragma unroll
     for (int s = 0; s < (DEQ ? 0 : NSV); ++s)
       wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
-    if constexpr (DEQ) wza[0] = u32x4_t{ones_a, ones_a, ones_a, ones_a};
   };
 
   // S^T = K Q^T for one 32-key block; the A operands are the widened K rows in LDS
@@ -939,7 +943,8 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 #pragma unroll
         for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) racc[j] *= alpha;
+      for (int j = 0; j < (DEQ ? 0 : 16); ++j) racc[j] *= alpha;
+      if constexpr (DEQ) l_part *= alpha;
 #pragma unroll
       for (int s = 0; s < NSVA; ++s) r_run[s] *= alpha;
     }
@@ -959,6 +964,11 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         else
           pop[kb][s][i >> 3][(i & 7) >> 1] =
               pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
+        if constexpr (DEQ) {   // += the two rounded weights (one v_dot2 against a pair of ones)
+          typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+          l_part = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
+                                                   __builtin_bit_cast(bf16x2_t, 0x3f803f80u), l_part, false);
+        }
       }
     if (!DEQ && tile_rem) {
       // the remainder term must see the same bf16-rounded weights as the MFMA
@@ -987,7 +997,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 #pragma unroll
       for (int d = 0; d < NDB; ++d) av[d] = vta[d];
 #pragma unroll
-      for (int s = 0; s < NSVA; ++s) aw[s] = wza[s];
+      for (int s = 0; s < (DEQ ? 0 : NSVA); ++s) aw[s] = wza[s];
       if (HOIST && c == 0) {
         load_v_operands(kb, 1);   // in flight under this chunk's MFMAs
         __builtin_amdgcn_sched_barrier(0);
@@ -1001,7 +1011,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
                                                           __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
       }
 #pragma unroll
-      for (int s = 0; s < NSVA; ++s) {
+      for (int s = 0; s < (DEQ ? 0 : NSVA); ++s) {
         u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
         racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
                                                        __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
@@ -1036,7 +1046,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   for (int s = 0; s < NSVA; ++s) r_run[s] += __shfl_xor(r_run[s], 32, 64);
   // rows 4..6 of racc are registers 0..2 of the upper lane half, rows 0..3 registers 0..3 of the lower
   // (DEQ: the denominator is row 0, the sum of the weights against the row of ones)
-  const float l_sum = DEQ ? __shfl(racc[0], col, 64) : __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
+  const float l_sum = DEQ ? l_part + __shfl_xor(l_part, 32, 64) : __shfl(racc[0] + racc[1] + racc[2], col + 32, 64);
   const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
   float rq[NSVA];
 #pragma unroll
@@ -1141,13 +1151,11 @@ void launch(const AttnParams &p, hipStream_t st) {
     }
   }
   if constexpr (D == 64 && AttnLds<D, BITS, GK, GV, CHAN>::kDeq) {
-    // The dequantizing kernels at D=64 fit 128 registers at the price of 36-96 bytes of spills,
-    // and two resident workgroups per compute unit hide each other's prologue and barriers:
-    // 5-13 % faster, except for one table of 8-bit codes (8 % slower: the most widening work).
-    if (!(CHAN && BITS == 8 && p.nseg == 1)) {
-      launch_shape<D, BITS, GK, GV, CHAN, 8, 4>(p, st);
-      return;
-    }
+    // The dequantizing kernels at D=64 fit 128 registers at the price of 24-48 bytes of spills,
+    // and two resident workgroups per compute unit hide each other's prologue and barriers
+    // (8-15 % faster than one workgroup at 140 registers).
+    launch_shape<D, BITS, GK, GV, CHAN, 8, 4>(p, st);
+    return;
   }
   launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
 }
