@@ -1155,9 +1155,9 @@ void launch(const AttnParams &p, hipStream_t st) {
     // and two resident workgroups per compute unit hide each other's prologue and barriers
     // (8-15 % faster than one workgroup at 140 registers).
     launch_shape<D, BITS, GK, GV, CHAN, 8, 4>(p, st);
-    return;
+  } else {
+    launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
   }
-  launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
 }
 
 template <int D, int BITS>
