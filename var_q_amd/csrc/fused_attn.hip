@@ -511,26 +511,40 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 
   constexpr int QUADS = BN * WPR / 4;                 // 16-byte pieces per packed tile
   constexpr int LPT = (QUADS + NT - 1) / NT;          // pieces per thread
-  u32x4_t kreg[LPT], vreg[LPT];
+  // The K tile is loaded in pieces of KPW words, small enough that every thread of the workgroup
+  // has one where the tile allows it (the thread that loads a piece widens it, so this spreads
+  // the widening evenly: 2-bit codes at D=64 would otherwise occupy a single wavefront).
+  // (the V tile is widened in (BN/2)*(D/8) items by the upper wavefronts; where those are fewer than
+  // the threads, the K pieces go to the threads that are left)
+  constexpr int K_THREADS = ((BN / 2) * (D / 8) < NT) ? NT - (BN / 2) * (D / 8) : NT;
+  // (measured: 5-9 % faster for 2-bit codes and at D=64; 4-bit codes at D=128 are 5 % slower in
+  // 8-byte pieces -- twice the per-piece parameter loads -- and keep 16-byte ones)
+  constexpr int KPW = (DEQ && (D == 64 || BITS == 2) && BN * WPR / K_THREADS < 4) ? (BN * WPR / K_THREADS < 2 ? 1 : 2) : 4;
+  constexpr int KPIECES = BN * WPR / KPW, KPPR = WPR / KPW;   // pieces per tile, per key row
+  constexpr int KLPT = (KPIECES + NT - 1) / NT;
+  u32x4_t kreg[KLPT], vreg[LPT];   // (a K piece uses the first KPW words of its register)
   float ksc = 0.f, kzp = 0.f, vsc = 0.f, vzp = 0.f, ksc0 = 0.f;
   // DEQ: scale and zero-point of the K groups that the thread's 16-byte pieces hold (a piece is
   // 128 / BITS channels of one key: one group, or two for 2-bit codes in groups of 32)
-  constexpr int CPP = 128 / BITS;                       // channels per piece
+  constexpr int CPP = KPW * 32 / BITS;                  // channels per piece
   constexpr int GPP = (DEQ && CPP > GK) ? CPP / GK : 1; // groups per piece
   constexpr bool KGP = DEQ && !CHAN;                    // K group parameters travel with the pieces
-  float kgs[KGP ? LPT * GPP : 1], kgz[KGP ? LPT * GPP : 1];
+  float kgs[KGP ? KLPT * GPP : 1], kgz[KGP ? KLPT * GPP : 1];
 
   auto prefetch_k = [&](int) {   // the next tile of the K stream
     const int t0 = tile_base + pk_tile * BN;
     ++pk_tile;
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) {
+    for (int i = 0; i < KLPT; ++i) {
       const int piece = tid + i * NT;
-      if (LPT * NT == QUADS || piece < QUADS) {
-        const int key = min(t0 + piece / (WPR / 4), p.Lk - 1);
-        kreg[i] = *reinterpret_cast<const u32x4_t *>(kw + key * kv_ts * WPR + (piece % (WPR / 4)) * 4);
+      if (KLPT * NT == KPIECES || piece < KPIECES) {
+        const int key = min(t0 + piece / KPPR, p.Lk - 1);
+        const u32 *src = kw + key * kv_ts * WPR + (piece % KPPR) * KPW;
+        if constexpr (KPW == 4) kreg[i] = *reinterpret_cast<const u32x4_t *>(src);
+        else if constexpr (KPW == 2) { const uint2 t = *reinterpret_cast<const uint2 *>(src); kreg[i][0] = t.x; kreg[i][1] = t.y; }
+        else kreg[i][0] = src[0];
         if constexpr (KGP) {
-          const int g0 = (piece % (WPR / 4)) * CPP / GK;   // first group of the piece
+          const int g0 = (piece % KPPR) * CPP / GK;   // first group of the piece
 #pragma unroll
           for (int j = 0; j < GPP; ++j) {
             const int64_t g = (kv_row0 + key * kv_ts) * NSK + g0 + j;
@@ -670,7 +684,12 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
     uint16_t *vt = lds_vt + (tile & 1) * D * VTS;
     widen_cursor(tile);
     const bool one_seg = !CHAN || tile_in_one_segment(tile);
-    for (int item = tid; item < (BN / 2) * (D / 8); item += NT) {
+    // (where the tile has fewer items than the workgroup has threads, the upper wavefronts take
+    // them: the K pieces are widened by the lower ones)
+    constexpr int V_ITEMS = (BN / 2) * (D / 8);
+    constexpr int V_ROT = V_ITEMS < NT ? NT - V_ITEMS : 0;
+    for (int item = tid - V_ROT; item < V_ITEMS; item += NT) {
+      if (V_ROT && item < 0) continue;
       const int kp2 = item & (BN / 2 - 1), oct = item / (BN / 2);
       const u32 *row = &vp[kp2 * 2 * RSV];
       u32 pr[8];
@@ -709,20 +728,22 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
     }
   };
 
-  // packed K of `tile` (in kreg) -> widened bf16 rows: each 16-byte piece holds OPQ octets
+  // packed K of `tile` (in kreg) -> widened bf16 rows: each piece holds OPQ octets
   // of one key, every octet becomes one 16-byte MFMA A operand
   auto widen_k = [&](int tile) {
     uint16_t *kx = lds_kx + (tile & 1) * BN * KXS;
-    constexpr int OPQ = 16 / BITS;            // octets per 16-byte piece
+    constexpr int OPQ = KPW * 4 / BITS;       // octets per piece
     widen_cursor(tile);
     const bool one_seg = !CHAN || tile_in_one_segment(tile);
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) {
+    for (int i = 0; i < KLPT; ++i) {
       const int piece = tid + i * NT;
-      if (LPT * NT == QUADS || piece < QUADS) {
-        const int key = piece / (WPR / 4), oct0 = (piece % (WPR / 4)) * OPQ;
+      if (KLPT * NT == KPIECES || piece < KPIECES) {
+        const int key = piece / KPPR, oct0 = (piece % KPPR) * OPQ;
         constexpr u32 KX = KCodec<BITS>::kStageXor;
-        const u32 q4[4] = {kreg[i][0] ^ KX, kreg[i][1] ^ KX, kreg[i][2] ^ KX, kreg[i][3] ^ KX};
+        u32 q4[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) q4[w] = w < KPW ? kreg[i][w] ^ KX : 0u;
         int sg = wseg;
         if constexpr (CHAN) {
           if (!one_seg) sg = key_segment(min(tile_base + tile * BN + key, p.Lk - 1));
