@@ -258,6 +258,49 @@ def prepare_rates(torch, dev):
             'tokens_per_s': round(Bp * Lp / dt, 1), 'algorithmic_MB': round(nbytes / 1e6, 2)}
 
 
+def pack_unpack_rates(torch, dev):
+    """The pack and unpack kernels on their own (the reference's pack_last_dim_to_int32 /
+    unpack_last_dim_from_int32 on int8 codes): configuration-4 shape [2,16,10521,128], INT4, INT2
+    and INT8, 40 back-to-back launches through the C ABI between one event pair; four sets of
+    source and destination buffers are cycled.  Bytes: the int8 codes plus the packed words, each moved once."""
+    from var_q_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    rows, c = B * H * L, D
+    gd = torch.Generator(device=dev).manual_seed(7007)
+    out = {'workload': 'int8 codes [2,16,10521,128] <-> packed int32 words, standalone pack / unpack kernels'}
+    for bits in (4, 2, 8):
+        lo, hi = -(1 << (bits - 1)), (1 << (bits - 1))
+        codes = [torch.randint(lo, hi, (rows, c), device=dev, generator=gd, dtype=torch.int8) for _ in range(4)]
+        words = [torch.empty((rows, c * bits // 32), dtype=torch.int32, device=dev) for _ in range(4)]
+        back = [torch.empty((rows, c), dtype=torch.int8, device=dev) for _ in range(4)]
+        i = [0]
+
+        def pack():
+            i[0] += 1
+            _lib.check(lib.varq_pack(codes[i[0] % 4].data_ptr(), rows, c, bits, words[i[0] % 4].data_ptr(), stream), 'varq_pack')
+
+        def unpack():
+            i[0] += 1
+            _lib.check(lib.varq_unpack(words[i[0] % 4].data_ptr(), rows, c, bits, back[i[0] % 4].data_ptr(), stream), 'varq_unpack')
+        for j in range(4):
+            i[0] = j - 1
+            pack()
+        t_p = timed_launches(torch, pack, reps=40, warm=8)
+        t_u = timed_launches(torch, unpack, reps=40, warm=8)
+        i[0] = 0
+        unpack()
+        torch.cuda.synchronize()
+        assert torch.equal(back[1], codes[1]), 'pack -> unpack does not return the codes'
+        nbytes = rows * c + rows * c * bits // 8
+        out['int%d' % bits] = {'pack_us': round(t_p * 1e6, 1), 'pack_GBps': round(nbytes / t_p / 1e9, 1),
+                               'pack_frac_hbm_peak': round(nbytes / t_p / 1e9 / HBM_PEAK_GBPS, 4),
+                               'unpack_us': round(t_u * 1e6, 1), 'unpack_GBps': round(nbytes / t_u / 1e9, 1),
+                               'unpack_frac_hbm_peak': round(nbytes / t_u / 1e9 / HBM_PEAK_GBPS, 4), 'algorithmic_MB': round(nbytes / 1e6, 2)}
+        del codes, words, back
+    return out
+
+
 def shipped_rule_latency(torch, dev, passes=5, warm=2):
     """The rules of the shipped JSON files (G_SCALE_HEAD_DIM, 8 bits), one layer, per scale
     quantize + cache K and V with the drop-in quantizers, then attend:
@@ -347,6 +390,7 @@ def main():
     ap.add_argument('--single-launches', action='store_true', help='quantize K and V in two launches instead of one')
     ap.add_argument('--no-rule', action='store_true', help='skip the shipped-rule latency leg (profiling runs)')
     ap.add_argument('--no-prepare', action='store_true', help='skip the producer-side (qkv_prepare) leg (profiling runs)')
+    ap.add_argument('--no-pack', action='store_true', help='skip the standalone pack / unpack leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -548,6 +592,7 @@ def main():
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
         'qkv_prepare_rates': None if args.no_prepare else prepare_rates(torch, dev),
+        'pack_unpack_rates': None if args.no_pack else pack_unpack_rates(torch, dev),
         'shipped_rule_latency': None if args.no_rule else shipped_rule_latency(torch, dev),
     }
     print(json.dumps(line), flush=True)
