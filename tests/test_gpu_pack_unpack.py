@@ -88,3 +88,33 @@ def test_dequant_ragged_channels_and_expanded_scale(dev):
     s = (torch.rand(1, 1, 3, 10, generator=g) + 0.1).expand(1, 5, 3, 10)     # stride-0 expand along L
     got = ops.dequant(words.to(dev), s.to(dev).expand(1, 5, 3, 10), None, 10, 4)
     assert torch.equal(got.cpu(), O.dequant_sym(q, s))
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('rows,c,word_offset', [(5, 64, 0), (5, 64, 1), (7, 16, 0), (3, 48, 2), (1, 16, 0), (1021, 128, 0), (1021, 128, 3)])
+def test_pack_unpack_word_tails_and_unaligned_words(dev, bits, rows, c, word_offset):
+    """The fast kernels move 16 bytes per thread; word counts that are not a multiple of four and
+    word buffers that start off a 16-byte boundary take the per-word kernel for the rest (or for
+    everything).  Through the C ABI, against the oracle's words."""
+    from var_q_amd import _lib
+    if c % (32 // bits):
+        pytest.skip('whole words only')
+    note('pack/unpack tails', bits, rows, c, word_offset)
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    lo, hi = O.qrange(bits)
+    g = torch.Generator().manual_seed(100 * bits + rows + word_offset)
+    q = torch.randint(lo, hi + 1, (rows, c), generator=g, dtype=torch.int8)
+    want, _ = O.pack_last_dim(q, bits)
+    wpr = c * bits // 32
+    qd = q.to(dev)
+    buf = torch.full((rows * wpr + 8,), 0x5a5a5a5a, dtype=torch.int32, device=dev)
+    words = buf[word_offset:word_offset + rows * wpr]
+    _lib.check(lib.varq_pack(qd.data_ptr(), rows, c, bits, words.data_ptr(), st), 'varq_pack')
+    torch.cuda.synchronize()
+    assert torch.equal(words.cpu().reshape(rows, wpr), want)
+    assert int(buf[word_offset + rows * wpr]) == 0x5a5a5a5a and (word_offset == 0 or int(buf[word_offset - 1]) == 0x5a5a5a5a), 'wrote past its words'
+    back = torch.full((rows * c + 16,), 99, dtype=torch.int8, device=dev)
+    _lib.check(lib.varq_unpack(words.data_ptr(), rows, c, bits, back.data_ptr(), st), 'varq_unpack')
+    torch.cuda.synchronize()
+    assert torch.equal(back[:rows * c].cpu().reshape(rows, c), q) and int(back[rows * c]) == 99
