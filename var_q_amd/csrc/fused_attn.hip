@@ -14,35 +14,39 @@
 //    S^T = K Q^T and O^T = V^T P^T, so that a lane owns one query column: row
 //    max/sum are per-lane (one cross-half exchange per tile) and the S^T
 //    accumulator registers are directly the B operand of the second MFMA.
-//  * The MFMA operands are exact small numbers derived from the codes, never
-//    scaled or rounded: a code lands in the top mantissa bits of a bf16 1.x
-//    (raw = (code + kOff) / kMul), which costs one shift and one and-or per two
-//    elements.  Scales are applied in fp32, zero-points ride on extra MFMA work:
-//       S[l,q]  = ck[l] * ( sum_d rawK[l,d] q[d]  -  (kzp[l]+kOff)/kMul * sum_d q[d] )
-//       O[q,:]  = ( kMul * sum_l p'[l,q] rawV[l,:]  -  sum_l p'[l,q] (vzp[l]+kOff) ) / sum_l p[l,q]
-//    The second term of S is a rank-1 update: both factors are split into three
-//    bf16 pieces and laid on the 16 contraction slots of one more MFMA per key
-//    block.  The second term of O is one more row of V^T (one more 32-row MFMA
-//    block whose row s carries vzp+kOff of V group s).  p' = bf16(p * vs[l]); with a
-//    single V group log2(vs)/ck is added to S through spare slots of the rank-1
-//    MFMA, so exp2 yields p * vs directly, and the denominator is accumulated as
-//    sum_l p'[l,q] / vs[l] by rows 4..6 of the extra block (1/vs in three bf16
-//    pieces): numerator and denominator then use the same rounded weights.
-//    V zero-points beyond +-kZmax (data offset by hundreds of quantization steps)
-//    or with a fractional part are split zp = zp_c + zp_r; the remainder goes
-//    through an fp32 correction term on tiles that have one.
-//  * Packed K and V tiles go HBM -> registers -> LDS as they are (16-byte loads,
-//    issued three tiles ahead, one workgroup barrier per tile).  K words are
-//    widened in registers by each wavefront straight into MFMA A operands,
-//    interleaved with the MFMAs (8 codes of one word = one lane's operand).  V is
-//    widened once per workgroup and written transposed to LDS (the PV contraction
-//    runs over keys).
+//  * Packed K and V tiles go HBM -> registers -> LDS (16-byte loads, issued one to three
+//    tiles ahead, one workgroup barrier per tile).  K is widened once per workgroup,
+//    straight from the registers it was loaded into, to LDS rows that are MFMA A operands;
+//    V goes to LDS packed and is widened and transposed by 2 keys x 8 channels per thread
+//    (the PV contraction runs over keys).  Widened tiles are double-buffered, packed V and
+//    the per-key parameters triple-buffered.
 //  * Key rows are fed to the first MFMA in a permuted order chosen so that each
 //    lane's accumulator registers hold 8 consecutive keys per 16-key chunk,
 //    which makes the V^T operand a single 16-byte LDS read.
 //  * Online softmax in the log2 domain against a reference that is only moved
 //    when some row's maximum exceeds it by 2^16: the common tile needs no
 //    subtraction and no rescale of the output accumulators.
+//  * Two forms of the operands (AttnLds::kDeq says which instantiation takes which):
+//    - dequantized: (code - zp) * scale in fp32, rounded to bf16, when a tile is widened -- the
+//      operands the reference's attention sees -- and a plain bf16 flash attention behind it;
+//      per-(head, channel) tables that change along the keys, several groups per key, every
+//      kernel at head dim 64 and the 8-bit kernels at head dim 128;
+//    - exact codes (one group per key of 4- or 2-bit codes at head dim 128): the MFMA operands
+//      are exact small numbers derived from the codes, never scaled or rounded.  A code lands in
+//      the top mantissa bits of a bf16 1.x (raw = (code + kOff) / kMul), which costs one shift and
+//      one and-or per two elements.  Scales are applied in fp32, zero-points ride on extra MFMA
+//      work:
+//         S[l,q]  = ck[l] * ( sum_d rawK[l,d] q[d]  -  (kzp[l]+kOff)/kMul * sum_d q[d] )
+//         O[q,:]  = ( kMul * sum_l p'[l,q] rawV[l,:]  -  sum_l p'[l,q] (vzp[l]+kOff) ) / sum_l p[l,q]
+//      The second term of S is a rank-1 update: both factors are split into three bf16 pieces
+//      and laid on the 16 contraction slots of one more MFMA per key block.  The second term of
+//      O is one more row of V^T (one more 32-row MFMA block whose row 0 carries vzp+kOff).
+//      p' = bf16(p * vs[l]): log2(vs)/ck is added to S through spare slots of the rank-1 MFMA,
+//      so exp2 yields p * vs directly, and the denominator is accumulated as sum_l p'[l,q] / vs[l]
+//      by rows 4..6 of the extra block (1/vs in three bf16 pieces): numerator and denominator
+//      then use the same rounded weights.  V zero-points beyond +-kZmax (data offset by hundreds
+//      of quantization steps) or with a fractional part are split zp = zp_c + zp_r; the remainder
+//      goes through an fp32 correction term on tiles that have one.
 #include <type_traits>
 
 #include "varq_common.h"
