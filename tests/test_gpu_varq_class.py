@@ -244,3 +244,26 @@ def test_layout_change_with_cached_steps_is_refused(dev):
     q.qkv_format = 'BLHc'
     with pytest.raises(ValueError, match='qkv_format was changed'):
         q.use_var_q(x)
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('method', ['G_SCALE_HEAD_DIM', 'G_TOKEN', 'G_HEAD_DIM', 'G_TENSOR'])
+def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method):
+    """use_var_q dequantizes only the new step and keeps the earlier values; calls of quant() and
+    cache() on their own in between (the fused path makes them) must not leave it with stale
+    values, and a result handed out earlier must not change when later steps arrive."""
+    note('VAR_Q incremental dequant', fmt, method)
+    ref, gpu = O.OracleVARQ(8, fmt, method), VAR_Q(8, fmt, method)
+    steps = _steps(fmt, torch.float32, seed=77) + _steps(fmt, torch.float32, seed=78)
+    held = []
+    for i, x in enumerate(steps):
+        if i in (2, 5):                      # a step cached without asking for the dequantized cache
+            ref.quant(x); ref.cache()
+            gpu.quant(x.to(dev)); gpu.cache()
+            continue
+        want, got = ref.use_var_q(x), gpu.use_var_q(x.to(dev))
+        assert got.shape == want.shape and torch.equal(got.cpu(), want), f'step {i}'
+        assert torch.equal(gpu.dequant_all().cpu(), want), f'step {i}: dequant_all'
+        held.append((got, want.clone()))
+    for got, want in held:
+        assert torch.equal(got.cpu(), want), 'an earlier result changed'

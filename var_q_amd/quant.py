@@ -167,6 +167,8 @@ class VAR_Q:
         self._c_item = _Growable(self.dim_cat, room)
         self._c_scale = _Growable(self.dim_cat, room)
         self._c_zp = _Growable(self.dim_cat, room)
+        # the dequantized cache as use_var_q hands it out, kept from step to step (see use_var_q)
+        self._c_deq = _Growable(self.dim_cat, room)
 
     def reserve_tokens(self, n_tokens: int):
         """Size the cache buffers for n_tokens at their first allocation (an extension: the
@@ -174,7 +176,7 @@ class VAR_Q:
         when they run out, and a caller that knows the schedule's length avoids those copies).
         Takes effect for buffers not allocated yet."""
         self._reserved_tokens = int(n_tokens)
-        for g in (self._tok_scale, self._tok_zp, self._c_item, self._c_scale, self._c_zp):
+        for g in (self._tok_scale, self._tok_zp, self._c_item, self._c_scale, self._c_zp, self._c_deq):
             g.min_capacity = max(64, self._reserved_tokens)
 
     @property
@@ -441,9 +443,26 @@ class VAR_Q:
         return self._dequant(self.cached_item, self.cached_scale, self.cached_zp)
 
     def use_var_q(self, item: torch.Tensor) -> torch.Tensor:
+        """quant + cache + dequant_all (VAR_Q/quant.py:226-230).  The reference dequantizes the whole
+        cache at every step; under the appending methods the codes and scales of earlier steps never
+        change, so their fp32 values are kept from step to step and only the new step is
+        dequantized and put behind them: the same values (the step's scale is what the expanded
+        cached scale holds for its tokens), O(step) instead of O(cache) per call.  The result is the
+        valid prefix of that buffer (like `cached_item`, a view that is not contiguous when the
+        buffer has room to spare).  `dequant_all()` itself still recomputes everything."""
         self.quant(item)
         self.cache()
-        return self.dequant_all()
+        d, n = self._c_deq, self.quantized_item.size(self.dim_cat)
+        if self.quant_method == 'G_HEAD_DIM' or self._c_item.buf is None or d.dim != self.dim_cat or d.len + n != self._c_item.len:
+            # (the replacing method; or the kept values are not those of the cache's earlier steps:
+            # quant() and cache() were also called on their own, or the layout was re-assigned)
+            full = self.dequant_all()
+            if self.quant_method != 'G_HEAD_DIM' and self._c_item.buf is not None:
+                self._c_deq = _Growable(self.dim_cat, self._c_item.min_capacity)
+                self._c_deq.append(full)
+            return full
+        d.append(self.dequant_current())
+        return d.view()
 
 
 def _dequant_views(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], c: int, bits: int,
