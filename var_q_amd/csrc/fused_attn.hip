@@ -946,18 +946,19 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         if (key >= lim_t) z[i] = -INFINITY;
       }
     }
-    float zmax = z[0];
+    // Moves the softmax reference to the row's current maximum: up only (never down) once
+    // something has been accumulated; the very first block takes its maximum as it is, negative
+    // or not (the accumulators are still zero, so alpha = 1 is exact).
+    auto move_reference = [&]() {
+      float zmax = z[0];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
-    {
-      // the other lane half of the same query, without a trip through LDS
-      const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
-      zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
-    }
-    if (first || __any(zmax > kRescaleAt)) {
-      // Move the reference to the row's current maximum: up only (never down) once
-      // something has been accumulated; the very first block takes its maximum as it
-      // is, negative or not (the accumulators are still zero, so alpha = 1 is exact).
+      for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
+      {
+        // the other lane half of the same query, without a trip through LDS
+        const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
+        zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
+      }
+      if (!DEQ && !(first || __any(zmax > kRescaleAt))) return;
       const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
       const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
       m_ref += delta;
@@ -972,29 +973,53 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
       if constexpr (DEQ) l_part *= alpha;
 #pragma unroll
       for (int s = 0; s < NSVA; ++s) r_run[s] *= alpha;
-    }
-    first = false;
-    float pv[16];
+    };
+    // exp2 of the logits, rounded to bf16 pairs for the MFMA; DEQ: also their sum (this lane's keys)
+    float blk = 0.f;
+    auto weights = [&]() {
+      float pv[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
+      for (int i = 0; i < 16; ++i) pv[i] = __builtin_amdgcn_exp2f(z[i]);
+      blk = 0.f;
 #pragma unroll
-    for (int s = 0; s < NSVA; ++s)
+      for (int s = 0; s < NSVA; ++s)
 #pragma unroll
-      for (int i2 = 0; i2 < 8; ++i2) {
-        const int i = 2 * i2;
-        const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-        if constexpr (FOLD_SV || DEQ) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
-        else if constexpr (HOIST)
-          pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[kb][s][i], pv[i + 1] * svv[kb][s][i + 1]);
-        else
-          pop[kb][s][i >> 3][(i & 7) >> 1] =
-              pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
-        if constexpr (DEQ) {   // += the two rounded weights (one v_dot2 against a pair of ones)
-          typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-          l_part = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
-                                                   __builtin_bit_cast(bf16x2_t, 0x3f803f80u), l_part, false);
+        for (int i2 = 0; i2 < 8; ++i2) {
+          const int i = 2 * i2;
+          const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
+          if constexpr (FOLD_SV || DEQ) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
+          else if constexpr (HOIST)
+            pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[kb][s][i], pv[i + 1] * svv[kb][s][i + 1]);
+          else
+            pop[kb][s][i >> 3][(i & 7) >> 1] =
+                pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
+          if constexpr (DEQ) {   // += the two rounded weights (one v_dot2 against a pair of ones)
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            blk = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
+                                                  __builtin_bit_cast(bf16x2_t, 0x3f803f80u), blk, false);
+          }
         }
+    };
+    if constexpr (DEQ) {
+      // The reference has to move when a logit exceeds it by 2^16.  Rather than look for the
+      // row maximum in every block (eleven instructions of sixty), the weights are computed
+      // against the reference as it stands and their sum is looked at, which the denominator
+      // needs anyway: a weight above 2^16 (or an overflow to infinity) shows in it, and the block
+      // is then redone with the reference moved.  (A sum above 2^16 without such a weight moves
+      // the reference too, which is harmless.)
+      if (first) move_reference();
+      weights();
+      if (!first && __any(!(blk <= 65536.f))) {
+        move_reference();
+        weights();
       }
+      l_part += blk;
+      first = false;
+    } else {
+      move_reference();
+      first = false;
+      weights();
+    }
     if (!DEQ && tile_rem) {
       // the remainder term must see the same bf16-rounded weights as the MFMA
 #pragma unroll
