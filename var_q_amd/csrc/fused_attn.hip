@@ -23,9 +23,11 @@
 //  * Key rows are fed to the first MFMA in a permuted order chosen so that each
 //    lane's accumulator registers hold 8 consecutive keys per 16-key chunk,
 //    which makes the V^T operand a single 16-byte LDS read.
-//  * Online softmax in the log2 domain against a reference that is only moved
-//    when some row's maximum exceeds it by 2^16: the common tile needs no
-//    subtraction and no rescale of the output accumulators.
+//  * Online softmax in the log2 domain against a reference that is only moved when a logit
+//    gets 16 octaves above the maximum it was set from, and that is found out from the weights
+//    (their sum, or the exponent bits of the packed bf16 pairs), not by a search for the row
+//    maximum: the common tile needs no maximum, no subtraction and no rescale of the output
+//    accumulators; the rare one is computed twice.
 //  * Two forms of the operands (AttnLds::kDeq says which instantiation takes which):
 //    - dequantized: (code - zp) * scale in fp32, rounded to bf16, when a tile is widened -- the
 //      operands the reference's attention sees -- and a plain bf16 flash attention behind it;
@@ -66,7 +68,7 @@ constexpr int BM = NW * 32;    // queries per workgroup (32 per wavefront)
 // other wavefronts have no queries.
 constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kRescaleAt = 16.f;   // move the softmax reference when a row max exceeds it by 2^16
+constexpr float kHeadroom = 15.f;   // exact-code kernels: octaves between a fresh softmax reference and the row maximum
 
 constexpr int kMaxSegments = 16;
 constexpr int kChanTableRows = 4;   // LDS rows per segment of the per-channel tables
@@ -958,8 +960,9 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
         zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
       }
-      if (!DEQ && !(first || __any(zmax > kRescaleAt))) return;
-      const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
+      // exact codes: the reference goes kHeadroom octaves above the maximum (see below)
+      constexpr float up = DEQ ? 0.f : kHeadroom;
+      const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax + up) : fmaxf(zmax + up, 0.f);
       const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
       m_ref += delta;
 #pragma unroll
@@ -1016,9 +1019,29 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
       l_part += blk;
       first = false;
     } else {
-      move_reference();
-      first = false;
+      // Here the denominator is summed by the MFMA, so there is no sum to look at; the packed
+      // weights themselves are: all are >= 0, so bit 14 of a bf16 (the top exponent bit) says
+      // "this weight is 2 or more" (infinities included), and an OR over the block's eight words
+      // finds one.  The reference is put kHeadroom octaves above the maximum when it moves, so
+      // weights start at 2^-kHeadroom or below -- bf16 and the fp32 sums keep their relative
+      // precision there -- and it moves again only for a logit 1 + kHeadroom octaves above that
+      // maximum.
+      if (first) move_reference();
       weights();
+      if (!first) {
+        u32 any_w = 0;
+#pragma unroll
+        for (int s = 0; s < NSVA; ++s)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) any_w |= pop[kb][s][h][j];
+        if (__any((any_w & 0x40004000u) != 0)) {
+          move_reference();
+          weights();
+        }
+      }
+      first = false;
     }
     if (!DEQ && tile_rem) {
       // the remainder term must see the same bf16-rounded weights as the MFMA
