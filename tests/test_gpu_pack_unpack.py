@@ -80,6 +80,29 @@ def test_dequant_matches_oracle(dev, bits, out_dtype):
             assert torch.equal(got8.cpu(), want.to(out_dtype)), name + ' (int8 codes)'
 
 
+@pytest.mark.parametrize('L,c,group', [(680, 64, 32), (680, 64, 64), (300, 128, 64), (257, 64, 8), (40, 64, 16),
+                                       (700, 96, 24), (700, 96, 48), (513, 128, 128), (90, 192, 32)])
+@pytest.mark.parametrize('bits', [4, 8, 2])
+def test_dequant_items_per_lane_and_group_sizes(dev, L, c, group, bits):
+    """The launch gives a lane four, two or one octets depending on how many octets a (batch,
+    head) pair has and how full its last block would be, and finds an octet's group by a shift
+    when the group is 8 times a power of two, by a division otherwise."""
+    if c % (32 // bits):
+        pytest.skip('rows of whole words only')
+    note('dequant items per lane', L, c, group, bits)
+    g = torch.Generator().manual_seed(L + c + group + bits)
+    lo, hi = O.qrange(bits)
+    q = torch.randint(lo, hi + 1, (2, 3, L, c), generator=g, dtype=torch.int8)
+    words, _ = O.pack_last_dim(q, bits)
+    s = torch.rand(2, 3, L, c // group, generator=g) + 0.01
+    z = torch.randint(-9, 9, (2, 3, L, c // group), generator=g).float()
+    want = O.dequant_groupwise(q, s, z, group)
+    got = ops.dequant(words.to(dev), s.to(dev), z.to(dev), c, bits, torch.bfloat16)
+    assert torch.equal(got.cpu(), want.to(torch.bfloat16))
+    got = ops.dequant(words.to(dev), s.to(dev), None, c, bits, torch.float32)
+    assert torch.equal(got.cpu(), O.dequant_groupwise(q, s, None, group))
+
+
 def test_dequant_ragged_channels_and_expanded_scale(dev):
     note('dequant ragged')
     g = torch.Generator().manual_seed(9)

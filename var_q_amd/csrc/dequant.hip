@@ -22,6 +22,7 @@ struct DeqParams {
   int64_t octets_per_pair;
   int c, c8, wpr, bits, group;
   int c8_shift;            // log2(c8) when c8 is a power of two, else -1
+  int g8_shift;            // log2(group / 8) when group is 8 times a power of two, else -1
 };
 
 template <int ODT> __device__ __forceinline__ void store8(void *out, int64_t elem, const float (&f)[8], int n_valid) {
@@ -115,7 +116,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(DeqParams p) {
       else if (p.bits == 8) { const int2 t = *reinterpret_cast<const int2 *>(src + col * 2); w0[u] = t.x; w1[u] = t.y; }
       else { w0[u] = src[col >> 1]; w1[u] = 0; }
       if (!chan) {
-        const int64_t g = sbase0 + i2 * p.ss2 + (col * 8 / p.group) * p.ss3;
+        const int gi = p.g8_shift >= 0 ? col >> p.g8_shift : col * 8 / p.group;   // (block-uniform choice)
+        const int64_t g = sbase0 + i2 * p.ss2 + gi * p.ss3;
         sv[u] = p.scale[g];
         zv[u] = p.zp ? p.zp[g] : 0.f;
       }
@@ -272,11 +274,19 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
   }
   p.octets_per_pair = s[2] * p.c8;
   p.c8_shift = -1;
-  for (int sh = 0; sh < 20; ++sh)
+  p.g8_shift = -1;
+  for (int sh = 0; sh < 20; ++sh) {
     if ((1 << sh) == p.c8) p.c8_shift = sh;
+    if ((8 << sh) == group) p.g8_shift = sh;
+  }
   // four items per lane where a pair has the work for it (the last block's idle lanes weigh less
   // than the wavefront turnover they save), one otherwise
-  const int U = p.octets_per_pair >= 2048 ? 4 : 1;
+  // (two where four would leave more than a twelfth of the last block's lanes idle)
+  int U = p.octets_per_pair >= 2048 ? 4 : 1;
+  if (U == 4) {
+    const int64_t t4 = (p.octets_per_pair + 1023) / 1024;
+    if ((t4 * 1024 - p.octets_per_pair) * 12 > t4 * 1024) U = 2;
+  }
   const int64_t tiles = (p.octets_per_pair + 256 * U - 1) / (256 * U);
   // a pair with few rows wastes lanes of its last block only; pairs map to grid.y/z (limit 65535 each)
   VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 1024 && s[1] <= 65535 && s[0] <= 65535, "dequant: shape exceeds the grid limits");
@@ -285,6 +295,7 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
 #define VARQ_DEQ(ODT_)                                                                       \
   do {                                                                                       \
     if (U == 4) hipLaunchKernelGGL((dequant_kernel<ODT_, 4>), grid, dim3(256), 0, st, p);    \
+    else if (U == 2) hipLaunchKernelGGL((dequant_kernel<ODT_, 2>), grid, dim3(256), 0, st, p); \
     else hipLaunchKernelGGL((dequant_kernel<ODT_, 1>), grid, dim3(256), 0, st, p);           \
   } while (0)
   if (out_dtype == VARQ_F32) VARQ_DEQ(VARQ_F32);
