@@ -281,9 +281,10 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
   }
   // four items per lane where a pair has the work for it (the last block's idle lanes weigh less
   // than the wavefront turnover they save), one otherwise
-  // (two where four would leave more than a twelfth of the last block's lanes idle)
+  // (two where four would leave more than a twelfth of the last block's lanes idle; not for
+  // per-channel tables, where a lane's pieces share one load of its eight scales and zero-points)
   int U = p.octets_per_pair >= 2048 ? 4 : 1;
-  if (U == 4) {
+  if (U == 4 && !(group == 1 && p.ss3 == 1 && p.ss2 == 0)) {
     const int64_t t4 = (p.octets_per_pair + 1023) / 1024;
     if ((t4 * 1024 - p.octets_per_pair) * 12 > t4 * 1024) U = 2;
   }
