@@ -1216,10 +1216,12 @@ template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
   if constexpr (D == 64) {
     // more (batch, head) pairs than compute units, at most four wavefronts of queries each:
-    // small workgroups, two to a compute unit (same arithmetic, same results)
+    // workgroups of four wavefronts (same arithmetic, same results).  Also for one or two
+    // wavefronts of queries: the wavefronts without queries share the staging and the widening
+    // of the tiles, which is what such a workgroup spends its time on (workgroups of two
+    // wavefronts, also two to a compute unit by their LDS, took 20-35 % longer on 16-64 queries).
     if (p.Lq <= 128 && p.bh_total > device_cus()) {
-      if (p.Lq <= 64) launch_shape<D, BITS, GK, GV, CHAN, 2>(p, st);
-      else launch_shape<D, BITS, GK, GV, CHAN, 4>(p, st);
+      launch_shape<D, BITS, GK, GV, CHAN, 4>(p, st);
       return;
     }
   }
