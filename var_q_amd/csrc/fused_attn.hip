@@ -347,6 +347,10 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   // form is faster was measured (see AttnLds::kDeq).
   constexpr bool DEQ = AttnLds<D, BITS, GK, GV, CHAN>::kDeq;
   constexpr int NSKA = DEQ ? 1 : NSK, NSVA = DEQ ? 1 : NSV;   // accumulators / weight sets
+  // (Exact codes are instantiated for one group per key only, so NSKA = NSVA = 1 in every kernel that
+  // exists; the exact-code form is nevertheless written for any group count -- its loops over
+  // groups are single passes today -- because AttnLds::kDeq is a measured choice that may move.)
+  static_assert(DEQ || (NSK == 1 && NSV == 1), "exact codes with several groups per key: AttnLds::kDeq sends those to the dequantizing form");
   static_assert(NW >= NSK && NW >= NSV && NW >= 2, "one wavefront per K group and per V group stages the parameters");
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
