@@ -60,12 +60,10 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(u32)))) u32 u32x4_t;
 
 constexpr int NW = 8;          // wavefronts per workgroup
-constexpr int NT = NW * 64;    // threads per workgroup
 constexpr int BM = NW * 32;    // queries per workgroup (32 per wavefront)
-// Smaller workgroups for launches of many (batch, head) pairs with at most 64 or 128
-// queries each (the first steps of a scale schedule at a large batch): two or four
-// wavefronts, so that two workgroups share a compute unit instead of one workgroup whose
-// other wavefronts have no queries.
+// (The D=64 kernels also exist with four wavefronts per workgroup, for launches of many (batch,
+// head) pairs with at most 128 queries each -- the first steps of a scale schedule at a large
+// batch -- see launch().)
 constexpr int BN = 64;   // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kHeadroom = 15.f;   // exact-code kernels: octaves between a fresh softmax reference and the row maximum
@@ -198,13 +196,6 @@ __device__ __forceinline__ void split3_bf16(float x, u32 &h0, u32 &h1, u32 &h2) 
   const float x1 = u2f(f2u(r1) & 0xffff0000u);
   const float x2 = r1 - x1;
   h0 = f2u(x0) >> 16; h1 = f2u(x1) >> 16; h2 = f2u(x2) >> 16;
-}
-
-// Code held in `bits` bits at `shift` of a word that was staged with the codec's xor: 4- and
-// 2-bit fields hold code + 2^(bits-1) as unsigned numbers, bytes are signed as they are.
-template <int BITS> __device__ __forceinline__ float staged_code(u32 w, int shift) {
-  if constexpr (BITS == 8) return (float)((int)(w << (24 - shift)) >> 24);
-  else return (float)((int)((w >> shift) & ((1u << BITS) - 1u)) - (1 << (BITS - 1)));
 }
 
 // MFMA row r (0..31) of the S^T block carries key kperm(r) of the 32-key block
