@@ -186,6 +186,9 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *   kv_limit   device int32 [Lq]: query i sees keys j < kv_limit[i]
  *              (block-causal next-scale mask of VAR/models/var.py:110-114,
  *              limit = end of the query's own scale); NULL = all Lk visible.
+ *              A query whose limit is 0 sees no key and gets zeros.
+ *   Lq == 0    nothing is done (q and out may be NULL then); Lq > 0 with
+ *              Lk == 0 is VARQ_ERR_INVALID (no keys to attend).
  *   layout     VARQ_LAYOUT_BHLC: the shapes above.  VARQ_LAYOUT_BLHC: q, out
  *              [B, Lq, Hq, D], words [B, Lk_stride, Hkv, D*bits/32], scales
  *              [B, Lk_stride, Hkv, D/group] -- the layout of the reference's

@@ -204,3 +204,51 @@ def test_full_size_invariants(dev):
               for t in (*kq, *vq)]
     assert torch.equal(ops.fused_attn(q, *longer, bits, bits, Lk, scale), base)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('D,bits,g', [(128, 4, 128), (64, 8, 64)])
+def test_no_queries_no_keys_and_queries_that_see_nothing(dev, D, bits, g):
+    """The corners of the entry points: a call without queries does nothing, a call with queries
+    but no keys is refused, and a query whose key limit is 0 gets zeros (its softmax has no
+    terms) while its neighbours in the same wavefront get their values; token scales and
+    per-(head, channel) tables."""
+    from var_q_amd import VarqError
+    gen = torch.Generator().manual_seed(D + bits)
+    B, H, Lq, Lk = 2, 3, 37, 70
+    k = torch.randn(B, H, Lk, D, generator=gen).bfloat16()
+    v = torch.randn(B, H, Lk, D, generator=gen).bfloat16()
+    q = torch.randn(B, H, Lq, D, generator=gen).bfloat16()
+    kw, ks, kz, kd = _quantize(k, g, bits)
+    vw, vs, vz, vd = _quantize(v, g, bits)
+    dk, dv = [t.to(dev) for t in (kw, ks, kz)], [t.to(dev) for t in (vw, vs, vz)]
+    scale = 1 / math.sqrt(D)
+    note('fused_attn: no queries')
+    out0 = ops.fused_attn(q[:, :, :0].contiguous().to(dev), *dk, *dv, bits, bits, Lk, scale)
+    torch.cuda.synchronize()
+    assert out0.shape == (B, H, 0, D)
+    note('fused_attn: no keys')
+    with pytest.raises(VarqError, match='no keys'):
+        ops.fused_attn(q.to(dev), *dk, *dv, bits, bits, 0, scale)
+    lim = torch.randint(1, Lk + 1, (Lq,), generator=gen).int()
+    lim[[0, 5, 31, 32, 36]] = 0
+    bias = torch.zeros(Lq, Lk)
+    bias[torch.arange(Lk)[None, :] >= lim[:, None].long()] = float('-inf')
+    seen = lim > 0
+    note('fused_attn: queries with key limit 0')
+    out = ops.fused_attn(q.to(dev), *dk, *dv, bits, bits, Lk, scale, kv_limit=lim.to(dev)).cpu()
+    assert float(out[:, :, ~seen].abs().max()) == 0.0
+    _compare(out[:, :, seen], O.attention_ref(q[:, :, seen], kd, vd, scale, bias[seen]),
+             O.attention_exact(q[:, :, seen].float(), kd, vd, scale, bias[seen]), 'limit 0 neighbours')
+    # the same through the per-(head, channel) tables
+    cq, cs, cz = O.quant_reduce(k, (0, 2), bits, True)
+    cvq, cvs, cvz = O.quant_reduce(v, (0, 2), bits, True)
+    ckd, cvd = O.dequant_asym(cq, cs, cz), O.dequant_asym(cvq, cvs, cvz)
+    tab = lambda t: t.reshape(H, D).contiguous().to(dev)
+    args = (O.pack_last_dim(cq, bits)[0].to(dev), tab(cs), tab(cz), O.pack_last_dim(cvq, bits)[0].to(dev), tab(cvs), tab(cvz))
+    note('fused_attn_channel: no keys, key limit 0')
+    with pytest.raises(VarqError, match='no keys'):
+        ops.fused_attn_channel(q.to(dev), *args, bits, 0, scale)
+    out = ops.fused_attn_channel(q.to(dev), *args, bits, Lk, scale, kv_limit=lim.to(dev)).cpu()
+    assert float(out[:, :, ~seen].abs().max()) == 0.0
+    _compare(out[:, :, seen], O.attention_ref(q[:, :, seen], ckd, cvd, scale, bias[seen]),
+             O.attention_exact(q[:, :, seen].float(), ckd, cvd, scale, bias[seen]), 'limit 0 neighbours, tables', oracle_bar=2e-2)

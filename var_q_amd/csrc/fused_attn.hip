@@ -1336,8 +1336,10 @@ extern "C" int varq_fused_attn(const void *q, void *out,
                                int Lq, int Lk, int Lk_stride, int D,
                                const int32_t *kv_limit, float softmax_scale, int layout,
                                void *workspace, size_t workspace_bytes, int splits, void *stream) {
-  VARQ_CHECK_ARG(q && out && k_words && v_words && k_scale && v_scale, "fused_attn: null pointer");
   VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn: bad sizes");
+  // (no queries: nothing to do, and q and out may be the null pointers of empty tensors)
+  VARQ_CHECK_ARG(Lq == 0 || (q && out), "fused_attn: null pointer");
+  VARQ_CHECK_ARG(Lq == 0 || Lk == 0 || (k_words && v_words && k_scale && v_scale), "fused_attn: null pointer");
   VARQ_CHECK_ARG(head_map || Hkv == Hq, "fused_attn: Hkv != Hq needs a head map");
   VARQ_CHECK_ARG(D == 64 || D == 128, "fused_attn: D must be 64 or 128 (got %d)", D);
   VARQ_CHECK_ARG(k_bits == 2 || k_bits == 4 || k_bits == 8, "fused_attn: bits must be 2, 4 or 8 (got %d)", k_bits);
@@ -1393,7 +1395,9 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
                                        int Lq, int Lk, int Lk_stride, int D,
                                        const int32_t *kv_limit, float softmax_scale, int layout,
                                        void *workspace, size_t workspace_bytes, int splits, void *stream) {
-  VARQ_CHECK_ARG(q && out && k_words && v_words && k_chan_scale && v_chan_scale, "fused_attn_channel: null pointer");
+  // (no queries: nothing to do, and q and out may be the null pointers of empty tensors)
+  VARQ_CHECK_ARG(Lq == 0 || (q && out), "fused_attn_channel: null pointer");
+  VARQ_CHECK_ARG(Lq == 0 || Lk == 0 || (k_words && v_words && k_chan_scale && v_chan_scale), "fused_attn_channel: null pointer");
   VARQ_CHECK_ARG(nseg >= 1 && nseg <= kMaxSegments, "fused_attn_channel: nseg must be 1..%d (got %d)", kMaxSegments, nseg);
   VARQ_CHECK_ARG(nseg == 1 || host_seg_end, "fused_attn_channel: segment ends missing");
   VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn_channel: bad sizes");
