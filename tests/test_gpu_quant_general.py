@@ -209,3 +209,15 @@ def test_two_tensors_in_the_same_launches(dev, mask):
             want = ops.quant_pack(x, dims, bits, asym=asym, pack=pack)
             assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
             assert (got[2] is None) == (want[2] is None) and (got[2] is None or torch.equal(got[2], want[2]))
+
+
+def test_empty_pair_and_empty_dequant(dev):
+    """Tensors without rows reach the library as null pointers: nothing to do, no error."""
+    note('general: empty pair, empty dequant')
+    x = torch.empty(2, 3, 0, 64, dtype=torch.bfloat16, device=dev)
+    (q0, s0, z0), (q1, s1, z1) = ops.quant_pack_pair(x, x, (0, 2), 4, asym=True)
+    assert q0.shape == (2, 3, 0, 8) and q1.shape == (2, 3, 0, 8) and s0.shape == (1, 3, 1, 64)
+    w = torch.empty(2, 3, 0, 8, dtype=torch.int32, device=dev)
+    s = torch.empty(2, 3, 0, 1, device=dev)
+    assert ops.dequant(w, s, s, 64, 4, torch.bfloat16).shape == (2, 3, 0, 64)
+    torch.cuda.synchronize()

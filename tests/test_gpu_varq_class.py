@@ -267,3 +267,29 @@ def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method):
         held.append((got, want.clone()))
     for got, want in held:
         assert torch.equal(got.cpu(), want), 'an earlier result changed'
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('method', ['G_SCALE_HEAD_DIM', 'G_TOKEN_HEAD', 'G_TOKEN'])
+def test_empty_step_is_refused_and_changes_nothing(dev, fmt, method):
+    """A step without tokens: the reference fails in its amax over an empty dim
+    (VAR_Q/quant.py:113, a RuntimeError of torch); here the quantizer says so itself, before
+    anything is launched or cached, and the next step continues where the last one ended."""
+    from var_q_amd.quant import fused_step
+    g = torch.Generator().manual_seed(11)
+    shape = (lambda n: (2, 3, n, 64)) if fmt == 'BHLc' else (lambda n: (2, n, 3, 64))
+    dim = 2 if fmt == 'BHLc' else 1
+    steps = [torch.randn(*shape(n), generator=g).bfloat16().to(dev) for n in (4, 9)]
+    empty = torch.empty(*shape(0), dtype=torch.bfloat16, device=dev)
+    note('empty step', fmt, method)
+    a, b = VAR_Q(8, fmt, method), VAR_Q(8, fmt, method)
+    with pytest.raises(RuntimeError, match='nothing to quantize'):
+        VAR_Q(8, fmt, method).use_var_q(empty)
+    r0 = a.use_var_q(steps[0])
+    b.use_var_q(steps[0])
+    with pytest.raises(RuntimeError, match='nothing to quantize'):
+        a.use_var_q(empty)
+    with pytest.raises(RuntimeError, match='nothing to quantize'):
+        fused_step(empty, empty, empty, a, VAR_Q(8, fmt, method), 0.1)
+    assert a.cached_item.size(dim) == 4 and torch.equal(a.dequant_all(), r0)
+    assert torch.equal(a.use_var_q(steps[1]), b.use_var_q(steps[1]))

@@ -247,6 +247,8 @@ extern "C" int varq_dequant(const int32_t *words, const int8_t *codes_i8, const 
   VARQ_CHECK_ARG(host_shape4 && host_scale_strides4, "dequant: null shape/strides");
   const int64_t *s = host_shape4;
   VARQ_CHECK_ARG(s[0] >= 0 && s[1] >= 0 && s[2] >= 0 && s[3] > 0 && s[3] <= (1 << 20), "dequant: bad shape");
+  // (a tensor without rows may come as null pointers: nothing to do)
+  if (s[0] * s[1] * s[2] == 0) return VARQ_OK;
   VARQ_CHECK_ARG((words != nullptr) != (codes_i8 != nullptr), "dequant: exactly one of words/codes must be given");
   VARQ_CHECK_ARG(!words || bits == 2 || bits == 4 || bits == 8, "dequant: bits must be 2, 4 or 8 (got %d)", bits);
   VARQ_CHECK_ARG(out_dtype >= 0 && out_dtype <= 2, "dequant: bad output dtype %d", out_dtype);

@@ -696,6 +696,10 @@ extern "C" int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, con
                                 int bits, int asym, float eps, int32_t *words0, int8_t *codes0, float *scale0, float *zp0,
                                 int32_t *words1, int8_t *codes1, float *scale1, float *zp1,
                                 const int64_t *host_out_map, void *workspace, size_t workspace_bytes, void *stream) {
+  // (tensors without rows may come as null pointers: nothing to do, as in varq_quant_pack)
+  if (host_shape4 && host_shape4[0] >= 0 && host_shape4[1] >= 0 && host_shape4[2] >= 0 &&
+      host_shape4[0] * host_shape4[1] * host_shape4[2] == 0 && host_shape4[3] > 0)
+    return VARQ_OK;
   VARQ_CHECK_ARG(x1, "quant_pack2: null second tensor");
   return quant_pack_impl(x0, x1, x_dtype, host_shape4, reduce_mask, bits, asym, eps, words0, codes0, scale0, zp0,
                          words1, codes1, scale1, zp1, host_out_map, workspace, workspace_bytes, stream);

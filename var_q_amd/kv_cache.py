@@ -170,7 +170,7 @@ class PackedKVCache:
     def attend(self, q: torch.Tensor, softmax_scale: float, kv_limit: Optional[torch.Tensor] = None,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fused dequant attention of q [B,H,Lq,D] (bf16) over the cached tokens."""
-        assert self.len > 0
+        assert self.len > 0, 'attend on an empty cache: append keys and values first'
         if out is None:
             out = torch.empty_like(q)
         asym = not self.symmetric

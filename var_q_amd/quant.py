@@ -240,6 +240,9 @@ class VAR_Q:
             raise ValueError(f"[VAR-Q]: Invalid quantization method: {m}")
         if self.pack_to_int32:
             assert self.quant_bits in (2, 4, 8), "bit-pack only implements 2/4/8 bits"
+        if item.numel() == 0:
+            # (the reference fails in its amax over an empty dim, VAR_Q/quant.py:113)
+            raise RuntimeError(f'[VAR-Q]: nothing to quantize: item of shape {tuple(item.shape)}')
         q, s, z = self._quantize(item)
         if self.pack_to_int32:
             c, vals = item.shape[-1], 32 // self.quant_bits
@@ -257,6 +260,8 @@ class VAR_Q:
         table row for a step of the shipped rule, nothing launched, no state changed.  None
         when the quantizer or the item is of another kind."""
         bits = self.quant_bits
+        if isinstance(x, torch.Tensor) and x.numel() == 0:
+            return None                       # (quant() says why an empty step is refused)
         if self.quant_method != 'G_SCALE_HEAD_DIM' or not self.pack_to_int32 or bits not in (2, 4, 8):
             return None
         if not isinstance(x, torch.Tensor) or x.dim() != 4 or not x.is_cuda or not x.is_contiguous() \
