@@ -892,9 +892,14 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
       wza[s] = *reinterpret_cast<const u32x4_t *>(&wz[rowsel[s] + (kb * 2 + c) * 16 + half * 8]);
   };
 
+  // A wavefront raises its priority while it issues the MFMAs of a phase.  Measured per kernel
+  // (same run, bit-identical results): at D=128 that is worth 5 % for 4-bit codes (0.725 against
+  // 0.762 ms at the configuration-4 shape) and costs 1-3.5 % for 2-bit and 8-bit codes, whose
+  // widening has more to do beside the MFMAs; at D=64 it makes no difference.
+  constexpr bool MFMA_PRIO = !(D == 128 && BITS != 4);
   // S^T = K Q^T for one 32-key block; the A operands are the widened K rows in LDS
   auto qk = [&](int kb) {
-    __builtin_amdgcn_s_setprio(1);
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(1);
     const int krow_i = kb * 32 + kperm(col);
 #pragma unroll
     for (int s = 0; s < NSKA; ++s) {
@@ -917,7 +922,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
       sacc[kb][kAcc * (ch / (GK / 16))] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
           __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][kAcc * (ch / (GK / 16))], 0, 0, 0);
     }
-    __builtin_amdgcn_s_setprio(0);
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
   };
 
   // logits -> P'^T operands of one block: online softmax against a lazily moved reference
@@ -1057,7 +1062,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   // feeds the extra block: its row s collects the zero-point sum of group s and rows
   // 4..6 (group 0 only) the softmax denominator
   auto pv_mfma = [&](int kb, bool preloaded) {
-    __builtin_amdgcn_s_setprio(1);
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       u32x4_t av[NDB], aw[NSVA];
@@ -1085,7 +1090,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
                                                        __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
       }
     }
-    __builtin_amdgcn_s_setprio(0);
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
   };
 
   for (int tile = 0; tile < n_tiles; ++tile) {
