@@ -131,11 +131,24 @@ def c5_latency(torch, dev, passes=10, warm=3):
             'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes}
 
 
+PREWARM_MS = 50.0     # 0 (--fixed-prewarm): warm up by launch count only, so that separate runs launch alike
+
+
 def timed_launches(torch, fn, reps=20, warm=5, rounds=5):
     """Seconds per call of fn: `reps` back-to-back launches between one event pair on the
-    current stream, median of `rounds` such measurements."""
-    for _ in range(warm):
-        fn()
+    current stream, median of `rounds` such measurements, after at least `warm` launches and
+    PREWARM_MS of them (the clocks of an idle GPU take tens of milliseconds to come up)."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    done = 0
+    while True:
+        for _ in range(max(warm, 5)):
+            fn()
+        done += max(warm, 5)
+        e1.record()
+        e1.synchronize()
+        if e0.elapsed_time(e1) >= PREWARM_MS or done >= 5000:
+            break
     ts = []
     for _ in range(rounds):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -413,7 +426,13 @@ def main():
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
+    ap.add_argument('--fixed-prewarm', action='store_true',
+                    help='warm the secondary legs up by launch count instead of by time, so that the launches of '
+                         'separate profiling runs can be matched by their order')
     args = ap.parse_args()
+    if args.fixed_prewarm:
+        global PREWARM_MS
+        PREWARM_MS = 0.0
     if args.gpus != 1:
         print('bench.py measures one GPU: this path has no collectives and is not sharded; '
               'run with --gpus 1 (got --gpus %d)' % args.gpus, file=sys.stderr)
