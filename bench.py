@@ -116,9 +116,7 @@ def c5_latency(torch, dev, passes=10, warm=3):
         for (q, k, v), o in zip(steps, outs):
             cache.append(k, v)
             cache.attend(q, 1.0 / math.sqrt(D5), out=o)
-    for _ in range(warm):
-        one_pass()
-    torch.cuda.synchronize()
+    warm_passes(torch, one_pass, warm)
     t0 = time.perf_counter()
     for _ in range(passes):
         one_pass()
@@ -132,6 +130,16 @@ def c5_latency(torch, dev, passes=10, warm=3):
 
 
 PREWARM_MS = 50.0     # 0 (--fixed-prewarm): warm up by launch count only, so that separate runs launch alike
+
+
+def warm_passes(torch, one_pass, warm):
+    """At least `warm` passes and PREWARM_MS of them before a pass-level timing."""
+    t0 = time.perf_counter()
+    done = 0
+    while done < warm or ((time.perf_counter() - t0) * 1e3 < PREWARM_MS and done < 1000):
+        one_pass()
+        torch.cuda.synchronize()
+        done += 1
 
 
 def timed_launches(torch, fn, reps=20, warm=5, rounds=5):
@@ -350,9 +358,7 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
 
         res = {}
         for name, fused in (('dropin_dequant_sdpa_ms', False), ('fused_ms', True)):
-            for _ in range(warm):
-                one_pass(fused)
-            torch.cuda.synchronize()
+            warm_passes(torch, lambda: one_pass(fused), warm)
             t0 = time.perf_counter()
             for _ in range(passes):
                 one_pass(fused)
@@ -368,9 +374,7 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             one_pass(True)
-        for _ in range(warm):
-            graph.replay()
-        torch.cuda.synchronize()
+        warm_passes(torch, graph.replay, warm)
         t0 = time.perf_counter()
         for _ in range(2 * passes):
             graph.replay()
