@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 6
+#define VARQ_ABI_VERSION 7
 
 enum varq_status {
   VARQ_OK = 0,
@@ -42,6 +42,22 @@ enum varq_dtype { VARQ_F32 = 0, VARQ_BF16 = 1, VARQ_F16 = 2 };
 
 /* K/V tensor layouts of the reference's quantizer (qkv_format, VAR_Q/quant.py:34-37) */
 enum varq_layout { VARQ_LAYOUT_BHLC = 0, VARQ_LAYOUT_BLHC = 1 };
+
+/*
+ * What the matrix operands of the fused attention hold.
+ * VARQ_ATTN_REFERENCE_ROUNDING (the default form): K and V are dequantized as tiles enter LDS,
+ *   (code - zp) * scale in fp32, and rounded to the attention's 16-bit type -- the very operands
+ *   the reference's attention backend sees after dequant_all() and the downcast of its call
+ *   (VAR_Q/quant.py:216-224, VAR/models/basic_var.py:158, Infinity/infinity/models/basic.py:344).
+ * VARQ_ATTN_EXACT_CODES (opt-in): the operands are exact images of the integer codes, scales
+ *   and zero-points are applied in fp32 to the products, so K and V are never rounded.  Closer
+ *   to the unrounded mathematics than the reference itself (whose bf16 rounding of K and V
+ *   moves an output by up to a few percent of its range on heavy-tailed data), hence farther
+ *   from the reference; a few percent faster.  Exists for one scale group per key of 4- or
+ *   2-bit codes at D = 128 in bf16; every other shape computes with reference rounding whatever
+ *   is asked for.
+ */
+enum varq_attn_form { VARQ_ATTN_REFERENCE_ROUNDING = 0, VARQ_ATTN_EXACT_CODES = 1 };
 
 int varq_abi_version(void);
 const char *varq_last_error(void);
@@ -105,7 +121,9 @@ int varq_quant_pack_rows2(const void *x0, const void *x1, int x_dtype, int64_t n
  *           len of a [B,H,cap,..] buffer is {n, cap - n, len}, a [B,n,H,c] step in
  *           a [B,cap,H,..] buffer {n*H, (cap - n)*H, len*H}.
  *   workspace  >= varq_quant_workspace_bytes(...) bytes, any contents
- *   scale, zp and workspace are 16-byte aligned
+ *   scale, zp and workspace are 16-byte aligned when the channel dim is kept and c is a
+ *   multiple of 8 (those kernels move eight adjacent groups' parameters in 16-byte pieces);
+ *   4-byte aligned otherwise
  * bits in 2..8 when only codes are requested, {2,4,8} when words are.
  */
 size_t varq_quant_workspace_bytes(const int64_t *host_shape4, int reduce_mask);
@@ -134,6 +152,10 @@ int varq_quant_pack2(const void *x0, const void *x1, int x_dtype, const int64_t 
  * (the six methods of VAR_Q/quant.py:75-95 need at most 8 MiB at the benchmark shapes).
  * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams,
  * two threads) race; calls ordered on one stream do not.
+ * The address of a device's copy is looked up once per device, by the first call of either
+ * function below with that device current.  That lookup is a runtime query, so it has to happen
+ * outside graph capture: call varq_quant_static_scratch_bytes() (or the entry point itself) once
+ * on each device before capturing.  Recorded into a graph, the entry point is kernel launches only.
  */
 #define VARQ_STATIC_SCRATCH_BYTES (16u << 20)
 size_t varq_quant_static_scratch_bytes(void);
@@ -176,7 +198,13 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *   out[b,h,i,:] = softmax_j( softmax_scale * q[b,h,i,:] . K[b,h,j,:] + mask(i,j) ) V[b,h,j,:]
  *   K = (k_codes - k_zp) * k_scale,  V likewise, never materialized.
  *
- *   q, out     bf16 [B, Hq, Lq, D]
+ *   q, out     [B, Hq, Lq, D] of io_dtype: VARQ_BF16 (the Infinity path, bf16 autocast:
+ *              Infinity/tools/run_infinity.py:519) or VARQ_F16 (the VAR path, fp16 autocast:
+ *              scripts/inference_multi_VAR.py:123, VAR/models/basic_var.py:157-158).  It is
+ *              also the type dequantized K and V are rounded to and the type of the MFMA
+ *              operands; accumulation is fp32 either way.  VARQ_F16 needs D = 64 (the head
+ *              dim of every VAR model).
+ *   operand_form  one of varq_attn_form (above)
  *   k_words    int32 [B, Hkv, Lk_stride, D*k_bits/32]; only rows < Lk are read
  *   k_scale/zp fp32  [B, Hkv, Lk_stride, D/k_group]   (zp NULL = symmetric)
  *   v_*        same for V
@@ -214,7 +242,7 @@ int varq_fused_attn(const void *q, void *out,
                     const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                     int B, int Hq, int Hkv, const int32_t *head_map,
                     int Lq, int Lk, int Lk_stride, int D,
-                    const int32_t *kv_limit, float softmax_scale, int layout,
+                    const int32_t *kv_limit, float softmax_scale, int layout, int io_dtype, int operand_form,
                     void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*
@@ -234,8 +262,9 @@ int varq_fused_attn(const void *q, void *out,
  *                        every logit of a query by the same amount, which the softmax cancels
  *                        (K is then offset per channel before it is rounded to bf16)
  * K and V are dequantized with the tables of each key's segment as tiles enter LDS,
- * (code - zp) * scale in fp32 rounded to bf16: the operands of the reference's attention
- * after dequant_all (VAR_Q/quant.py:216-224) and its bf16 attention call.
+ * (code - zp) * scale in fp32 rounded to io_dtype (bf16 or fp16, as in varq_fused_attn): the
+ * operands of the reference's attention after dequant_all (VAR_Q/quant.py:216-224) and the
+ * downcast of its attention call.
  *   nseg, host_seg_end   1..16 segments; host int32 [nseg] (may be NULL when nseg == 1)
  *   everything else as in varq_fused_attn; one bit-width for K and V.
  */
@@ -245,7 +274,7 @@ int varq_fused_attn_channel(const void *q, void *out,
                             int nseg, const int32_t *host_seg_end,
                             int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                             int Lq, int Lk, int Lk_stride, int D,
-                            const int32_t *kv_limit, float softmax_scale, int layout,
+                            const int32_t *kv_limit, float softmax_scale, int layout, int io_dtype,
                             void *workspace, size_t workspace_bytes, int splits, void *stream);
 
 /*

@@ -25,7 +25,7 @@ def test_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
     assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
-    assert lib.varq_abi_version() == _lib.ABI_VERSION == 6
+    assert lib.varq_abi_version() == _lib.ABI_VERSION == 7
 
 
 def test_invalid_arguments_are_rejected_on_the_host():
@@ -62,14 +62,20 @@ def test_invalid_arguments_are_rejected_on_the_host():
     rc = lib.varq_quant_pack_static(fake, 0, i64([8, 4096, 16, 128]), 0b0001, 8, 0, 1e-12, fake, None, fake, None, None, None)
     assert rc == -4 and b'static' in lib.varq_last_error()
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128,
-                             1, 2, 2, None, 16, 16, 16, 96, None, 1.0, 0, None, 0, 0, None)
+                             1, 2, 2, None, 16, 16, 16, 96, None, 1.0, 0, 1, 0, None, 0, 0, None)
     assert rc == -1 and b'D must be' in lib.varq_last_error()
     rc = lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 8, 128,
-                             1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, None, 0, 0, None)
+                             1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, 1, 0, None, 0, 0, None)
     assert rc == -2
+    # the type of q / out and the operand form: fp32 queries, an unknown form, fp16 at head dim 128
+    dt = lambda io, form, D=128: lib.varq_fused_attn(fake, fake, fake, fake, fake, 4, D, fake, fake, fake, 4, D,
+                                                     1, 2, 2, None, 16, 16, 16, D, None, 1.0, 0, io, form, None, 0, 0, None)
+    assert dt(0, 0) == -1 and b'io_dtype' in lib.varq_last_error()
+    assert dt(1, 2) == -1 and b'operand_form' in lib.varq_last_error()
+    assert dt(2, 0) == -2 and b'fp16' in lib.varq_last_error()
     # keys shared out over workgroups: the split count and its workspace are checked first
     tok = lambda splits, ws=None, nbytes=0: lib.varq_fused_attn(
-        fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128, 1, 2, 2, None, 16, 640, 640, 128, None, 1.0, 0,
+        fake, fake, fake, fake, fake, 4, 128, fake, fake, fake, 4, 128, 1, 2, 2, None, 16, 640, 640, 128, None, 1.0, 0, 1, 0,
         ws, nbytes, splits, None)
     assert tok(9) == -1 and b'splits' in lib.varq_last_error()
     assert tok(2) == -1 and b'workspace' in lib.varq_last_error()
@@ -85,7 +91,7 @@ def test_invalid_arguments_are_rejected_on_the_host():
     # per-channel attention: segment table checks
     i32 = lambda v: (ctypes.c_int32 * len(v))(*v)
     chan = lambda nseg, ends, Lk=16, D=128: lib.varq_fused_attn_channel(
-        fake, fake, fake, fake, None, fake, fake, None, nseg, ends, 8, 1, 2, 2, None, 16, Lk, 16, D, None, 1.0, 0, None, 0, 0, None)
+        fake, fake, fake, fake, None, fake, fake, None, nseg, ends, 8, 1, 2, 2, None, 16, Lk, 16, D, None, 1.0, 0, 1, None, 0, 0, None)
     assert chan(0, None) == -1 and b'nseg' in lib.varq_last_error()
     assert chan(17, None) == -1 and b'nseg' in lib.varq_last_error()
     assert chan(2, None) == -1 and b'segment ends missing' in lib.varq_last_error()
@@ -93,8 +99,11 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert chan(2, i32([40, 16])) == -1 and b'beyond' in lib.varq_last_error()
     assert chan(1, None, D=96) == -1 and b'D must be' in lib.varq_last_error()
     rc = lib.varq_fused_attn_channel(fake, fake, fake, ctypes.c_void_p(0x1004), None, fake, fake, None, 1, None,
-                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, None, 0, 0, None)
+                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, 1, None, 0, 0, None)
     assert rc == -1 and b'aligned' in lib.varq_last_error()
+    rc = lib.varq_fused_attn_channel(fake, fake, fake, fake, None, fake, fake, None, 1, None,
+                                     8, 1, 2, 2, None, 16, 16, 16, 128, None, 1.0, 0, 2, None, 0, 0, None)
+    assert rc == -2 and b'fp16' in lib.varq_last_error()
     # empty inputs are a no-op success
     assert chan(1, None, Lk=0) == -1          # queries but no keys
     assert lib.varq_pack(None, 0, 16, 4, None, None) == 0

@@ -10,9 +10,10 @@ the keys shared between workgroups.
 The yardstick.  At +-100 octaves the softmax is so sharp that rounding the dequantized K to bf16
 (what the reference's attention and the oracle do) moves a logit by up to 100 * 2^-9 = 0.2 octaves
 and the oracle's output by 0.1-0.2 from the fp64 value of the unrounded operands.  The
-dequantizing kernels round the same way and are held to the oracle as in test_gpu_attention.py;
-the exact-code kernels do not round and land within 1e-2 of the fp64 value instead.  A result
-passes when it is within the tolerance of either: cosine >= 0.9995 and max-abs <= 2e-2 x range
+dequantizing kernels (the default form) round the same way and are held to the oracle as in
+test_gpu_attention.py; the exact-code kernels (`exact_codes=True`) do not round and land within
+1e-2 of the fp64 value instead.  This file tests the softmax bookkeeping, not parity: a result
+passes when it is within the tolerance of either, cosine >= 0.9995 and max-abs <= 2e-2 x range
 against the fp64 value, or test_gpu_attention.py's comparison with the oracle."""
 import math
 
@@ -29,7 +30,7 @@ pytestmark = pytest.mark.gpu
 LQ, LK = 70, 300
 
 
-def _check(out, ref, exact, what):
+def _check(out, ref, exact, what, exact_codes=False):
     o, e = out.double().cpu(), exact.double()
     span = max(1.0, float(e.abs().max()))
     err = float((o - e).abs().max())
@@ -38,7 +39,7 @@ def _check(out, ref, exact, what):
     if err <= 2e-2 * span and cos >= 0.9995:
         print(f'[attn] {what}: range {span:.3g}  kernel-fp64 {err:.4g}  cosine {cos:.6f}', flush=True)
         return
-    _compare(out, ref, exact, what)
+    _compare(out, ref, exact, what, exact_codes=exact_codes)
 
 
 def _profile(name):
@@ -82,10 +83,12 @@ def _limit(kind, seed):
 
 
 @pytest.mark.parametrize('prof', ['up', 'down', 'step', 'saw', 'late'])
-@pytest.mark.parametrize('D,bits,gk,gv', [(128, 4, 128, 128), (128, 2, 128, 128), (128, 8, 128, 128), (128, 4, 64, 64), (128, 2, 32, 32),
-                                          (64, 4, 64, 64), (64, 8, 32, 32)])
+@pytest.mark.parametrize('D,bits,gk,gv,exact_codes',
+                         [(128, 4, 128, 128, True), (128, 2, 128, 128, True), (128, 4, 128, 128, False), (128, 2, 128, 128, False),
+                          (128, 8, 128, 128, False), (128, 4, 64, 64, False), (128, 2, 32, 32, False), (64, 4, 64, 64, False),
+                          (64, 8, 32, 32, False)])
 @pytest.mark.parametrize('splits,limit', [(0, 'all'), (3, 'limit')])
-def test_token_scales(dev, prof, D, bits, gk, gv, splits, limit):
+def test_token_scales(dev, prof, D, bits, gk, gv, exact_codes, splits, limit):
     q, k, v = _data(D, prof, 17 * D + bits)
     lim, bias = _limit(limit, 5 + bits)
     kq, ks, kz = O.quant_groupwise(k, gk, bits, True)
@@ -95,10 +98,11 @@ def test_token_scales(dev, prof, D, bits, gk, gv, splits, limit):
     note('softmax range, token scales', prof, D, bits, gk, gv, splits, limit)
     put = lambda t: None if t is None else t.to(dev)
     out = ops.fused_attn(put(q), put(O.pack_last_dim(kq, bits)[0]), put(ks), put(kz), put(O.pack_last_dim(vq, bits)[0]), put(vs),
-                         put(vz), bits, bits, LK, scale, kv_limit=put(lim), splits=splits)
+                         put(vz), bits, bits, LK, scale, kv_limit=put(lim), splits=splits, exact_codes=exact_codes)
     torch.cuda.synchronize()
     _check(out, O.attention_ref(q, kd, vd, scale, bias), O.attention_exact(q.float(), kd, vd, scale, bias),
-           f'softmax range {prof} D={D} int{bits} g{gk}/{gv} splits={splits} {limit}')
+           f'softmax range {prof} D={D} int{bits} g{gk}/{gv} splits={splits} {limit}' + (' exact codes' if exact_codes else ''),
+           exact_codes)
 
 
 @pytest.mark.parametrize('prof', ['up', 'down', 'step', 'saw', 'late'])

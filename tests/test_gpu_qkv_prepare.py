@@ -106,3 +106,29 @@ def test_cache_append_from_qkv_mixed_bits(dev):
         assert torch.equal(q_gpu.cpu().view(torch.int16), q_ref.view(torch.int16))
     assert a.len == b.len == 21
     assert torch.equal(a.dequant('k'), b.dequant('k')) and torch.equal(a.dequant('v'), b.dequant('v'))
+
+
+@pytest.mark.parametrize('bits', [8, 4])
+def test_zero_points_around_the_rounding_shortcuts_limit(dev, bits):
+    """v is quantized as it comes (no norm, no rotation): rows of integers offset by about 2^21
+    and 2^22 quantization steps put the zero-point on either side of the limit up to which the
+    kernel rounds by adding 1.5 * 2^23; beyond it the division path must take over."""
+    B, L, H, c = 1, 26, 1, 64
+    qkv = torch.zeros(B, L, 3, H, c)
+    bases = (2 ** 21 - 300, 2 ** 21 - 128, 2 ** 21 - 1, 2 ** 21, 2 ** 21 + 200, 2 ** 22 - 400, 2 ** 22 - 256,
+             2 ** 22 - 130, 2 ** 22 - 128, 2 ** 22 - 1, 2 ** 22, 2 ** 22 + 300, 2 ** 23 - 256)
+    k = torch.arange(c, dtype=torch.float32) * 255 // (c - 1)
+    for i, base in enumerate(bases):
+        qkv[0, 2 * i, 2, 0] = k + float(base)
+        qkv[0, 2 * i + 1, 2, 0] = -(k + float(base))
+    qkv[:, :, :2] = torch.randn(B, L, 2, H, c, generator=torch.Generator().manual_seed(4))
+    _, _, v_ref = O.prepare_qkv(qkv, None, False)
+    W = c * bits // 32
+    kw, vw = (torch.zeros(B, H, L, W, dtype=torch.int32, device=dev) for _ in range(2))
+    ks, kz, vs, vz = (torch.zeros(B, H, L, 1, device=dev) for _ in range(4))
+    q_out = torch.empty(B, H, L, c, dtype=torch.bfloat16, device=dev)
+    note('qkv_prepare zero-point limit', bits)
+    ops.qkv_prepare_append(qkv.to(dev), q_out, c, bits, True, 1e-12, kw, ks, kz, vw, vs, vz, [B, L, H, H * L, 1, L, 0, -1])
+    cq, cs, cz = O.quant_groupwise(v_ref, c, bits, True)
+    assert torch.equal(vs.cpu(), cs) and torch.equal(vz.cpu(), cz)
+    assert torch.equal(vw.cpu(), O.pack_last_dim(cq, bits)[0])

@@ -189,3 +189,23 @@ def test_pair_launch_equals_two_launches(dev, bits, group, asym, dtype):
         if x is not None:
             assert torch.equal(x, y)
     assert not torch.equal(a_k[0], a_v[0])        # the two tensors did differ
+
+
+def _offset_rows(c):
+    """fp32 rows of integers base .. base+255 (scale 1 for 8-bit affine codes), with bases that put
+    the zero-point on either side of 2^21 and 2^22: the kernel's rounding shortcut needs the
+    clamped quotient, up to 128 beyond the zero-point, inside +-2^22."""
+    rows = []
+    for base in (2 ** 21 - 300, 2 ** 21 - 128, 2 ** 21 - 1, 2 ** 21, 2 ** 21 + 200, 2 ** 22 - 400, 2 ** 22 - 256,
+                 2 ** 22 - 130, 2 ** 22 - 128, 2 ** 22 - 1, 2 ** 22, 2 ** 22 + 300, 2 ** 23 - 256):
+        for sign in (1.0, -1.0):
+            k = torch.arange(c, dtype=torch.float32) * 255 // (c - 1)
+            rows.append(sign * (k + float(base)) if sign > 0 else -(k + float(base)))
+    return torch.stack(rows)
+
+
+@pytest.mark.parametrize('bits', [8, 4, 2])
+@pytest.mark.parametrize('c,group', [(128, 128), (64, 64), (64, 32)])
+def test_zero_points_around_the_rounding_shortcuts_limit(dev, bits, c, group):
+    note('quant_rows zero-point limit', bits, c, group)
+    _check(_offset_rows(c), group, bits, True, dev)

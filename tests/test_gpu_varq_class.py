@@ -248,12 +248,15 @@ def test_layout_change_with_cached_steps_is_refused(dev):
 
 @pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
 @pytest.mark.parametrize('method', ['G_SCALE_HEAD_DIM', 'G_TOKEN', 'G_HEAD_DIM', 'G_TENSOR'])
-def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method):
-    """use_var_q dequantizes only the new step and keeps the earlier values; calls of quant() and
-    cache() on their own in between (the fused path makes them) must not leave it with stale
-    values, and a result handed out earlier must not change when later steps arrive."""
-    note('VAR_Q incremental dequant', fmt, method)
-    ref, gpu = O.OracleVARQ(8, fmt, method), VAR_Q(8, fmt, method)
+@pytest.mark.parametrize('keep', [True, False])
+def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method, keep):
+    """With keep_dequantized=True use_var_q dequantizes only the new step and keeps the earlier
+    values; calls of quant() and cache() on their own in between (the fused path makes them) must
+    not leave it with stale values, and a result handed out earlier must not change when later
+    steps arrive.  Without the flag (the default) nothing is kept and every call returns a fresh
+    tensor, like the reference."""
+    note('VAR_Q incremental dequant', fmt, method, keep)
+    ref, gpu = O.OracleVARQ(8, fmt, method), VAR_Q(8, fmt, method, keep_dequantized=keep)
     steps = _steps(fmt, torch.float32, seed=77) + _steps(fmt, torch.float32, seed=78)
     held = []
     for i, x in enumerate(steps):
@@ -265,6 +268,8 @@ def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method):
         assert got.shape == want.shape and torch.equal(got.cpu(), want), f'step {i}'
         assert torch.equal(gpu.dequant_all().cpu(), want), f'step {i}: dequant_all'
         held.append((got, want.clone()))
+        if not keep:
+            assert gpu._c_deq.buf is None, 'the default keeps no dequantized copy of the cache'
     for got, want in held:
         assert torch.equal(got.cpu(), want), 'an earlier result changed'
 
@@ -293,3 +298,18 @@ def test_empty_step_is_refused_and_changes_nothing(dev, fmt, method):
         fused_step(empty, empty, empty, a, VAR_Q(8, fmt, method), 0.1)
     assert a.cached_item.size(dim) == 4 and torch.equal(a.dequant_all(), r0)
     assert torch.equal(a.use_var_q(steps[1]), b.use_var_q(steps[1]))
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('bits,pack', [(8, True), (8, False), (5, False)])
+def test_table_rows_off_a_16_byte_boundary(dev, fmt, bits, pack):
+    """H * c not a multiple of four: the rows of the per-step scale table behind the first are
+    not 16-byte aligned (H=3, c=30: row 1 starts at byte 360).  Such a shape takes the kernels
+    that move one parameter at a time, which need no such alignment; every step must work and
+    match the oracle."""
+    note('VAR_Q odd table rows', fmt, bits, pack)
+    ref, gpu = O.OracleVARQ(bits, fmt, 'G_SCALE_HEAD_DIM', pack_to_int32=pack), VAR_Q(bits, fmt, 'G_SCALE_HEAD_DIM', pack_to_int32=pack)
+    for i, x in enumerate(_steps(fmt, torch.float32, seed=5, H=3, c=30)):
+        want, got = ref.use_var_q(x), gpu.use_var_q(x.to(dev))
+        assert torch.equal(got.cpu(), want), f'step {i}'
+        assert torch.equal(gpu.scale.cpu(), ref.scale) and torch.equal(gpu.cached_item.cpu(), ref.cached_item)

@@ -81,3 +81,46 @@ def test_static_scratch_rejects_what_does_not_fit(dev):
     rc = lib.varq_quant_pack_static(x.data_ptr(), 0, sh, 0b0001, 8, 0, 1e-12, x.data_ptr(), None, x.data_ptr(), None,
                                     None, None)
     assert rc == -4 and b'static' in lib.varq_last_error()
+
+
+def test_static_entry_recorded_into_a_graph(dev):
+    """The entry point under HIP graph capture, its named use: the scratch address is looked up
+    by the warm-up call before the capture, the capture records kernel launches only, and every
+    replay on new input equals the eager result bit for bit."""
+    lib = _lib.load()
+    assert lib.varq_quant_static_scratch_bytes() >= (8 << 20)      # the warm-up call, outside capture
+    B, H, L, c, bits, mask = 2, 6, 77, 64, 4, 0b0101
+    gen = torch.Generator(device=dev).manual_seed(17)
+    x = torch.randn(B, H, L, c, device=dev, generator=gen).bfloat16()
+    sh = _lib.i64arr([B, H, L, c])
+    words = torch.zeros(B, H, L, c * bits // 32, dtype=torch.int32, device=dev)
+    scale, zp = torch.zeros(1, H, 1, c, device=dev), torch.zeros(1, H, 1, c, device=dev)
+
+    def run(stream):
+        _lib.check(lib.varq_quant_pack_static(x.data_ptr(), 1, sh, mask, bits, 1, 1e-12, words.data_ptr(), None,
+                                              scale.data_ptr(), zp.data_ptr(), None, stream), 'varq_quant_pack_static')
+
+    note('no-alloc graph: warm-up on a side stream')
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    note('no-alloc graph: capture')
+    with torch.cuda.graph(graph):
+        run(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.normal_(generator=gen)
+        note('no-alloc graph: eager', rep)
+        run(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want = [t.clone() for t in (words, scale, zp)]
+        for t in (words, scale, zp):
+            t.zero_()
+        note('no-alloc graph: replay', rep)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(want, (words, scale, zp)):
+            assert torch.equal(a, b), f'replay {rep}: the graph and the eager call differ'

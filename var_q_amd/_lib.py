@@ -7,7 +7,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, 'libvarq_hip.so')
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 SYMBOLS = {
     'varq_abi_version': (c_int, []),
@@ -35,7 +35,7 @@ SYMBOLS = {
                                 c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p,
                                 c_int, c_int, c_int, c_int,
-                                c_void_p, c_float, c_int, c_void_p, c_size_t, c_int, c_void_p]),
+                                c_void_p, c_float, c_int, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p]),
     'varq_fused_attn_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     'varq_fused_attn_channel': (c_int, [c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p,
@@ -43,7 +43,7 @@ SYMBOLS = {
                                         c_int, POINTER(c_int32),
                                         c_int, c_int, c_int, c_int, c_void_p,
                                         c_int, c_int, c_int, c_int,
-                                        c_void_p, c_float, c_int, c_void_p, c_size_t, c_int, c_void_p]),
+                                        c_void_p, c_float, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p]),
     'varq_qkv_prepare_append': (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_int, c_float,
                                         c_void_p, c_void_p, c_int,

@@ -28,12 +28,11 @@
 //    (their sum, or the exponent bits of the packed bf16 pairs), not by a search for the row
 //    maximum: the common tile needs no maximum, no subtraction and no rescale of the output
 //    accumulators; the rare one is computed twice.
-//  * Two forms of the operands (AttnLds::kDeq says which instantiation takes which):
-//    - dequantized: (code - zp) * scale in fp32, rounded to bf16, when a tile is widened -- the
-//      operands the reference's attention sees -- and a plain bf16 flash attention behind it;
-//      per-(head, channel) tables that change along the keys, several groups per key, every
-//      kernel at head dim 64 and the 8-bit kernels at head dim 128;
-//    - exact codes (one group per key of 4- or 2-bit codes at head dim 128): the MFMA operands
+//  * Two forms of the operands:
+//    - dequantized (the default of every kernel): (code - zp) * scale in fp32, rounded to the
+//      attention's 16-bit type (bf16, or fp16 for the VAR path) when a tile is widened -- the
+//      operands the reference's attention sees -- and a plain flash attention behind it;
+//    - exact codes (opt-in; one group per key of 4- or 2-bit codes at head dim 128, bf16): the MFMA operands
 //      are exact small numbers derived from the codes, never scaled or rounded.  A code lands in
 //      the top mantissa bits of a bf16 1.x (raw = (code + kOff) / kMul), which costs one shift and
 //      one and-or per two elements.  Scales are applied in fp32, zero-points ride on extra MFMA
@@ -94,6 +93,9 @@ struct AttnParams {
   // workspace, the output is written directly.
   int nsplit;
   float *ws_o, *ws_ml;
+  // the caller asked for exact codes in the MFMA operands where such a kernel exists (host side only)
+  int exact_codes;
+  int f16;   // q, out and the MFMA operands are fp16 (host side only: it selects the instantiation)
   // memory layout, in rows (a row = the D values of one token of one head):
   // q/out row = b*q_bs + h*q_hs + i*q_ts, key row = b*kv_bs + slot*kv_hs + j*kv_ts.
   // BHLc: (H*L, L, 1); BLHc (the layout of the flash-attention call): (L*H, 1, H).
@@ -187,6 +189,27 @@ __device__ __forceinline__ u32 pack_bf16_rne(float lo, float hi) {
   f2 v = {lo, hi};
   bf2 b = __builtin_convertvector(v, bf2);
   return __builtin_bit_cast(u32, b);
+}
+__device__ __forceinline__ u32 pack_f16_rne(float lo, float hi) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 v = {lo, hi};
+  h2 b = __builtin_convertvector(v, h2);
+  return __builtin_bit_cast(u32, b);
+}
+// two fp32 values rounded to nearest-even into a pair of the attention's 16-bit type
+template <bool F16> __device__ __forceinline__ u32 pack_io_rne(float lo, float hi) {
+  if constexpr (F16) return pack_f16_rne(lo, hi);
+  else return pack_bf16_rne(lo, hi);
+}
+// D (32x32 fp32) += A (32x16) B (16x32), operands in the attention's 16-bit type
+template <bool F16> __device__ __forceinline__ floatx16_t mfma_32x32x16(u32x4_t a, u32x4_t b, floatx16_t c) {
+  if constexpr (F16) {
+    typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
 }
 // x = h0 + h1 + h2 exactly, each piece a bf16 (returned as its 16 bits): three
 // 8-bit slices of the 24-bit significand
@@ -290,12 +313,17 @@ template <int G> __device__ __forceinline__ int k_octet(int ch, int h) {
 }
 
 // LDS layout of the attention kernel (bytes), shared by kernel and launcher.
-// kDeq: the kernel dequantizes when a tile is widened (see the kernel) and has no rank-1 operands:
-// per-channel tables, more than one K or V group per key, and -- by measurement -- every kernel
-// at D=64 and the 8-bit kernels at D=128.  Exact codes in the MFMA operands remain where they are
-// the faster form: one group per key of 4- or 2-bit codes at D=128 (configuration 4).
-template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
-  static constexpr bool kDeq = CHAN || (D / GK > 1 || D / GV > 1) || D == 64 || BITS == 8;
+// kDeq: the kernel dequantizes when a tile is widened (see the kernel) and has no rank-1 operands.
+// That is the form of every kernel unless the caller asks for exact codes (EXACT), which exist
+// where they were measured to be the faster form: one group per key of 4- or 2-bit codes at
+// D=128.  (Per-channel tables, more than one K or V group per key, every kernel at D=64 and the
+// 8-bit kernels at D=128 are faster dequantizing, and have no exact-code instantiation.)
+template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnForms {
+  static constexpr bool kHasExact = !CHAN && D / GK == 1 && D / GV == 1 && D == 128 && BITS != 8;
+};
+template <int D, int BITS, int GK, int GV, bool CHAN, bool EXACT = false> struct AttnLds {
+  static_assert(!EXACT || AttnForms<D, BITS, GK, GV, CHAN>::kHasExact, "no exact-code form of this kernel");
+  static constexpr bool kDeq = !EXACT;
   static constexpr int WPR = D * BITS / 32;
   static constexpr int RSV = WPR + 1;       // packed V row stride (words): odd, bank spread
   static constexpr bool kFoldSv = !kDeq && (D / GV == 1);   // one V group: its scale rides inside the logits
@@ -322,8 +350,12 @@ template <int D, int BITS, int GK, int GV, bool CHAN> struct AttnLds {
 // that knows nothing of tables or segments.
 // WPS: wavefronts per SIMD the register allocation aims at (2, or 4: two 8-wavefront workgroups
 // per compute unit at 128 registers, which the D=64 kernels that dequantize afford)
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8, int WPS = 2>
+// F16: q, out and the MFMA operands are fp16 instead of bf16 (dequantized K and V are rounded to
+// fp16, as the reference's fp16 attention call sees them: VAR/models/basic_var.py:157-158 under the
+// fp16 autocast of scripts/inference_multi_VAR.py:123); dequantizing kernels only.
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV = 8, int WPS = 2, bool EXACT = false, bool F16 = false>
 __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p) {
+  static_assert(!(F16 && EXACT), "the exact-code form builds bf16 images of the codes");
   static_assert(!CHAN || (GK == D && GV == D), "per-channel tables go with the single-group kernels");
   constexpr int NW = NWV, NT = NWV * 64, BM = NWV * 32;   // (shadow the defaults of the file)
   constexpr int NSK = D / GK, NSV = D / GV;
@@ -335,19 +367,19 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   // V groups per key, exact codes in the MFMAs would need one logit accumulator and one rank-1
   // MFMA per K group and one set of weights and one extra MFMA per V group (19 -> 28 MFMAs per
   // key block at four groups, and registers that do not exist); where there is one group, which
-  // form is faster was measured (see AttnLds::kDeq).
-  constexpr bool DEQ = AttnLds<D, BITS, GK, GV, CHAN>::kDeq;
+  // form is faster was measured (see AttnForms).
+  constexpr bool DEQ = AttnLds<D, BITS, GK, GV, CHAN, EXACT>::kDeq;
   constexpr int NSKA = DEQ ? 1 : NSK, NSVA = DEQ ? 1 : NSV;   // accumulators / weight sets
   // (Exact codes are instantiated for one group per key only, so NSKA = NSVA = 1 in every kernel that
   // exists; the exact-code form is nevertheless written for any group count -- its loops over
-  // groups are single passes today -- because AttnLds::kDeq is a measured choice that may move.)
-  static_assert(DEQ || (NSK == 1 && NSV == 1), "exact codes with several groups per key: AttnLds::kDeq sends those to the dequantizing form");
+  // groups are single passes today -- because AttnForms::kHasExact is a measured choice that may move.)
+  static_assert(DEQ || (NSK == 1 && NSV == 1), "exact codes with several groups per key: AttnForms sends those to the dequantizing form");
   static_assert(NW >= NSK && NW >= NSV && NW >= 2, "one wavefront per K group and per V group stages the parameters");
   constexpr int WPR = D * BITS / 32;        // packed words per key row
   constexpr int NCH = D / 16;               // contraction chunks of QK^T
   constexpr int NDB = D / 32;               // 32-row blocks of O^T
   constexpr int VTS = BN + 8;               // V^T row stride (bf16 elements)
-  using L = AttnLds<D, BITS, GK, GV, CHAN>;
+  using L = AttnLds<D, BITS, GK, GV, CHAN, EXACT>;
 
   // Pipelined LDS buffers (one workgroup barrier per tile):
   //   packed V and the per-key parameters of tile t live in slot t % 3, the
@@ -711,18 +743,18 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         const float s0[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w}, z0[8] = {za.x, za.y, za.z, za.w, zb.x, zb.y, zb.z, zb.w};
         if (one_seg || sg1 == sg0) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z0[j]) * s0[j], (f1[j] - z0[j]) * s0[j]);
+          for (int j = 0; j < 8; ++j) pr[j] = pack_io_rne<F16>((f0[j] - z0[j]) * s0[j], (f1[j] - z0[j]) * s0[j]);
         } else {
           const float *t1s = lds_tab + (sg1 * TR + 2) * D + oct * 8;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z0[j]) * s0[j], (f1[j] - t1s[D + j]) * t1s[j]);
+          for (int j = 0; j < 8; ++j) pr[j] = pack_io_rne<F16>((f0[j] - z0[j]) * s0[j], (f1[j] - t1s[D + j]) * t1s[j]);
         }
       } else if constexpr (DEQ) {
         // code images -> values of the two keys, (raw - z') * s' in fp32, rounded to bf16
         const float *pt = lds_par + (tile % 3) * L::kParFloats + (oct * 8 / GV) * BN + kp2 * 2;
         const float2 z2 = *reinterpret_cast<const float2 *>(pt + P_VZ), s2 = *reinterpret_cast<const float2 *>(pt + P_SV);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) pr[j] = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
+        for (int j = 0; j < 8; ++j) pr[j] = pack_io_rne<F16>((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * VTS + kp2 * 2]) = pr[j];
@@ -764,7 +796,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
             const float sc[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w}, zc[8] = {za.x, za.y, za.z, za.w, zb.x, zb.y, zb.z, zb.w};
 #pragma unroll
             for (int m = 0; m < 4; ++m)
-              a[m] = pack_bf16_rne((f[2 * m] - zc[2 * m]) * sc[2 * m], (f[2 * m + 1] - zc[2 * m + 1]) * sc[2 * m + 1]);
+              a[m] = pack_io_rne<F16>((f[2 * m] - zc[2 * m]) * sc[2 * m], (f[2 * m + 1] - zc[2 * m + 1]) * sc[2 * m + 1]);
           } else if constexpr (DEQ) {
             // code images -> values: (raw - (zp + kOff) / kMul) * (kMul * ks), the reference's
             // (code - zp) * scale with both factors rescaled exactly, rounded to bf16
@@ -772,7 +804,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
             const float zk = (kgz[i * GPP + gl] + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul);
             const float sk = kgs[i * GPP + gl] * KCodec<BITS>::kMul;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((f[2 * m] - zk) * sk, (f[2 * m + 1] - zk) * sk);
+            for (int m = 0; m < 4; ++m) a[m] = pack_io_rne<F16>((f[2 * m] - zk) * sk, (f[2 * m + 1] - zk) * sk);
           }
           *reinterpret_cast<u32x4_t *>(&kx[key * KXS + (oct0 + j) * 8]) = u32x4_t{a[0], a[1], a[2], a[3]};
         }
@@ -910,8 +942,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         sacc[kb][s] = zero;   // (dequantized operands: no zero-point term)
       } else {
         // starts the accumulator with the zero-point term (see bq above)
-        sacc[kb][s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kz[(s * BN + krow_i) * 2 + half]),
-                                                              __builtin_bit_cast(bf16x8_t, bq[s]), zero, 0, 0, 0);
+        sacc[kb][s] = mfma_32x32x16<F16>(kz[(s * BN + krow_i) * 2 + half], bq[s], zero);
       }
     }
     const uint16_t *krow = &kx[krow_i * KXS];
@@ -919,8 +950,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
     for (int ch = 0; ch < NCH; ++ch) {
       const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&krow[k_octet<GK>(ch, half) * 8]);
       constexpr int kAcc = DEQ ? 0 : 1;
-      sacc[kb][kAcc * (ch / (GK / 16))] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-          __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, qb[ch]), sacc[kb][kAcc * (ch / (GK / 16))], 0, 0, 0);
+      sacc[kb][kAcc * (ch / (GK / 16))] = mfma_32x32x16<F16>(av, qb[ch], sacc[kb][kAcc * (ch / (GK / 16))]);
     }
     if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
   };
@@ -990,16 +1020,22 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         for (int i2 = 0; i2 < 8; ++i2) {
           const int i = 2 * i2;
           const int key = kb * 32 + 16 * (i >> 3) + 8 * half + (i & 7);
-          if constexpr (FOLD_SV || DEQ) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i], pv[i + 1]);
+          if constexpr (FOLD_SV || DEQ) pop[kb][s][i >> 3][(i & 7) >> 1] = pack_io_rne<F16>(pv[i], pv[i + 1]);
           else if constexpr (HOIST)
             pop[kb][s][i >> 3][(i & 7) >> 1] = pack_bf16_rne(pv[i] * svv[kb][s][i], pv[i + 1] * svv[kb][s][i + 1]);
           else
             pop[kb][s][i >> 3][(i & 7) >> 1] =
                 pack_bf16_rne(pv[i] * par[P_SV + s * BN + key], pv[i + 1] * par[P_SV + s * BN + key + 1]);
           if constexpr (DEQ) {   // += the two rounded weights (one v_dot2 against a pair of ones)
-            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-            blk = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
-                                                  __builtin_bit_cast(bf16x2_t, 0x3f803f80u), blk, false);
+            if constexpr (F16) {
+              typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+              blk = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
+                                           __builtin_bit_cast(f16x2_t, 0x3c003c00u), blk, false);
+            } else {
+              typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+              blk = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pop[kb][s][i >> 3][(i & 7) >> 1]),
+                                                    __builtin_bit_cast(bf16x2_t, 0x3f803f80u), blk, false);
+            }
           }
         }
     };
@@ -1012,7 +1048,10 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
       // the reference too, which is harmless.)
       if (first) move_reference();
       weights();
-      if (!first && __any(!(blk <= 65536.f))) {
+      // (fp16 weights end at 65504: there the reference moves at a block sum of 2^15, which keeps
+      // every weight of an accepted block finite; an overflowed one makes the sum infinite)
+      constexpr float kMoveAt = F16 ? 32768.f : 65536.f;
+      if (!first && __any(!(blk <= kMoveAt))) {
         move_reference();
         weights();
       }
@@ -1080,14 +1119,12 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         constexpr int DBS = GV / 32;  // 32-row blocks per V scale group
         const int s = DEQ ? 0 : d / DBS;
         u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
-        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[d]),
-                                                          __builtin_bit_cast(bf16x8_t, bv), oacc[d], 0, 0, 0);
+        oacc[d] = mfma_32x32x16<F16>(av[d], bv, oacc[d]);
       }
 #pragma unroll
       for (int s = 0; s < (DEQ ? 0 : NSVA); ++s) {
         u32x4_t bv = {pop[kb][s][c][0], pop[kb][s][c][1], pop[kb][s][c][2], pop[kb][s][c][3]};
-        racc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, aw[s]),
-                                                       __builtin_bit_cast(bf16x8_t, bv), racc, 0, 0, 0);
+        racc = mfma_32x32x16<F16>(aw[s], bv, racc);
       }
     }
     if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
@@ -1145,7 +1182,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
         if (shared_out) {
           *reinterpret_cast<float4 *>(wptr + d * 32 + 8 * g4 + 4 * half) = make_float4(o0, o1, o2, o3);
         } else {
-          uint2 v = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
+          uint2 v = make_uint2(pack_io_rne<F16>(o0, o1), pack_io_rne<F16>(o2, o3));
           *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = v;
         }
       }
@@ -1155,7 +1192,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 
 // One thread per (query row, four channels): the shares' outputs weighted by their softmax
 // mass l * 2^(m - M), M the largest reference among the shares that saw a key.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
   const int64_t rows = (int64_t)p.bh_total * p.Lq;
   const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1182,15 +1219,15 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
   const int hq = p.head_map ? p.head_map[hs] : hs;
   __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D + c0;
-  *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_bf16_rne(acc[0] * inv, acc[1] * inv), pack_bf16_rne(acc[2] * inv, acc[3] * inv));
+  *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_io_rne<F16>(acc[0] * inv, acc[1] * inv), pack_io_rne<F16>(acc[2] * inv, acc[3] * inv));
 }
 
 int device_cus();
 
-template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, int WPS = 2>
+template <int D, int BITS, int GK, int GV, bool CHAN, int NWV, int WPS = 2, bool EXACT = false, bool F16 = false>
 void launch_shape(const AttnParams &p, hipStream_t st) {
   // (the per-channel tables take LDS by the number of segments of the launch)
-  constexpr int lds_base = (AttnLds<D, BITS, GK, GV, CHAN>::kBytes + 15) / 16 * 16, lds_seg = CHAN ? kChanTableRows * D * 4 : 0;
+  constexpr int lds_base = (AttnLds<D, BITS, GK, GV, CHAN, EXACT>::kBytes + 15) / 16 * 16, lds_seg = CHAN ? kChanTableRows * D * 4 : 0;
   constexpr int lds_max = lds_base + kMaxSegments * lds_seg;
   static_assert(lds_max <= 160 * 1024, "LDS budget");
   const int lds_bytes = lds_base + p.nseg * lds_seg;
@@ -1199,21 +1236,29 @@ void launch_shape(const AttnParams &p, hipStream_t st) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
   if (dev < 0 || !configured[dev]) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS, EXACT, F16>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);
     if (dev >= 0) configured[dev] = true;
   }
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
-  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS>), grid, dim3(NWV * 64), lds_bytes, st, p);
+  hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS, EXACT, F16>), grid, dim3(NWV * 64), lds_bytes, st, p);
   if (p.nsplit > 1) {
     const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
-    hipLaunchKernelGGL((combine_splits_kernel<D>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((combine_splits_kernel<D, F16>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
   }
 }
 
 template <int D, int BITS, int GK, int GV, bool CHAN = false>
 void launch(const AttnParams &p, hipStream_t st) {
+  if constexpr (D == 64) {
+    // fp16 operands (the VAR path; every VAR model has head dim 64)
+    if (p.f16) {
+      if (p.Lq <= 128 && p.bh_total > device_cus()) launch_shape<D, BITS, GK, GV, CHAN, 4, 2, false, true>(p, st);
+      else launch_shape<D, BITS, GK, GV, CHAN, 8, 4, false, true>(p, st);
+      return;
+    }
+  }
   if constexpr (D == 64) {
     // more (batch, head) pairs than compute units, at most four wavefronts of queries each:
     // workgroups of four wavefronts (same arithmetic, same results).  Also for one or two
@@ -1225,12 +1270,18 @@ void launch(const AttnParams &p, hipStream_t st) {
       return;
     }
   }
-  if constexpr (D == 64 && AttnLds<D, BITS, GK, GV, CHAN>::kDeq) {
-    // The dequantizing kernels at D=64 fit 128 registers at the price of 24-48 bytes of spills,
+  if constexpr (D == 64) {
+    // The kernels at D=64 fit 128 registers at the price of 24-48 bytes of spills,
     // and two resident workgroups per compute unit hide each other's prologue and barriers
     // (8-15 % faster than one workgroup at 140 registers).
     launch_shape<D, BITS, GK, GV, CHAN, 8, 4>(p, st);
   } else {
+    if constexpr (AttnForms<D, BITS, GK, GV, CHAN>::kHasExact) {
+      if (p.exact_codes) {
+        launch_shape<D, BITS, GK, GV, CHAN, 8, 2, true>(p, st);
+        return;
+      }
+    }
     launch_shape<D, BITS, GK, GV, CHAN, 8>(p, st);
   }
 }
@@ -1339,9 +1390,14 @@ extern "C" int varq_fused_attn(const void *q, void *out,
                                const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,
                                int B, int Hq, int Hkv, const int32_t *head_map,
                                int Lq, int Lk, int Lk_stride, int D,
-                               const int32_t *kv_limit, float softmax_scale, int layout,
+                               const int32_t *kv_limit, float softmax_scale, int layout, int io_dtype, int operand_form,
                                void *workspace, size_t workspace_bytes, int splits, void *stream) {
   VARQ_CHECK_ARG(B > 0 && Hq > 0 && Hkv > 0 && Lq >= 0 && Lk >= 0 && Lk_stride >= Lk, "fused_attn: bad sizes");
+  VARQ_CHECK_ARG(io_dtype == VARQ_BF16 || io_dtype == VARQ_F16, "fused_attn: io_dtype must be VARQ_BF16 (1) or VARQ_F16 (2), got %d", io_dtype);
+  VARQ_CHECK_ARG(operand_form == VARQ_ATTN_REFERENCE_ROUNDING || operand_form == VARQ_ATTN_EXACT_CODES,
+                 "fused_attn: operand_form must be 0 (reference rounding) or 1 (exact codes), got %d", operand_form);
+  if (io_dtype == VARQ_F16 && D != 64)
+    return varq_set_error(VARQ_ERR_UNSUPPORTED, "fused_attn: fp16 queries need D = 64 (got %d); D = 128 is served in bf16", D);
   // (no queries: nothing to do, and q and out may be the null pointers of empty tensors)
   VARQ_CHECK_ARG(Lq == 0 || (q && out), "fused_attn: null pointer");
   VARQ_CHECK_ARG(Lq == 0 || Lk == 0 || (k_words && v_words && k_scale && v_scale), "fused_attn: null pointer");
@@ -1372,6 +1428,8 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  p.f16 = io_dtype == VARQ_F16;
+  p.exact_codes = operand_form == VARQ_ATTN_EXACT_CODES && !p.f16;
   if (int e = set_layout(p, layout, "fused_attn")) return e;
   if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn")) return e;
   hipStream_t st = (hipStream_t)stream;
@@ -1398,8 +1456,11 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
                                        int nseg, const int32_t *host_seg_end,
                                        int bits, int B, int Hq, int Hkv, const int32_t *head_map,
                                        int Lq, int Lk, int Lk_stride, int D,
-                                       const int32_t *kv_limit, float softmax_scale, int layout,
+                                       const int32_t *kv_limit, float softmax_scale, int layout, int io_dtype,
                                        void *workspace, size_t workspace_bytes, int splits, void *stream) {
+  VARQ_CHECK_ARG(io_dtype == VARQ_BF16 || io_dtype == VARQ_F16, "fused_attn_channel: io_dtype must be VARQ_BF16 (1) or VARQ_F16 (2), got %d", io_dtype);
+  if (io_dtype == VARQ_F16 && D != 64)
+    return varq_set_error(VARQ_ERR_UNSUPPORTED, "fused_attn_channel: fp16 queries need D = 64 (got %d); D = 128 is served in bf16", D);
   // (no queries: nothing to do, and q and out may be the null pointers of empty tensors)
   VARQ_CHECK_ARG(Lq == 0 || (q && out), "fused_attn_channel: null pointer");
   VARQ_CHECK_ARG(Lq == 0 || Lk == 0 || (k_words && v_words && k_chan_scale && v_chan_scale), "fused_attn_channel: null pointer");
@@ -1442,6 +1503,8 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
   p.scale_log2e = softmax_scale * kLog2e;
+  p.f16 = io_dtype == VARQ_F16;
+  p.exact_codes = 0;
   if (int e = set_layout(p, layout, "fused_attn_channel")) return e;
   if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn_channel"))
     return e;

@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     vz = group_zp<BITS, ASYM>(vmn, vs, vr, wave_plain);
   }
   u32 kw0, kw1, vw0, vw1;
-  const bool fast = wave_plain && __builtin_amdgcn_ballot_w64(!(fabsf(kz) <= 0x1p22f && fabsf(vz) <= 0x1p22f)) == 0;
+  const bool fast = wave_plain && __builtin_amdgcn_ballot_w64(!(fabsf(kz) <= 0x1p21f && fabsf(vz) <= 0x1p21f)) == 0;
   pack_octet<BITS, ASYM>(k, ks, kr, kz, fast, kw0, kw1);
   pack_octet<BITS, ASYM>(v, vs, vr, vz, fast, vw0, vw1);
 

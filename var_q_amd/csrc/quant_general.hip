@@ -631,8 +631,11 @@ int quant_pack_impl(const void *x, const void *x1, int x_dtype, const int64_t *h
   if (workspace_bytes < need)
     return varq_set_error(VARQ_ERR_WORKSPACE, "quant_pack: workspace %zu < %zu bytes", workspace_bytes, need);
   VARQ_CHECK_ARG(rows * s[3] < (1ll << 40), "quant_pack: tensor too large");
-  VARQ_CHECK_ARG((((uintptr_t)workspace | (uintptr_t)scale | (uintptr_t)zp | (uintptr_t)scale1 | (uintptr_t)zp1) & 15) == 0,
-                 "quant_pack: scale, zp and workspace must be 16-byte aligned");
+  // only the tiled kernels that keep the channel dim move scales, zero-points and partials in
+  // 16-byte pieces; every other path reads and writes them one word at a time
+  const uintptr_t par_align = (tiled && !(reduce_mask & 8)) ? 15 : 3;
+  VARQ_CHECK_ARG((((uintptr_t)workspace | (uintptr_t)scale | (uintptr_t)zp | (uintptr_t)scale1 | (uintptr_t)zp1) & par_align) == 0,
+                 "quant_pack: scale, zp and workspace must be %d-byte aligned for this shape", (int)par_align + 1);
 
   GenParams p;
   p.x = x;
@@ -736,7 +739,14 @@ int scratch_for_current_device(void **out) {
 }
 }  // namespace
 
-extern "C" size_t varq_quant_static_scratch_bytes(void) { return (size_t)VARQ_STATIC_SCRATCH_BYTES; }
+// Also the warm-up call: it looks the current device's copy of the array up (a runtime query that
+// must not happen while a stream is being captured into a graph), so that the entry point below
+// finds the address already there.  Without a usable device it only reports the size.
+extern "C" size_t varq_quant_static_scratch_bytes(void) {
+  void *ws = nullptr;
+  (void)scratch_for_current_device(&ws);
+  return (size_t)VARQ_STATIC_SCRATCH_BYTES;
+}
 
 extern "C" int varq_quant_pack_static(const void *x, int x_dtype, const int64_t *host_shape4, int reduce_mask, int bits,
                                       int asym, float eps, int32_t *words, int8_t *codes, float *scale, float *zp,

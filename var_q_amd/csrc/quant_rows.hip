@@ -244,7 +244,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   // e = x - q0*s is exact in one fma, and RN(q0 + e*r) is the correctly rounded
   // quotient (Markstein's correction step).  That holds for every finite x unless
   // the significand of s is all ones or the residual can underflow; such groups,
-  // and zero-points beyond 2^22, take the fp64 route below.
+  // and zero-points beyond 2^21 (the clamped quotient, up to 128 beyond the zero-point, must stay
+  // inside +-2^22 for the rounding trick below), take the fp64 route below.
   const float r = 1.0f / s;
   const bool plain = s > 0x1p-96f && s < 0x1p96f && (f2u(s) & 0x7fffffu) != 0x7fffffu;
   auto quotient = [&](float x) {
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   };
   const bool wave_plain = __builtin_amdgcn_ballot_w64(!plain) == 0;
   if (ASYM) zp = kMin - rintf(wave_plain ? quotient(mn) : mn / s);
-  const bool big_zp = ASYM && !(fabsf(zp) <= 0x1p22f);
+  const bool big_zp = ASYM && !(fabsf(zp) <= 0x1p21f);
 
   // Codes: clamp(rint(t) + zp, qmin, qmax) = rint(clamp(t, qmin - zp, qmax - zp)) + zp
   // (the bounds are integers).  Adding 1.5 * 2^23 rounds the clamped quotient to

@@ -164,6 +164,11 @@ class _QuantizedSelfAttention(nn.Module):
         o = self.packed_cache.attend(q, scale)                                          # [B,H,L,c]
         return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(x.dtype)
 
+    def _attn_dtype(self, main_type):
+        """dtype of the fused attention: the module's compute dtype where the kernels have it
+        (fp16 at head dim 64, the VAR models), bf16 otherwise."""
+        return torch.float16 if (main_type == torch.float16 and self.head_dim == 64) else torch.bfloat16
+
     def _cache_and_attend(self, q, k, v, scale: float, attn_bias, out_dtype):
         B = q.shape[0]
         l_dim = 1 if self.layout == 'BLHc' else 2
@@ -171,7 +176,9 @@ class _QuantizedSelfAttention(nn.Module):
         if self.caching and self.fused == 'quantizer':
             if attn_bias is not None:
                 raise ValueError('the fused backend takes the mask as a key limit per query, not as a bias tensor')
-            o = fused_step(q, k, v, self.k_quant, self.v_quant, scale)                    # in the layout of q
+            # the attention runs in the module's compute dtype, like the reference's call
+            # (q.to(dtype=main_type), VAR/models/basic_var.py:158): fp16 for VAR, bf16 for Infinity
+            o = fused_step(q.to(self._attn_dtype(out_dtype)), k, v, self.k_quant, self.v_quant, scale)   # in the layout of q
             if self.layout == 'BHLc':
                 o = o.transpose(1, 2)
             return o.reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
@@ -183,7 +190,7 @@ class _QuantizedSelfAttention(nn.Module):
                                                   self.group_size, q.device, symmetric=self.symmetric)
             self.packed_cache.append(k, v, layout=self.layout)
             qh = q if self.layout == 'BHLc' else q.transpose(1, 2)
-            o = self.packed_cache.attend(qh.to(torch.bfloat16).contiguous(), scale)       # [B,H,L,c]
+            o = self.packed_cache.attend(qh.to(self._attn_dtype(out_dtype)).contiguous(), scale)   # [B,H,L,c]
             return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
         if self.caching:
             if self.enable_quantization:

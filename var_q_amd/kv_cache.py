@@ -168,8 +168,10 @@ class PackedKVCache:
         return q_out
 
     def attend(self, q: torch.Tensor, softmax_scale: float, kv_limit: Optional[torch.Tensor] = None,
-               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Fused dequant attention of q [B,H,Lq,D] (bf16) over the cached tokens."""
+               out: Optional[torch.Tensor] = None, exact_codes: bool = False) -> torch.Tensor:
+        """Fused dequant attention of q [B,H,Lq,D] (bf16; fp16 at D=64) over the cached tokens.
+        K and V enter the products rounded to q's dtype, as in the reference; exact_codes=True
+        selects the form that does not round them where it exists (see ops.fused_attn)."""
         assert self.len > 0, 'attend on an empty cache: append keys and values first'
         if out is None:
             out = torch.empty_like(q)
@@ -190,7 +192,7 @@ class PackedKVCache:
                                c.v_words, c.v_scale, c.v_zp if asym else None,
                                c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
                                head_map=c.head_map if many else None, out=out,
-                               splits=1 if side else self.splits)   # classes side by side fill the device already
+                               splits=1 if side else self.splits, exact_codes=exact_codes)   # classes side by side fill the device already
             if stream is not main:
                 self._join[i - 1].record(stream)
                 main.wait_event(self._join[i - 1])

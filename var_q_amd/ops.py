@@ -355,6 +355,8 @@ def qkv_prepare_append(qkv: torch.Tensor, q_out: torch.Tensor, group: int, bits:
 # fused dequant flash-attention
 # ---------------------------------------------------------------------------
 _LAYOUTS = {'BHLc': 0, 'BLHc': 1}
+# dtypes of q / out (the library's dtype codes): bf16 everywhere, fp16 for head dim 64 (the VAR path)
+_ATTN_DT = {torch.bfloat16: 1, torch.float16: 2}
 
 
 def _attn_dims(q, k_words, layout):
@@ -383,10 +385,16 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
                v_words: torch.Tensor, v_scale: torch.Tensor, v_zp: Optional[torch.Tensor],
                k_bits: int, v_bits: int, Lk: int, softmax_scale: float,
                kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
-               out: Optional[torch.Tensor] = None, splits: int = 0, layout: str = 'BHLc') -> torch.Tensor:
-    """q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32;
+               out: Optional[torch.Tensor] = None, splits: int = 0, layout: str = 'BHLc',
+               exact_codes: bool = False) -> torch.Tensor:
+    """q [B,Hq,Lq,D] bf16 (or fp16 at D=64, the VAR path); k/v_words [B,Hkv,Lstride,D*bits/32] int32;
     k/v_scale (zp) [B,Hkv,Lstride,D/group] fp32; attends keys 0..Lk-1.
-    Returns out [B,Hq,Lq,D] bf16 (rows of heads not in head_map are untouched).
+    Returns out [B,Hq,Lq,D] of q's dtype (rows of heads not in head_map are untouched).
+    K and V enter the matrix products dequantized and rounded to q's dtype, as the reference's
+    attention sees them.  exact_codes=True asks for the form that never rounds K and V (exact
+    code images in the products, scales applied in fp32): closer to the unrounded mathematics,
+    farther from the reference, a few percent faster; it exists for 4- and 2-bit codes with one
+    group per key at D=128 in bf16 and is ignored elsewhere.
     layout 'BLHc': every tensor has tokens before heads instead ([B,Lq,Hq,D], [B,Lstride,Hkv,...]),
     the layout of the reference's flash-attention call.
     splits: over how many workgroups the keys of a query block are shared out (0: the
@@ -394,7 +402,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_scale, 'k_scale'), (v_scale, 'v_scale')):
         _gpu(t, n)
         assert t.is_contiguous(), f'{n} must be contiguous'
-    assert q.dtype == torch.bfloat16 and q.dim() == 4
+    assert q.dtype in _ATTN_DT and q.dim() == 4, 'q must be bf16 or fp16'
     B, Hq, Lq, D, Hkv, Lstride, Wk = _attn_dims(q, k_words, layout)
     assert v_words.shape[:3] == k_words.shape[:3]
     assert Wk * 32 == D * k_bits and v_words.shape[3] * 32 == D * v_bits
@@ -402,6 +410,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     k_group, v_group = D // k_scale.shape[3], D // v_scale.shape[3]
     if out is None:
         out = torch.empty_like(q)
+    assert out.dtype == q.dtype, 'out must have the dtype of q'
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
@@ -417,7 +426,8 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
                                   k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp), k_bits, k_group,
                                   v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), v_bits, v_group,
                                   B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                  _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ptr(ws), ws_bytes,
+                                  _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ATTN_DT[q.dtype],
+                                  int(bool(exact_codes)), _ptr(ws), ws_bytes,
                                   int(splits), _stream(q)), 'varq_fused_attn')
     return out
 
@@ -432,7 +442,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
     """Attention over a cache quantized per (head, channel): the scale layout of the
     reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
     (G_TENSOR, G_SCALE) expanded to the table, and the affine per-head-per-dim variant.
-    q [B,Hq,Lq,D] bf16; k/v_words [B,Hkv,Lstride,D*bits/32] int32; k_chan_scale,
+    q [B,Hq,Lq,D] bf16 (or fp16 at D=64); k/v_words [B,Hkv,Lstride,D*bits/32] int32; k_chan_scale,
     v_chan_scale, v_chan_zp fp32 with at least nseg*Hkv*D elements (any shape that flattens to
     [>= nseg, Hkv, D]).  seg_ends (at most 16 increasing key counts, the last one = Lk) says
     where the tables change along the keys: a cache filled step by step by the reference's
@@ -443,7 +453,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                  (v_chan_scale, 'v_chan_scale')):
         _gpu(t, n)
         assert t.is_contiguous(), f'{n} must be contiguous'
-    assert q.dtype == torch.bfloat16 and q.dim() == 4
+    assert q.dtype in _ATTN_DT and q.dim() == 4, 'q must be bf16 or fp16'
     B, Hq, Lq, D, Hkv, Lstride, W = _attn_dims(q, k_words, layout)
     assert v_words.shape == k_words.shape and W * 32 == D * bits
     nseg = 1 if seg_ends is None else len(seg_ends)
@@ -459,6 +469,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                 f'{n} must be fp32 [nseg, Hkv, D] (more tables than segments are allowed)'
     if out is None:
         out = torch.empty_like(q)
+    assert out.dtype == q.dtype, 'out must have the dtype of q'
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
@@ -474,6 +485,6 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                                           k_words.data_ptr(), k_chan_scale.data_ptr(), _ptr(k_chan_zp),
                                           v_words.data_ptr(), v_chan_scale.data_ptr(), _ptr(v_chan_zp),
                                           nseg, ends, bits, B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                          _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ptr(ws), ws_bytes,
-                                          int(splits), _stream(q)), 'varq_fused_attn_channel')
+                                          _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ATTN_DT[q.dtype],
+                                          _ptr(ws), ws_bytes, int(splits), _stream(q)), 'varq_fused_attn_channel')
     return out

@@ -110,7 +110,7 @@ class _Growable:
 class VAR_Q:
     def __init__(self, quant_bits: int = 8, qkv_format: str = 'BLHc', quant_method: str = 'G_SCALE_HEAD_DIM',
                  blk_idx: int = 0, pack_to_int32: bool = True, eps: float = 1e-12, debug: bool = False,
-                 symmetric: bool = True, group_size: Optional[int] = None):
+                 symmetric: bool = True, group_size: Optional[int] = None, keep_dequantized: bool = False):
         assert qkv_format in ('BLHc', 'BHLc'), f"Invalid qkv_format: {qkv_format}"
         assert quant_method in _REF_METHODS + _EXT_METHODS, f"Invalid quant_method: {quant_method}"
         assert 1 < quant_bits <= 8, "Only support (2..8] bits (common 2/4/8 bits); bit-pack implementation covers 2/4/8 bits"
@@ -125,6 +125,9 @@ class VAR_Q:
         self.debug = debug
         self.symmetric = symmetric
         self.group_size = group_size
+        # use_var_q keeps the fp32 values it handed out from step to step (see use_var_q): faster,
+        # and 4 bytes per cached element resident for the life of the quantizer.  Off unless asked for.
+        self.keep_dequantized = keep_dequantized
         self.qkv_format = qkv_format   # property: also derives dim_cat / dim_map
         self.bound_min = -(2 ** (quant_bits - 1))
         self.bound_max = (2 ** (quant_bits - 1)) - 1
@@ -448,15 +451,22 @@ class VAR_Q:
         return self._dequant(self.cached_item, self.cached_scale, self.cached_zp)
 
     def use_var_q(self, item: torch.Tensor) -> torch.Tensor:
-        """quant + cache + dequant_all (VAR_Q/quant.py:226-230).  The reference dequantizes the whole
-        cache at every step; under the appending methods the codes and scales of earlier steps never
-        change, so their fp32 values are kept from step to step and only the new step is
-        dequantized and put behind them: the same values (the step's scale is what the expanded
-        cached scale holds for its tokens), O(step) instead of O(cache) per call.  The result is the
-        valid prefix of that buffer (like `cached_item`, a view that is not contiguous when the
-        buffer has room to spare).  `dequant_all()` itself still recomputes everything."""
+        """quant + cache + dequant_all (VAR_Q/quant.py:226-230).  Like the reference, the whole
+        cache is dequantized into a fresh fp32 tensor at every step and nothing of it is kept.
+
+        With `keep_dequantized=True` (constructor) the fp32 values are kept from step to step
+        instead: under the appending methods the codes and scales of earlier steps never change,
+        so only the new step is dequantized and put behind them -- the same values (the step's
+        scale is what the expanded cached scale holds for its tokens), O(step) instead of
+        O(cache) per call.  The result is then the valid prefix of that buffer (like
+        `cached_item`, a view that is not contiguous when the buffer has room to spare).  The
+        price is memory: 4 bytes per cached element (up to 8 while the buffer has doubled), i.e.
+        two to four times an unquantized bf16 cache, resident until the quantizer is deleted --
+        172 MB per tensor at [2,16,10521,128].  `dequant_all()` itself always recomputes everything."""
         self.quant(item)
         self.cache()
+        if not self.keep_dequantized:
+            return self.dequant_all()
         d, n = self._c_deq, self.quantized_item.size(self.dim_cat)
         if self.quant_method == 'G_HEAD_DIM' or self._c_item.buf is None or d.dim != self.dim_cat or d.len + n != self._c_item.len:
             # (the replacing method; or the kept values are not those of the cache's earlier steps:
@@ -504,14 +514,18 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     Infinity/infinity/models/basic.py:339-351).
 
     q [B,H,Lq,c] for quantizers in layout 'BHLc', [B,Lq,H,c] for 'BLHc' (the layout of the
-    reference's flash-attention call and of VAR-VAR_Q-8.json), cast to bf16; both quantizers in
+    reference's flash-attention call and of VAR-VAR_Q-8.json).  The attention runs in q's dtype
+    when that is fp16 and c = 64 -- the VAR path, whose attention call casts q, k and v to fp16
+    (VAR/models/basic_var.py:157-158 under the fp16 autocast of scripts/inference_multi_VAR.py:123)
+    -- and in bf16 otherwise (q is cast); dequantized K and V are rounded to that type, as the
+    reference's downcast does.  Both quantizers in
     the same layout, packed, same bit-width, c in {64, 128}, after at least one `cache()`.  Methods whose scale is shared by the
     tokens of a step (G_SCALE_HEAD_DIM -- the shipped rule --, G_HEAD_DIM, G_TENSOR, G_SCALE,
     G_HEAD) go through one table per cached step, at most MAX_TABLE_STEPS steps; per-token
     methods (G_TOKEN, G_TOKEN_HEAD, G_GROUP) through per-token scales.  Everything the
     kernels read is kept current by `cache()`, so a call launches the attention and nothing
-    else.  kv_limit: int32 [Lq], query i sees keys j < kv_limit[i].  Returns bf16
-    in the shape of q."""
+    else.  kv_limit: int32 [Lq], query i sees keys j < kv_limit[i].  Returns a tensor of the
+    attention's dtype in the shape of q."""
     layout = k_quant.qkv_format
     if v_quant.qkv_format != layout:
         raise ValueError(f'fused_attention: K is cached in layout {layout}, V in {v_quant.qkv_format}')
@@ -530,7 +544,7 @@ def fused_attention(q: torch.Tensor, k_quant: VAR_Q, v_quant: VAR_Q, softmax_sca
     c = k_quant._pack_meta['orig_c']
     if c not in (64, 128):
         raise ValueError(f'fused_attention: head dim {c} not supported (64 or 128)')
-    q = q.to(torch.bfloat16).contiguous()
+    q = (q if (q.dtype == torch.float16 and c == 64) else q.to(torch.bfloat16)).contiguous()
     assert q.dim() == 4 and q.shape[0] == B and q.shape[1 if bhl else 2] == H and q.shape[3] == c, \
         'q must be [B,H,Lq,c] (BHLc) or [B,Lq,H,c] (BLHc)'
     km, vm = k_quant.quant_method, v_quant.quant_method
