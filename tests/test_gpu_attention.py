@@ -278,3 +278,72 @@ def test_no_queries_no_keys_and_queries_that_see_nothing(dev, D, bits, g):
     assert float(out[:, :, ~seen].abs().max()) == 0.0
     _compare(out[:, :, seen], O.attention_ref(q[:, :, seen], ckd, cvd, scale, bias[seen]),
              O.attention_exact(q[:, :, seen].float(), ckd, cvd, scale, bias[seen]), 'limit 0 neighbours, tables', oracle_bar=2e-2)
+
+
+@pytest.mark.parametrize('bits', [4, 8, 2])
+@pytest.mark.parametrize('gk,gv', [(64, 64), (32, 64), (32, 32)])
+def test_fp16_operands_head_dim_64(dev, bits, gk, gv):
+    """fp16 q / out and fp16 MFMA operands (dequantized K and V rounded to fp16), the dtype of the
+    reference's VAR attention call (VAR/models/basic_var.py:157-158 under the fp16 autocast of
+    scripts/inference_multi_VAR.py:123), against the oracle's attention in fp16: token scales in
+    one launch of 8-wavefront workgroups and, with many (batch, head) pairs of few queries, of
+    4-wavefront ones; per-(head, channel) tables with three segments; keys shared out; a key limit."""
+    D, scale = 64, 1.0 / 8
+    for B, H, Lq, Lk, splits in ((2, 3, 200, 333, 0), (40, 8, 36, 91, 0), (1, 2, 150, 700, 3)):
+        g = torch.Generator().manual_seed(bits * 100 + gk + Lq)
+        k = O.synth_kv((B, H, Lk, D), 11 + bits, 'student4').half()
+        v = O.synth_kv((B, H, Lk, D), 12 + bits, 'student4').half()
+        q = torch.randn(B, H, Lq, D, generator=g).half()
+        lim = torch.randint(1, Lk + 1, (Lq,), generator=g).int()
+        bias = torch.zeros(Lq, Lk)
+        bias[torch.arange(Lk)[None, :] >= lim[:, None].long()] = float('-inf')
+        kw, ks, kz, kd = _quantize(k, gk, bits)
+        vw, vs, vz, vd = _quantize(v, gv, bits)
+        note('fused_attn fp16', (B, H, Lq, Lk), bits, gk, gv, splits)
+        args = [t.to(dev) for t in (kw, ks, kz, vw, vs, vz)]
+        out = ops.fused_attn(q.to(dev), *args, bits, bits, Lk, scale, kv_limit=lim.to(dev), splits=splits)
+        assert out.dtype == torch.float16
+        if B * H < 64:
+            _compare(out, O.attention_ref(q, kd, vd, scale, bias, dtype=torch.float16), O.attention_exact(q.float(), kd, vd, scale, bias),
+                     f'fp16 int{bits} g{gk}/{gv} {Lq}x{Lk}')
+        else:   # (the oracle on a sample of the pairs)
+            for b in (0, B - 1):
+                _compare(out[b:b + 1], O.attention_ref(q[b:b + 1], kd[b:b + 1], vd[b:b + 1], scale, bias, dtype=torch.float16),
+                         O.attention_exact(q[b:b + 1].float(), kd[b:b + 1], vd[b:b + 1], scale, bias), f'fp16 int{bits} small workgroups, entry {b}')
+
+
+@pytest.mark.parametrize('bits,asym', [(8, False), (4, True), (2, True)])
+def test_fp16_operands_channel_tables(dev, bits, asym):
+    D, H, Lq, scale = 64, 3, 100, 1.0 / 8
+    cuts = [40, 113, 300]
+    g = torch.Generator().manual_seed(bits)
+    q = torch.randn(2, H, Lq, D, generator=g).half()
+    per = []
+    for seed in (21, 22):
+        x = O.synth_kv((2, H, cuts[-1], D), seed + bits).half()
+        ws, ds, ss, zs, a = [], [], [], [], 0
+        for e in cuts:
+            cq, s, z = O.quant_reduce(x[:, :, a:e], (0, 2), bits, asym)
+            ws.append(O.pack_last_dim(cq, bits)[0])
+            ds.append(O.dequant_asym(cq, s, z) if asym else O.dequant_sym(cq, s))
+            ss.append(s.reshape(H, D))
+            zs.append(None if z is None else z.reshape(H, D))
+            a = e
+        per.append((torch.cat(ws, 2).contiguous(), torch.stack(ss).contiguous(), torch.stack(zs).contiguous() if asym else None, torch.cat(ds, 2)))
+    (kw, ks, kz, kd), (vw, vs, vz, vd) = per
+    put = lambda t: None if t is None else t.to(dev)
+    note('fused_attn_channel fp16', bits, asym)
+    out = ops.fused_attn_channel(put(q), put(kw), put(ks), put(kz), put(vw), put(vs), put(vz), bits, cuts[-1], scale, seg_ends=cuts)
+    assert out.dtype == torch.float16
+    _compare(out, O.attention_ref(q, kd, vd, scale, dtype=torch.float16), O.attention_exact(q.float(), kd, vd, scale),
+             f'fp16 tables int{bits}', oracle_bar=1e-2)
+
+
+def test_fp16_needs_head_dim_64(dev):
+    from var_q_amd import VarqError
+    g = torch.Generator().manual_seed(1)
+    k = torch.randn(1, 2, 50, 128, generator=g).bfloat16()
+    kw, ks, kz, _ = _quantize(k, 128, 4)
+    q = torch.randn(1, 2, 8, 128, generator=g).half().to(dev)
+    with pytest.raises(VarqError, match='fp16'):
+        ops.fused_attn(q, kw.to(dev), ks.to(dev), kz.to(dev), kw.to(dev), ks.to(dev), kz.to(dev), 4, 4, 50, 0.1)

@@ -213,3 +213,70 @@ def test_config5_full_schedule_mixed_bits(dev):
         ref = O.attention_ref(q, kd[:, :, :pos], vd[:, :, :pos], scale)
         _compare(out, ref, _exact(q, kd[:, :, :pos], vd[:, :, :pos], scale, dev), f'c5 scale {p}')
     assert cache.len == L == 10521
+
+
+def test_config5_full_size_seeded_bits(dev):
+    """Configuration 5 at the size it is named at: B=8 (4 images x CFG pair), H=16, the seeded
+    per-head bit-widths of bench.py, the 13 scales on heavy-tailed data (Student-t, nu=4, one
+    channel x20, generated on the device).  Checked: for one (batch, head) per bit-width class the
+    cache contents bit for bit against the oracle and that head's attention at scales 1, 8, 32
+    and 64 against the oracle's bf16 attention (bench.c5_check, which bench.py's own leg runs);
+    and on the last scale's launch -- all 128 (batch, head) pairs, the three classes side by
+    side, the library's choice of key sharing -- what holds at any size (`_properties`)."""
+    import bench
+    B, H, D, g = bench.C5_B, bench.C5_H, bench.C5_D, bench.C5_GROUP
+    bits = bench.c5_head_bits(torch)
+    assert sorted(set(bits)) == [2, 4, 8] and len(bits) == H
+    pn = schedules.INFINITY_PATCH_NUMS
+    ns = schedules.tokens_per_scale(pn)
+    L = sum(ns)
+    gen = torch.Generator(device=dev).manual_seed(5505)
+
+    def student(n):
+        x = torch.randn(B, H, n, D, device=dev, generator=gen)
+        chi = torch.randn(4, B, H, n, D, device=dev, generator=gen).square_().mean(0)
+        x = x / chi.sqrt_()
+        x[..., 77] *= 20.0
+        return x.bfloat16()
+    steps = [(torch.randn(B, H, n, D, device=dev, generator=gen).bfloat16(), student(n), student(n)) for n in ns]
+    cache = PackedKVCache(B, H, L, D, bits, g, dev)
+    scale = 1.0 / math.sqrt(D)
+    outs = []
+    for i, (q, k, v) in enumerate(steps):
+        note('config 5 full size: scale', pn[i], 'tokens', ns[i])
+        cache.append(k, v)
+        outs.append(cache.attend(q, scale))
+    torch.cuda.synchronize()
+    assert cache.len == L
+    note('config 5 full size: against the oracle')
+    res = bench.c5_check(torch, O, dev, cache, steps, outs, bits)
+    print('[c5 full size]', res, flush=True)
+    assert res['cache_bit_exact'], res
+    assert res['attn_maxabs_over_range_max'] <= 2e-2 and res['attn_cosine_min'] >= 0.9995, res
+    assert len(res['pairs']) == 3
+
+    # the last scale's queries over the whole cache, class by class into one output
+    q = steps[-1][0]
+
+    def run(kv_limit=None, perm=None, pad=0, v=None):
+        out = torch.zeros_like(q)
+        for ci, c in enumerate(cache.classes):
+            kt = [c.k_words, c.k_scale, c.k_zp]
+            vt = [c.v_words, c.v_scale, c.v_zp] if v is None else list(v[ci])
+            if perm is not None:
+                kt, vt = [t[:, :, perm].contiguous() for t in kt], [t[:, :, perm].contiguous() for t in vt]
+            if pad:
+                junk = lambda t: torch.full_like(t[:, :, :pad], 0x7f if t.dtype == torch.int32 else 1e30)
+                kt, vt = [torch.cat([t, junk(t)], 2).contiguous() for t in kt], [torch.cat([t, junk(t)], 2).contiguous() for t in vt]
+            ops.fused_attn(q, *kt, *vt, c.bits, c.bits, L, scale, kv_limit=kv_limit, head_map=c.head_map, out=out,
+                           splits=1)       # (as attend() launches classes that run side by side)
+        return out
+
+    # V caches that dequantize to 1.25 everywhere: every field holds code 1 (2 and 8 bits) or 5 (4 bits)
+    vconst = []
+    for c in cache.classes:
+        byte, code = {2: (0x55, 1), 4: (0x55, 5), 8: (0x01, 1)}[c.bits]
+        vs = torch.rand(c.v_scale.shape, device=dev, generator=gen) + 0.5
+        vconst.append((torch.full_like(c.v_words, int.from_bytes(bytes([byte] * 4), 'little', signed=True)), vs, code - 1.25 / vs))
+    base = _properties(run, vconst, L, dev, 'config 5')
+    assert torch.equal(base, outs[-1]), 'the classes launched one by one and PackedKVCache.attend differ'

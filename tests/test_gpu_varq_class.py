@@ -89,16 +89,19 @@ def test_per_head_extension_single_call(dev):
 @pytest.mark.parametrize('method', list(O.METHODS))
 @pytest.mark.parametrize('bits', [4, 8])
 @pytest.mark.parametrize('fmt', ['BHLc', 'BLHc'])
-def test_fused_attention_over_quantizer_caches(dev, method, bits, fmt):
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_fused_attention_over_quantizer_caches(dev, method, bits, fmt, dtype):
     """`fused_attention` over the packed caches of two drop-in quantizers, all six methods of
     the reference in both of its layouts (BLHc is what its flash-attention call and
     VAR-VAR_Q-8.json use, BHLc what Infinity-VAR_Q-8.json names), four steps, against the
-    oracle class's dequant_all -> bf16 SDPA on the CPU (the path the reference runs:
-    VAR_Q/quant.py:216-230 into the attention backend).
+    oracle class's dequant_all -> SDPA on the CPU (the path the reference runs:
+    VAR_Q/quant.py:216-230 into the attention backend) in the dtype of q: bf16 (Infinity), or
+    fp16, the dtype of the VAR path (VAR/models/basic_var.py:157-158 under the fp16 autocast of
+    scripts/inference_multi_VAR.py:123), which the head-dim-64 kernels run in as well.
     Tolerance: cosine >= 0.9995, max-abs 2e-2 in units of the output range."""
     from var_q_amd.quant import fused_attention
-    note('fused_attention', method, bits, fmt)
-    ks, vs = _steps(fmt, torch.bfloat16, seed=20 + bits), _steps(fmt, torch.bfloat16, seed=30 + bits)
+    note('fused_attention', method, bits, fmt, dtype)
+    ks, vs = _steps(fmt, dtype, seed=20 + bits), _steps(fmt, dtype, seed=30 + bits)
     rk, rv = O.OracleVARQ(bits, fmt, method, pack_to_int32=False), O.OracleVARQ(bits, fmt, method, pack_to_int32=False)
     gk, gv = VAR_Q(bits, fmt, method), VAR_Q(bits, fmt, method)
     g = torch.Generator().manual_seed(5)
@@ -108,10 +111,12 @@ def test_fused_attention_over_quantizer_caches(dev, method, bits, fmt):
         for qz, item in ((gk, k), (gv, v)):
             qz.quant(item.to(dev))
             qz.cache()
-        q = torch.randn(k.shape[0], k.shape[1], k.shape[2], k.shape[3], generator=g).bfloat16()
-        out = bhl(fused_attention(q.to(dev), gk, gv, 0.125).float().cpu())
+        q = torch.randn(k.shape[0], k.shape[1], k.shape[2], k.shape[3], generator=g).to(dtype)
+        got = fused_attention(q.to(dev), gk, gv, 0.125)
+        assert got.dtype == dtype
+        out = bhl(got.float().cpu())
         assert out.shape == bhl(q).shape
-        ref = O.attention_ref(bhl(q), bhl(kd), bhl(vd), 0.125).float()
+        ref = O.attention_ref(bhl(q), bhl(kd), bhl(vd), 0.125, dtype=dtype).float()
         span = max(1.0, float(ref.abs().max()))
         err = float((out - ref).abs().max())
         cos = float(torch.nn.functional.cosine_similarity(out.flatten().double(), ref.flatten().double(), dim=0))
