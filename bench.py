@@ -13,9 +13,10 @@ After the timed region (and outside `value`): the quantize+pack kernel and the
 unpack+dequant kernel of configuration 4 timed as back-to-back launches between one
 event pair (kernel time without the dispatch gaps); the CPU baseline (1 thread and all
 threads, per stage, median of 3) with the parity check of the timed GPU results against
-it; and legs for configurations 2, 3 and 5 and for the shipped JSON rules.
+it; a leg for few queries over the whole packed cache (where the KV-read fraction of HBM peak
+is the bound); and legs for configurations 2, 3 and 5 and for the shipped JSON rules.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-c2] [--no-c3] [--no-c5] [--no-prepare] [--no-rule]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-hbm] [--no-c2] [--no-c3] [--no-c5] [--no-prepare] [--no-rule]
 """
 import argparse
 import json
@@ -449,6 +450,38 @@ def shipped_rule_latency(torch, dev, passes=5, warm=2):
     return out
 
 
+def hbm_regime_rates(torch, dev, kv_sets):
+    """The regime in which the metric's "KV-read fraction of HBM peak" is a bound: a few queries
+    over the whole packed cache of configuration 4 (INT4 group 128, B=2, H=16, 10 521 keys),
+    Lq = 16 and 64, where the arithmetic intensity (4 * Lq flop per packed byte) is below or near
+    the machine balance.  The four packed caches of the timed steps are cycled (4 x 48.5 MB of
+    codes, scales and zero-points), so the reads come from HBM.  Reports the time, the packed-KV
+    GB/s and its fraction of the 8 TB/s peak, and how the keys were shared out."""
+    from var_q_amd import _lib, ops
+    lib = _lib.load()
+    _, kv_bytes, _ = algorithmic_bytes()
+    out = {'workload': 'INT4 g128 packed cache of configuration 4 [B=2,H=16,Lk=10521,D=128]; Lq queries per (batch, head) '
+                       'over all keys, 4 packed caches cycled', 'kv_MB': round(kv_bytes / 1e6, 2)}
+    gd = torch.Generator(device=dev).manual_seed(8008)
+    scale = 1.0 / math.sqrt(D)
+    for lq in (16, 64):
+        q = torch.randn(B, H, lq, D, device=dev, generator=gd).bfloat16()
+        o = torch.empty_like(q)
+        i = [0]
+
+        def fn():
+            t = kv_sets[i[0] % len(kv_sets)]
+            i[0] += 1
+            ops.fused_attn(q, t['kw'], t['ks'], t['kz'], t['vw'], t['vs'], t['vz'], BITS, BITS, L, scale, out=o)
+        dt = timed_launches(torch, fn, reps=40, warm=8)
+        flops = 4 * B * H * lq * L * D
+        out['Lq%d' % lq] = {'us': round(dt * 1e6, 1), 'kv_read_GBps': round(kv_bytes / dt / 1e9, 1),
+                            'kv_read_frac_hbm_peak': round(kv_bytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                            'TFLOPs': round(flops / dt / 1e12, 1),
+                            'key_shares': int(lib.varq_fused_attn_key_shares(B, H, lq, L, D, GROUP, GROUP))}
+    return out
+
+
 def attention_check(torch, dev, out, q, kd, vd, ref, scale):
     """The timed attention output against the oracle (cosine) and against an fp64 evaluation of
     the same formula on the oracle's dequantized operands (max-abs in units of the output
@@ -484,6 +517,7 @@ def main():
     ap.add_argument('--single-launches', action='store_true', help='quantize K and V in two launches instead of one')
     ap.add_argument('--no-rule', action='store_true', help='skip the shipped-rule latency leg (profiling runs)')
     ap.add_argument('--no-prepare', action='store_true', help='skip the producer-side (qkv_prepare) leg (profiling runs)')
+    ap.add_argument('--no-hbm', action='store_true', help='skip the few-queries-over-a-long-cache leg (profiling runs)')
     ap.add_argument('--no-pack', action='store_true', help='skip the standalone pack / unpack leg (profiling runs)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
@@ -710,6 +744,7 @@ def main():
                              'traffic': None if not traffic else traffic.get('dequant'),
                              'timing': '40 back-to-back launches through the C ABI between one HIP event pair, median of 5'},
         'cpu_baseline': cpu, 'checked_against_oracle': checked,
+        'hbm_regime_rates': None if args.no_hbm else hbm_regime_rates(torch, dev, outs),
         'config2_rates': None if args.no_c2 else c2_rates(torch, dev),
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev, check=not args.no_cpu),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),

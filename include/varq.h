@@ -229,7 +229,10 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *              up to 8 workgroups; their partial results (fp32) pass through the
  *              workspace and a second kernel combines them.  splits = 0: the library
  *              decides, and uses no more shares than the workspace holds (none
- *              without a workspace); 1: never; 2..8: exactly that many (an error if
+ *              without a workspace) -- with at most 64 queries over at least 1024 keys
+ *              (D = 128, one scale group per key, bf16) it takes a kernel of its own for
+ *              that regime, whose wavefronts all serve the same 32 queries on different
+ *              keys, with up to 64 shares; 1: never; 2..8: exactly that many (an error if
  *              the workspace is too small).  varq_fused_attn_workspace_bytes gives the
  *              size for a shape (0 when the library would not share the keys out);
  *              device memory, 16-byte aligned, used only during the call's kernels.
@@ -237,6 +240,10 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  * dividing D.
  */
 size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk, int D, int nseg, int splits);
+/* Over how many workgroups varq_fused_attn shares the keys of a query block out when that is left
+ * to it (splits = 0) and the workspace has room; 1 = not at all.  (A report for callers and
+ * benchmarks; no counterpart in the reference.) */
+int varq_fused_attn_key_shares(int B, int Hkv, int Lq, int Lk, int D, int k_group, int v_group);
 int varq_fused_attn(const void *q, void *out,
                     const int32_t *k_words, const float *k_scale, const float *k_zp, int k_bits, int k_group,
                     const int32_t *v_words, const float *v_scale, const float *v_zp, int v_bits, int v_group,

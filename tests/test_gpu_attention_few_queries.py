@@ -1,0 +1,117 @@
+"""The kernel for few queries over a long cache (at most 64 queries per (batch, head), at least
+1024 keys, one scale group per key at head dim 128), which `fused_attn` takes when the sharing of
+the keys is left to it: against the oracle path unpack -> dequant -> bf16 SDPA (strict bar, as
+in test_gpu_attention.py), and against the general kernel on the same inputs (`splits=1` keeps a
+launch on it): the two dequantize to the same bf16 operands and differ by summation order only."""
+import math
+
+import pytest
+import torch
+
+import varq_oracle as O
+from gpu_util import note
+from test_gpu_attention import _compare, _exact_fp64, _quantize
+from var_q_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dev, B, H, Lq, Lk, bits, seed, dist='normal', limit=False, layout='BHLc', Lstride=None, heads=None):
+    D, g = 128, 128
+    gen = torch.Generator().manual_seed(seed)
+    Hkv = H if heads is None else len(heads)
+    k = O.synth_kv((B, Hkv, Lk, D), seed + 1, dist).bfloat16()
+    v = O.synth_kv((B, Hkv, Lk, D), seed + 2, dist).bfloat16()
+    q = torch.randn(B, H, Lq, D, generator=gen).bfloat16()
+    kw, ks, kz, kd = _quantize(k, g, bits)
+    vw, vs, vz, vd = _quantize(v, g, bits)
+    scale = 1.0 / math.sqrt(D)
+    lim = bias = None
+    if limit:
+        lim = torch.randint(0, Lk + 1, (Lq,), generator=gen).int()
+        lim[0] = Lk
+        bias = torch.zeros(Lq, Lk)
+        bias[torch.arange(Lk)[None, :] >= lim[:, None].long()] = float('-inf')
+    args = [kw, ks, kz, vw, vs, vz]
+    if Lstride:       # spare token rows behind the cached ones, filled with junk
+        args = [torch.cat([t, torch.full((B, Hkv, Lstride - Lk, t.shape[3]), 0x7f if t.dtype == torch.int32 else 1e30, dtype=t.dtype)], 2)
+                for t in args]
+    qd = q
+    if layout == 'BLHc':
+        args, qd = [t.transpose(1, 2).contiguous() for t in args], q.transpose(1, 2).contiguous()
+    args = [t.to(dev) for t in args]
+    hm = None if heads is None else torch.tensor(heads, dtype=torch.int32, device=dev)
+    kw_ = dict(kv_limit=None if lim is None else lim.to(dev), layout=layout, head_map=hm)
+    note('few queries', (B, H, Lq, Lk), bits, dist, 'limit' if limit else '', layout, Lstride, heads)
+    out0 = torch.zeros_like(qd).to(dev)
+    out = ops.fused_attn(qd.to(dev), *args, bits, bits, Lk, scale, out=out0, **kw_)
+    general = ops.fused_attn(qd.to(dev), *args, bits, bits, Lk, scale, splits=1, out=torch.zeros_like(out0), **kw_)
+    torch.cuda.synchronize()
+    if layout == 'BLHc':
+        out, general = out.transpose(1, 2), general.transpose(1, 2)
+    hsel = list(range(H)) if heads is None else heads
+    qs = q[:, hsel]
+    if lim is not None:
+        seen = lim > 0
+        assert float(out[:, :, ~seen].abs().max() if bool((~seen).any()) else 0.0) == 0.0, 'a query without keys must get zeros'
+        out, general, qs, bias = out[:, :, seen], general[:, :, seen], qs[:, :, seen], bias[seen]
+    out, general = out[:, hsel], general[:, hsel]
+    ref = O.attention_ref(qs, kd, vd, scale, bias)
+    _compare(out, ref, _exact_fp64(qs, kd, vd, scale, bias, dev), f'few queries {Lq}x{Lk} int{bits}')
+    span = max(1.0, float(ref.abs().max()))
+    assert float((out.float() - general.float()).abs().max().cpu()) <= span * 2 ** -6, 'the two kernels differ by more than two bf16 steps'
+    if heads is not None:
+        rest = [h for h in range(H) if h not in heads]
+        assert float(out0[:, rest].abs().max()) == 0.0, 'heads outside the map were written'
+
+
+@pytest.mark.parametrize('bits', [4, 2, 8])
+@pytest.mark.parametrize('Lq,Lk', [(16, 10521), (64, 4121), (1, 1024), (33, 2521), (32, 1055)])
+def test_against_oracle_and_general_kernel(dev, bits, Lq, Lk):
+    assert _lib.load().varq_fused_attn_key_shares(2, 3, Lq, Lk, 128, 128, 128) >= 1
+    _case(dev, 2, 3, Lq, Lk, bits, seed=bits * 1000 + Lq)
+
+
+@pytest.mark.parametrize('bits', [4, 8])
+def test_heavy_tails_key_limits_layouts_and_windows(dev, bits):
+    _case(dev, 1, 2, 16, 6425, bits, seed=11 + bits, dist='student4')
+    _case(dev, 2, 2, 40, 2000, bits, seed=12 + bits, limit=True)
+    _case(dev, 2, 3, 20, 1500, bits, seed=13 + bits, layout='BLHc')
+    _case(dev, 1, 2, 9, 1300, bits, seed=14 + bits, Lstride=1400, limit=True)
+    _case(dev, 2, 5, 12, 1100, bits, seed=15 + bits, heads=[4, 1, 2])
+
+
+def test_many_pairs_one_share_each(dev):
+    """Enough (batch, head) pairs to fill the device without sharing keys out: one workgroup per
+    pair, no workspace, output written directly."""
+    assert _lib.load().varq_fused_attn_key_shares(8, 128, 16, 1024, 128, 128, 128) == 1
+    _case(dev, 8, 128, 16, 1024, 4, seed=99)
+
+
+def test_config4_shape_properties(dev):
+    """The benchmark's shape (B=2, H=16, 10 521 keys, INT4 group 128, 16 queries) through what
+    holds at any size: a constant V gives that constant, key order does not matter, rows behind
+    the cached ones are not read."""
+    B, H, Lq, Lk, D, bits, g = 2, 16, 16, 10521, 128, 4, 128
+    gen = torch.Generator(device=dev).manual_seed(44)
+    k = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    v = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    q = torch.randn(B, H, Lq, D, device=dev, generator=gen).bfloat16()
+    kq, vq = ops.quant_pack_rows(k, g, bits, True), ops.quant_pack_rows(v, g, bits, True)
+    scale = 1 / math.sqrt(D)
+    assert _lib.load().varq_fused_attn_key_shares(B, H, Lq, Lk, D, g, g) > 8
+    note('few queries, config-4 shape: constant V')
+    vw = torch.full_like(vq[0], int.from_bytes(bytes([5 * 17] * 4), 'little', signed=True))
+    vs = torch.rand(B, H, Lk, 1, device=dev, generator=gen) + 0.5
+    out = ops.fused_attn(q, *kq, vw, vs, 5 - 1.25 / vs, bits, bits, Lk, scale)
+    assert float((out.float() - 1.25).abs().max()) <= 2 ** -7
+    note('few queries, config-4 shape: permuted keys, rows behind the end')
+    base = ops.fused_attn(q, *kq, *vq, bits, bits, Lk, scale)
+    perm = torch.randperm(Lk, device=dev, generator=gen)
+    other = ops.fused_attn(q, *[t[:, :, perm].contiguous() for t in kq], *[t[:, :, perm].contiguous() for t in vq], bits, bits, Lk, scale)
+    span = max(1.0, float(base.float().abs().max()))
+    assert float((other.float() - base.float()).abs().max()) <= max(2e-2 * span / 4, span * 2 ** -7)
+    longer = [torch.cat([t, torch.full_like(t[:, :, :300], 0x7f if t.dtype == torch.int32 else 1e30)], dim=2).contiguous()
+              for t in (*kq, *vq)]
+    assert torch.equal(ops.fused_attn(q, *longer, bits, bits, Lk, scale), base)
+    torch.cuda.synchronize()

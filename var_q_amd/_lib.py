@@ -37,6 +37,7 @@ SYMBOLS = {
                                 c_int, c_int, c_int, c_int,
                                 c_void_p, c_float, c_int, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p]),
     'varq_fused_attn_workspace_bytes': (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    'varq_fused_attn_key_shares': (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     'varq_fused_attn_channel': (c_int, [c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p,

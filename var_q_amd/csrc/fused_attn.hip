@@ -68,6 +68,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kHeadroom = 15.f;   // exact-code kernels: octaves between a fresh softmax reference and the row maximum
 
 constexpr int kMaxSegments = 16;
+constexpr int kMaxSplits_v = 8;        // shares of a query block's keys in the general kernel
+constexpr int kMaxKeyShares_v = 64;    // ... and in the kernel for few queries
 constexpr int kChanTableRows = 4;   // LDS rows per segment of the per-channel tables
 
 struct AttnParams {
@@ -1190,30 +1192,64 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   }
 }
 
-// One thread per (query row, four channels): the shares' outputs weighted by their softmax
-// mass l * 2^(m - M), M the largest reference among the shares that saw a key.
+// The shares' outputs weighted by their softmax mass l * 2^(m - M), M the largest reference among
+// the shares that saw a key.  A workgroup of 256 threads serves 2 query rows x (D/4) channel quads
+// x G groups of shares (G = 4 at D=128, 8 at D=64: the threads of a quad split the shares among
+// them): the weights of a row's shares are formed once, in LDS, and every thread then sums its
+// shares' quads with nothing between the loads but the weights.
 template <int D, bool F16>
 __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
+  constexpr int QUADS = D / 4, ROWS = 2, G = 256 / (ROWS * QUADS);
+  constexpr int kMaxS = 64;
+  static_assert(G >= 1 && kMaxS >= kMaxKeyShares_v && kMaxS >= kMaxSplits_v, "share counts");
+  __shared__ float w_lds[ROWS][kMaxS];
   const int64_t rows = (int64_t)p.bh_total * p.Lq;
-  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = item / (D / 4);
-  const int c0 = (int)(item % (D / 4)) * 4;
-  if (row >= rows) return;
-  float m_max = -INFINITY;
-  for (int s = 0; s < p.nsplit; ++s) {
-    const float2 ml = *reinterpret_cast<const float2 *>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-    if (ml.y > 0.f) m_max = fmaxf(m_max, ml.x);
+  const int tid = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+  // weights of the rows' shares
+  __shared__ float2 ml_lds[ROWS][kMaxS];
+  static_assert(ROWS * kMaxS <= 256, "one (row, share) per thread");
+  const int wr = tid / kMaxS, wsh = tid % kMaxS;
+  if (tid < ROWS * kMaxS) {
+    float2 ml = make_float2(0.f, 0.f);   // (denominator 0: an empty share)
+    if (wsh < p.nsplit && row0 + wr < rows) ml = *reinterpret_cast<const float2 *>(p.ws_ml + ((int64_t)wsh * rows + row0 + wr) * 2);
+    ml_lds[wr][wsh] = ml;
   }
+  __syncthreads();
+  if (tid < ROWS * kMaxS) {
+    float m_max = -INFINITY;
+    for (int t = 0; t < p.nsplit; ++t)
+      if (ml_lds[wr][t].y > 0.f) m_max = fmaxf(m_max, ml_lds[wr][t].x);
+    const float2 ml = ml_lds[wr][wsh];
+    w_lds[wr][wsh] = ml.y > 0.f ? ml.y * __builtin_amdgcn_exp2f(ml.x - m_max) : 0.f;
+  }
+  __syncthreads();
+  const int r = tid / (QUADS * G), gq = tid % (QUADS * G), grp = gq / QUADS, c0 = (gq % QUADS) * 4;
+  const int64_t row = row0 + r;
   float acc[4] = {0.f, 0.f, 0.f, 0.f}, wsum = 0.f;
-  for (int s = 0; s < p.nsplit; ++s) {
-    const float2 ml = *reinterpret_cast<const float2 *>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-    if (!(ml.y > 0.f)) continue;
-    const float w = ml.y * __builtin_amdgcn_exp2f(ml.x - m_max);
-    const float4 o = *reinterpret_cast<const float4 *>(p.ws_o + ((int64_t)s * rows + row) * D + c0);
-    acc[0] = __builtin_fmaf(w, o.x, acc[0]); acc[1] = __builtin_fmaf(w, o.y, acc[1]);
-    acc[2] = __builtin_fmaf(w, o.z, acc[2]); acc[3] = __builtin_fmaf(w, o.w, acc[3]);
-    wsum += w;
+  if (row < rows) {
+#pragma unroll 4
+    for (int s_ = grp; s_ < p.nsplit; s_ += G) {
+      const float w = w_lds[r][s_];
+      const float4 o = *reinterpret_cast<const float4 *>(p.ws_o + ((int64_t)s_ * rows + row) * D + c0);
+      acc[0] = __builtin_fmaf(w, o.x, acc[0]); acc[1] = __builtin_fmaf(w, o.y, acc[1]);
+      acc[2] = __builtin_fmaf(w, o.z, acc[2]); acc[3] = __builtin_fmaf(w, o.w, acc[3]);
+      wsum += w;
+    }
   }
+  if constexpr (G > 1) {
+    // the groups of a row's shares meet through LDS (group 0 collects)
+    __shared__ float part[256][5];
+    part[tid][0] = acc[0]; part[tid][1] = acc[1]; part[tid][2] = acc[2]; part[tid][3] = acc[3]; part[tid][4] = wsum;
+    __syncthreads();
+    if (grp != 0) return;
+#pragma unroll
+    for (int g2 = 1; g2 < G; ++g2) {
+      const float *o = part[tid + g2 * QUADS];
+      acc[0] += o[0]; acc[1] += o[1]; acc[2] += o[2]; acc[3] += o[3]; wsum += o[4];
+    }
+  }
+  if (row >= rows) return;
   const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
   const int bh = (int)(row / p.Lq), qrow = (int)(row % p.Lq);
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
@@ -1244,8 +1280,8 @@ void launch_shape(const AttnParams &p, hipStream_t st) {
   dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
   hipLaunchKernelGGL((fused_attn_kernel<D, BITS, GK, GV, CHAN, NWV, WPS, EXACT, F16>), grid, dim3(NWV * 64), lds_bytes, st, p);
   if (p.nsplit > 1) {
-    const int64_t items = (int64_t)p.bh_total * p.Lq * (D / 4);
-    hipLaunchKernelGGL((combine_splits_kernel<D, F16>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, p);
+    const int64_t rows = (int64_t)p.bh_total * p.Lq;
+    hipLaunchKernelGGL((combine_splits_kernel<D, F16>), dim3((unsigned)((rows + 1) / 2)), dim3(256), 0, st, p);
   }
 }
 
@@ -1314,7 +1350,7 @@ int set_layout(AttnParams &p, int layout, const char *who) {
 }
 
 // ---- sharing the keys of a query block out over several workgroups ---------------------
-constexpr int kMaxSplits = 8;
+constexpr int kMaxSplits = kMaxSplits_v;
 
 int device_cus() {
   static int cus[64] = {0};
@@ -1374,6 +1410,326 @@ int set_splits(AttnParams &p, int D, int tiles, int splits, void *workspace, siz
   return VARQ_OK;
 }
 
+
+// ---- few queries over a long cache (the regime bound by the reads of the packed cache) -----------
+// With at most a few dozen queries per (batch, head) the arithmetic intensity of the attention,
+// 32 * Lq / (bits_K + bits_V) flop per packed byte, is below the machine balance: the kernel above,
+// built around 256 queries per workgroup, leaves seven of its eight wavefronts without queries and
+// spends a workgroup barrier per 64 keys on the remaining one.  This kernel turns the work round:
+// all wavefronts of a workgroup serve the SAME 32 queries and each takes its own 32-key blocks of
+// the workgroup's share of the keys, from global memory straight to registers, with nothing shared
+// between wavefronts inside the key loop and no workgroup barrier in it:
+//  * K: a lane loads half a key row (the half its MFMA A operands come from), dequantizes it in
+//    registers -- (code - zp) * scale in fp32, rounded to bf16, the operands the reference's
+//    attention sees -- and feeds S^T = K Q^T directly; the Q^T operands sit in LDS, written once;
+//  * V: a lane widens items of two adjacent keys x 8 channels into a wavefront-private V^T tile
+//    in LDS (the second contraction runs over keys), read back as MFMA A operands by the same
+//    wavefront -- LDS requests of one wavefront are served in order, so no barrier is needed;
+//  * online softmax per lane against the running maximum;
+//  * the next block's packed words are requested before the current block's arithmetic.
+// The wavefronts' partial results are merged through LDS (two rounds), the workgroups' shares
+// through the workspace and combine_splits_kernel, as for the kernel above.
+// One scale group per key (group = D = 128), bf16, any layout, key limits, head maps.
+constexpr int FQ_NW = 4;             // wavefronts per workgroup
+constexpr int FQ_BK = 32;            // keys per block: one 32-row MFMA block
+constexpr int FQ_VTS = FQ_BK + 8;    // V^T row stride (bf16): 16-byte rows, bank spread
+constexpr int FQ_D = 128;
+constexpr int kFewQueries = 64;      // launches with at most this many queries per (batch, head) ...
+constexpr int kFewQMinKeys = 1024;   // ... over at least this many keys take this kernel
+constexpr int kMaxKeyShares = kMaxKeyShares_v;
+struct FewQLds {
+  static constexpr int kQ = 0;                                         // [8][64] 16-byte Q^T operands
+  static constexpr int kVt = kQ + 8 * 64 * 16;                         // [FQ_NW][D][FQ_VTS] bf16
+  static constexpr int kPar = kVt + FQ_NW * FQ_D * FQ_VTS * 2;         // [FQ_NW][2][32] fp32
+  static constexpr int kMl = kPar + FQ_NW * 2 * 32 * 4;                // [2][32][2] fp32 (merge)
+  static constexpr int kBytes = kMl + 2 * 32 * 2 * 4;
+  static_assert(2 * 64 * 64 * 4 <= FQ_NW * FQ_D * FQ_VTS * 2, "the merge slots reuse the V^T tiles");
+};
+
+template <int BITS>
+__global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnParams p) {
+  constexpr int D = FQ_D, WPR = D * BITS / 32, NCH = D / 16, NDB = D / 32;
+  constexpr int HW = WPR / 2;                 // packed words of half a key row
+  constexpr int KP = HW / 4;                  // 16-byte pieces of it
+  constexpr int OPQ = 16 / BITS;              // octets per piece
+  constexpr int UPR = BITS == 2 ? 8 : 16;     // V units per key row: a word, or the two words of an octet of bytes
+  constexpr int WPU = BITS == 8 ? 2 : 1;      // words per unit
+  constexpr int OPU = BITS == 2 ? 2 : 1;      // octets per unit
+  constexpr int IPL = 16 * UPR / 64;          // V items (two keys x one unit) per lane and block
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  u32x4_t *const lds_q = reinterpret_cast<u32x4_t *>(lds_raw + FewQLds::kQ);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, half = lane >> 5;
+  uint16_t *const vt = reinterpret_cast<uint16_t *>(lds_raw + FewQLds::kVt) + wave * D * FQ_VTS;
+  float *const par = reinterpret_cast<float *>(lds_raw + FewQLds::kPar) + wave * 2 * 32;
+  float *const lds_ml = reinterpret_cast<float *>(lds_raw + FewQLds::kMl);
+
+  // workgroup -> (batch * head, query tile, share), ids congruent mod 8 (one L2) for one (batch, head)
+  const int wg = blockIdx.x;
+  const int xcd = wg & 7, slot_s = wg >> 3;
+  const int split = slot_s % p.nsplit, slot = slot_s / p.nsplit;
+  const int bh = (slot / p.q_tiles) * 8 + xcd;
+  const int qt = slot % p.q_tiles;
+  if (bh >= p.bh_total) return;
+  const int b = bh / p.Hkv, hs = bh % p.Hkv;
+  const int hq = p.head_map ? p.head_map[hs] : hs;
+
+  // ---- the workgroup's 32 queries: Q^T operands to LDS, in the slot order of the K codec ----
+  for (int e = tid; e < NCH * 64; e += FQ_NW * 64) {
+    const int ch = e >> 6, l = e & 63;
+    const int qr = min(qt * 32 + (l & 31), p.Lq - 1);
+    const __bf16 *qp = p.q + (b * p.q_bs + hq * p.q_hs + qr * p.q_ts) * D + ((l >> 5) * 8 + ch) * 8;
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(qp);
+    u32x4_t o;
+#pragma unroll
+    for (int j2 = 0; j2 < 4; ++j2) {
+      const int d0 = KCodec<BITS>::slot_d(2 * j2), d1 = KCodec<BITS>::slot_d(2 * j2 + 1);
+      const u32 lo = (raw[d0 >> 1] >> (16 * (d0 & 1))) & 0xffffu, hi = (raw[d1 >> 1] >> (16 * (d1 & 1))) << 16;
+      o[j2] = lo | hi;
+    }
+    lds_q[e] = o;
+  }
+  const int qrow = qt * 32 + col;
+  const bool q_live = qrow < p.Lq;
+  int limit = p.kv_limit ? min(p.kv_limit[min(qrow, p.Lq - 1)], p.Lk) : p.Lk;
+  if (limit < 0) limit = 0;
+  // every wavefront holds the same queries: the largest and smallest limit need no exchange between them
+  int kv_end = q_live ? limit : 0, minlim = q_live ? limit : p.Lk;
+  for (int off = 1; off < 64; off <<= 1) {
+    kv_end = max(kv_end, __shfl_xor(kv_end, off, 64));
+    minlim = min(minlim, __shfl_xor(minlim, off, 64));
+  }
+  const int nb = (kv_end + FQ_BK - 1) / FQ_BK;
+  const int b_begin = (int)((int64_t)nb * split / p.nsplit), b_end = (int)((int64_t)nb * (split + 1) / p.nsplit);
+  __syncthreads();   // Q^T operands written
+
+  const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
+  const int64_t kv_ts = p.kv_ts;
+  const u32 *kw = p.k_words + kv_row0 * WPR;
+  const u32 *vw = p.v_words + kv_row0 * WPR;
+  u32 kmask = KCodec<BITS>::kMask;
+  asm volatile("" : "+v"(kmask));
+
+  floatx16_t oacc[NDB];
+#pragma unroll
+  for (int d = 0; d < NDB; ++d)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) oacc[d][j] = 0.f;
+  float m_ref = 0.f, l_part = 0.f;
+  bool first = true;
+
+  // packed words and parameters of one block, as loaded
+  u32x4_t kraw[KP];
+  u32 vraw[IPL][2][WPU];
+  float ksc, kzp, vsc, vzp;
+  auto request = [&](int blk) {
+    const int t0 = blk * FQ_BK;
+    const int key = min(t0 + kperm(col), p.Lk - 1);       // MFMA row `col` carries key kperm(col) of the block
+    const u32 *src = kw + key * kv_ts * WPR + half * HW;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) kraw[i] = *reinterpret_cast<const u32x4_t *>(src + 4 * i);
+    const int64_t g = kv_row0 + key * kv_ts;
+    ksc = p.k_scale[g];
+    kzp = p.k_zp ? p.k_zp[g] : 0.f;
+#pragma unroll
+    for (int i = 0; i < IPL; ++i) {
+      const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int vkey = min(t0 + 2 * kp + r, p.Lk - 1);
+        const u32 *vs_ = vw + vkey * kv_ts * WPR + u * WPU;
+        if constexpr (WPU == 2) { const uint2 t = *reinterpret_cast<const uint2 *>(vs_); vraw[i][r][0] = t.x; vraw[i][r][1] = t.y; }
+        else vraw[i][r][0] = vs_[0];
+      }
+    }
+    const int64_t gv = kv_row0 + min(t0 + col, p.Lk - 1) * kv_ts;
+    vsc = p.v_scale[gv];
+    vzp = p.v_zp ? p.v_zp[gv] : 0.f;
+  };
+
+  int blk = b_begin + wave;
+  if (blk < b_end) request(blk);
+  for (; blk < b_end; blk += FQ_NW) {
+    const int t0 = blk * FQ_BK;
+    // this block's operands out of the request registers (which the next block's request refills)
+    u32x4_t kcur[KP];
+    u32 vcur[IPL][2][WPU];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) kcur[i] = kraw[i];
+#pragma unroll
+    for (int i = 0; i < IPL; ++i)
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int w = 0; w < WPU; ++w) vcur[i][r][w] = vraw[i][r][w];
+    // (code - zp) * scale = (raw - (zp + kOff) / kMul) * (kMul * scale) for the code image `raw`
+    const float zk = (kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), sk = ksc * KCodec<BITS>::kMul;
+    if (half == 0) {
+      par[col] = (vzp + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+      par[32 + col] = vsc * VCodec<BITS>::kMul;
+    }
+    if (blk + FQ_NW < b_end) request(blk + FQ_NW);
+
+    // ---- S^T = K Q^T, K dequantized in registers ----
+    floatx16_t sacc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sacc[j] = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+      const int pc = ch / OPQ, j = ch % OPQ;
+      u32 q4[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) q4[w] = kcur[pc][w] ^ KCodec<BITS>::kStageXor;
+      float f[8];
+      k_values<BITS>(q4, j, kmask, f);
+      u32x4_t a;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((f[2 * m] - zk) * sk, (f[2 * m + 1] - zk) * sk);
+      sacc = mfma_32x32x16<false>(a, lds_q[ch * 64 + lane], sacc);
+    }
+
+    // ---- softmax of the block: register i <-> key t0 + 16*(i/8) + 8*half + i%8 ----
+    float z[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = p.scale_log2e * sacc[i];
+    if (t0 + FQ_BK > minlim) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (t0 + 16 * (i >> 3) + 8 * half + (i & 7) >= limit) z[i] = -INFINITY;
+    }
+    float zmax = z[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
+    {
+      const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
+      zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
+    }
+    // the reference follows the running maximum; the accumulators are rescaled in every block
+    // (64 multiplications, mostly by one): a branch around them makes the compiler copy the
+    // accumulators at its join, which costs more
+    {
+      const float m_new = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(m_ref, zmax);
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+      m_ref = m_new;
+      first = false;
+      l_part *= alpha;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
+    }
+    u32 pop[2][4];
+#pragma unroll
+    for (int i2 = 0; i2 < 8; ++i2) {
+      const int i = 2 * i2;
+      const u32 w = pack_bf16_rne(__builtin_amdgcn_exp2f(z[i] - m_ref), __builtin_amdgcn_exp2f(z[i + 1] - m_ref));
+      pop[i >> 3][(i & 7) >> 1] = w;
+      typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+      l_part = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), l_part, false);
+    }
+
+    // ---- V of the block -> V^T tile of this wavefront (bf16 values) ----
+#pragma unroll
+    for (int i = 0; i < IPL; ++i) {
+      const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
+      u32 r0[WPU], r1[WPU];
+#pragma unroll
+      for (int w = 0; w < WPU; ++w) { r0[w] = vcur[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vcur[i][1][w] ^ VCodec<BITS>::kStageXor; }
+      const float2 z2 = *reinterpret_cast<const float2 *>(par + 2 * kp), s2 = *reinterpret_cast<const float2 *>(par + 32 + 2 * kp);
+#pragma unroll
+      for (int o = 0; o < OPU; ++o) {
+        float f0[8], f1[8];
+        v_pair_values<BITS>(r0, r1, o, kmask, f0, f1);
+        const int oct = u * OPU + o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * FQ_VTS + kp * 2]) = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
+      }
+    }
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const u32x4_t bv = {pop[c][0], pop[c][1], pop[c][2], pop[c][3]};
+#pragma unroll
+      for (int d = 0; d < NDB; ++d) {
+        const u32x4_t av = *reinterpret_cast<const u32x4_t *>(&vt[(d * 32 + col) * FQ_VTS + c * 16 + half * 8]);
+        oacc[d] = mfma_32x32x16<false>(av, bv, oacc[d]);
+      }
+    }
+  }
+
+  // ---- merge the wavefronts' partial results: 2 and 3 into 0 and 1, then 1 into 0 ----
+  float l_sum = l_part + __shfl_xor(l_part, 32, 64);
+  float *const slots = reinterpret_cast<float *>(lds_raw + FewQLds::kVt);   // [2][64 registers][64 lanes]
+#pragma unroll
+  for (int stride = 2; stride >= 1; stride >>= 1) {
+    __syncthreads();   // (first round: every wavefront is done with its V^T tile)
+    if (wave >= stride && wave < 2 * stride) {
+      float *dst = slots + (wave - stride) * 64 * 64;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) dst[(d * 16 + j) * 64 + lane] = oacc[d][j];
+      if (half == 0) { lds_ml[((wave - stride) * 32 + col) * 2] = m_ref; lds_ml[((wave - stride) * 32 + col) * 2 + 1] = l_sum; }
+    }
+    __syncthreads();
+    if (wave < stride) {
+      const float *src = slots + wave * 64 * 64;
+      const float mb = lds_ml[(wave * 32 + col) * 2], lb = lds_ml[(wave * 32 + col) * 2 + 1];
+      const bool has_a = l_sum > 0.f, has_b = lb > 0.f;
+      const float M = (has_a && has_b) ? fmaxf(m_ref, mb) : has_b ? mb : m_ref;
+      const float wa = has_a ? __builtin_amdgcn_exp2f(m_ref - M) : 0.f, wb = has_b ? __builtin_amdgcn_exp2f(mb - M) : 0.f;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[d][j] = oacc[d][j] * wa + src[(d * 16 + j) * 64 + lane] * wb;
+      l_sum = l_sum * wa + lb * wb;
+      m_ref = M;
+    }
+  }
+  if (wave != 0 || !q_live) return;
+  const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
+  __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D;
+  const bool shared_out = p.nsplit > 1;
+  const int64_t prow = ((int64_t)split * p.bh_total + bh) * p.Lq + qrow;
+  float *wptr = p.ws_o + prow * D;
+  if (shared_out && half == 0) *reinterpret_cast<float2 *>(p.ws_ml + prow * 2) = make_float2(m_ref, l_sum);
+#pragma unroll
+  for (int d = 0; d < NDB; ++d)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
+      const float o0 = oacc[d][4 * g4 + 0] * inv, o1 = oacc[d][4 * g4 + 1] * inv, o2 = oacc[d][4 * g4 + 2] * inv, o3 = oacc[d][4 * g4 + 3] * inv;
+      if (shared_out) *reinterpret_cast<float4 *>(wptr + d * 32 + 8 * g4 + 4 * half) = make_float4(o0, o1, o2, o3);
+      else *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
+    }
+}
+
+// Whether a launch takes the few-queries kernel, and over how many workgroups the keys of a
+// (batch, head, 32 queries) are shared out then: enough for the two resident workgroups per
+// compute unit (the kernel holds ~200 registers), at least eight blocks per workgroup.
+bool fewq_eligible(int Lq, int Lk, int D, int k_group, int v_group) {
+  return D == FQ_D && k_group == D && v_group == D && Lq > 0 && Lq <= kFewQueries && Lk >= kFewQMinKeys;
+}
+int fewq_shares(int bh_total, int Lq, int Lk) {
+  const int64_t tiles = (int64_t)((bh_total + 7) / 8 * 8) * ((Lq + 31) / 32);
+  int64_t s = (2 * (int64_t)device_cus() + tiles - 1) / tiles;
+  const int64_t nb = (Lk + FQ_BK - 1) / FQ_BK;
+  if (s > nb / 8) s = nb / 8;
+  if (s > kMaxKeyShares) s = kMaxKeyShares;
+  return s < 1 ? 1 : (int)s;
+}
+
+template <int BITS> void launch_fewq(const AttnParams &p, hipStream_t st) {
+  const int bh_pad = (p.bh_total + 7) / 8 * 8;
+  dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
+  hipLaunchKernelGGL((fused_attn_fewq_kernel<BITS>), grid, dim3(FQ_NW * 64), FewQLds::kBytes, st, p);
+  if (p.nsplit > 1) {
+    const int64_t rows = (int64_t)p.bh_total * p.Lq;
+    hipLaunchKernelGGL((combine_splits_kernel<FQ_D, false>), dim3((unsigned)((rows + 1) / 2)), dim3(256), 0, st, p);
+  }
+}
+
 }  // namespace
 
 extern "C" size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk, int D, int nseg, int splits) {
@@ -1381,8 +1737,17 @@ extern "C" size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk
   const int64_t rows = (int64_t)B * Hkv * Lq;
   (void)nseg;   // (the tile count does not depend on the tables)
   const int tiles = (Lk + BN - 1) / BN;
-  const int n = splits ? splits : choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), tiles, rows, D);
+  int n = splits ? splits : choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), tiles, rows, D);
+  // (the group sizes are not known here: room for the few-queries kernel's shares whenever the
+  // other sizes would admit it)
+  if (splits == 0 && fewq_eligible(Lq, Lk, D, D, D)) n = max(n, fewq_shares(B * Hkv, Lq, Lk));
   return split_workspace_bytes(n, rows, D);
+}
+
+extern "C" int varq_fused_attn_key_shares(int B, int Hkv, int Lq, int Lk, int D, int k_group, int v_group) {
+  if (B <= 0 || Hkv <= 0 || Lq <= 0 || Lk <= 0 || (D != 64 && D != 128)) return 0;
+  if (fewq_eligible(Lq, Lk, D, k_group, v_group)) return fewq_shares(B * Hkv, Lq, Lk);
+  return choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), (Lk + BN - 1) / BN, (int64_t)B * Hkv * Lq, D);
 }
 
 extern "C" int varq_fused_attn(const void *q, void *out,
@@ -1431,8 +1796,23 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.f16 = io_dtype == VARQ_F16;
   p.exact_codes = operand_form == VARQ_ATTN_EXACT_CODES && !p.f16;
   if (int e = set_layout(p, layout, "fused_attn")) return e;
-  if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn")) return e;
   hipStream_t st = (hipStream_t)stream;
+  // few queries over a long cache, left to the library: the kernel whose wavefronts share the keys
+  if (splits == 0 && !p.f16 && !p.exact_codes && fewq_eligible(Lq, Lk, D, k_group, v_group)) {
+    const int64_t rows = (int64_t)p.bh_total * Lq;
+    int n = fewq_shares(p.bh_total, Lq, Lk);
+    while (n > 1 && (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < split_workspace_bytes(n, rows, D))) --n;
+    p.q_tiles = (Lq + 31) / 32;
+    p.nsplit = n;
+    p.ws_o = n > 1 ? reinterpret_cast<float *>(workspace) : nullptr;
+    p.ws_ml = n > 1 ? p.ws_o + (size_t)n * (size_t)rows * (size_t)D : nullptr;
+    if (k_bits == 4) launch_fewq<4>(p, st);
+    else if (k_bits == 8) launch_fewq<8>(p, st);
+    else launch_fewq<2>(p, st);
+    VARQ_CHECK_LAUNCH("fused_attn");
+    return VARQ_OK;
+  }
+  if (int e = set_splits(p, D, (Lk + BN - 1) / BN, splits, workspace, workspace_bytes, "fused_attn")) return e;
   int rc = -1;
   if (D == 128) {
     if (k_bits == 4) rc = dispatch_groups<128, 4>(p, k_group, v_group, st);
