@@ -228,3 +228,34 @@ def test_quantizer_backend_infinity_shipped_rule(dev):
         rng = a.abs().max().item()
         assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
         assert _cos(a, b) >= 0.9995
+
+
+@pytest.mark.parametrize('backend', ['quantizer', True])
+@pytest.mark.parametrize('layout', ['BLHc', 'BHLc'])
+def test_var_module_in_fp16_the_dtype_of_its_autocast(dev, backend, layout):
+    """The VAR hook in fp16, the dtype the reference's VAR inference runs attention in
+    (scripts/inference_multi_VAR.py:123; q, k, v cast at VAR/models/basic_var.py:157-158): the fused
+    backends attend in fp16 as well (head dim 64) and agree with the drop-in + fp16 SDPA."""
+    torch.manual_seed(8)
+    C, H = 512, 8
+    pn = (1, 2, 3, 4, 5, 6, 8, 10, 13, 16)
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, enable_quantization=True, max_tokens=680)
+    if backend is True:
+        kw.update(q_bits=4, quant_method='G_GROUP', group_size=64, symmetric=False)
+    else:
+        kw.update(q_bits=8, quant_method='G_SCALE_HEAD_DIM')
+    a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).half()
+    b_mod = hooks.VarSelfAttention(0, fused=backend, **kw).to(dev).half()
+    b_mod.load_state_dict(a_mod.state_dict())
+    assert b_mod._attn_dtype(torch.float16) == torch.float16 and b_mod._attn_dtype(torch.float32) == torch.bfloat16
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    for p in pn:
+        note('hooks fp16', backend, layout, p)
+        x = torch.randn(2, p * p, C, device=dev, dtype=torch.float16)
+        a, b = a_mod(x), b_mod(x)
+        assert b.dtype == torch.float16
+        a, b = a.float(), b.float()
+        rng = a.abs().max().item()
+        assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
+        assert _cos(a, b) >= 0.9995
