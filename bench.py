@@ -175,6 +175,23 @@ def c5_latency(torch, dev, passes=10, warm=3, check=True):
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / passes
     flops = sum(4 * B5 * H5 * n * sum(ns[:i + 1]) * D5 for i, n in enumerate(ns))
+    # the same pass recorded once into a HIP graph and replayed: the first eight scales are a few
+    # microseconds of GPU work each behind ~140 us of host work per scale (three bit-width classes
+    # on side streams), which a replay does not pay
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one_pass()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_pass()
+    warm_passes(torch, graph.replay, warm)
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt_graph = (time.perf_counter() - t0) / passes
     checked = None
     if check:
         import varq_oracle as O
@@ -185,7 +202,9 @@ def c5_latency(torch, dev, passes=10, warm=3, check=True):
     return {'workload': 'config 5: 13-scale Infinity schedule, B=8 H=16 D=128, per-head bits %s, group 64 asymmetric, '
                         'in-place append + fused attention per scale, one layer' % ''.join(str(b) for b in bits),
             'ms_per_layer_pass': round(dt * 1e3, 4), 'ms_per_image_per_layer': round(dt * 1e3 / 4, 4),
-            'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes, 'checked': checked}
+            'attn_TFLOPs_incl_append': round(flops / dt / 1e12, 2), 'passes': passes,
+            'graph_replay_ms_per_layer_pass': round(dt_graph * 1e3, 4), 'graph_replay_TFLOPs': round(flops / dt_graph / 1e12, 2),
+            'checked': checked}
 
 
 PREWARM_MS = 50.0     # 0 (--fixed-prewarm): warm up by launch count only, so that separate runs launch alike
@@ -479,7 +498,31 @@ def hbm_regime_rates(torch, dev, kv_sets):
                             'kv_read_frac_hbm_peak': round(kv_bytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
                             'TFLOPs': round(flops / dt / 1e12, 1),
                             'key_shares': int(lib.varq_fused_attn_key_shares(B, H, lq, L, D, GROUP, GROUP))}
+    out['config5_early_scales'] = c5_early_scales(torch, dev)
     return out
+
+
+def c5_early_scales(torch, dev):
+    """Configuration 5's scales of at most 64 queries (patch numbers 1, 2, 4, 6, 8 at B=8, H=16, mixed widths, group 64):
+    the attention call of each scale over its prefix of the packed cache, the three bit-width classes side by side.  These
+    caches are short (1 to 121 keys, 0.03 to 3.6 MB of packed K/V), so the calls are bound by launch latency, not by HBM:
+    the figures say how far."""
+    from var_q_amd import PackedKVCache
+    from var_q_amd.schedules import INFINITY_PATCH_NUMS
+    bits = c5_head_bits(torch)
+    ns = [pn * pn for pn in INFINITY_PATCH_NUMS if pn * pn <= 64]
+    cache = PackedKVCache(C5_B, C5_H, sum(ns), C5_D, bits, C5_GROUP, dev)
+    gd = torch.Generator(device=dev).manual_seed(5006)
+    res = {}
+    for n in ns:
+        q, k, v = (torch.randn(C5_B, C5_H, n, C5_D, device=dev, generator=gd).bfloat16() for _ in range(3))
+        cache.append(k, v)
+        o = torch.empty_like(q)
+        dt = timed_launches(torch, lambda: cache.attend(q, 1.0 / math.sqrt(C5_D), out=o), reps=20, warm=5)
+        kv = sum(2 * C5_B * cache.len * (C5_D * b // 8 + (C5_D // C5_GROUP) * 8) for b in bits)
+        res['Lq%d_Lk%d' % (n, cache.len)] = {'us': round(dt * 1e6, 1), 'kv_MB': round(kv / 1e6, 3), 'kv_read_GBps': round(kv / dt / 1e9, 1),
+                                             'kv_read_frac_hbm_peak': round(kv / dt / 1e9 / HBM_PEAK_GBPS, 5)}
+    return res
 
 
 def attention_check(torch, dev, out, q, kd, vd, ref, scale):
