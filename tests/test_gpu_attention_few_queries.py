@@ -115,3 +115,17 @@ def test_config4_shape_properties(dev):
               for t in (*kq, *vq)]
     assert torch.equal(ops.fused_attn(q, *longer, bits, bits, Lk, scale), base)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('seed', range(12))
+def test_seeded_random_shapes(dev, seed):
+    """Seeded random cases inside the kernel's range (1..64 queries, 1024..5000 keys, any batch and
+    head count, either layout, with and without key limits, spare rows, head subsets)."""
+    g = torch.Generator().manual_seed(9000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    B, H, Lq, Lk, bits = r(1, 3), r(1, 5), r(1, 64), r(1024, 5000), (4, 2, 8)[seed % 3]
+    heads = None
+    if H >= 3 and seed % 4 == 1:
+        heads = sorted(set(r(0, H - 1) for _ in range(2)))
+    _case(dev, B, H, Lq, Lk, bits, seed=700 + seed, dist=('normal', 'student4')[seed % 2], limit=seed % 3 == 0,
+          layout=('BHLc', 'BLHc')[(seed // 2) % 2] if heads is None else 'BHLc', Lstride=Lk + r(1, 200) if seed % 5 == 2 else None, heads=heads)
