@@ -98,6 +98,7 @@ struct AttnParams {
   // the caller asked for exact codes in the MFMA operands where such a kernel exists (host side only)
   int exact_codes;
   int f16;   // q, out and the MFMA operands are fp16 (host side only: it selects the instantiation)
+  int fq_share_blocks;   // few-queries kernel: 32-key blocks per share of the keys
   // memory layout, in rows (a row = the D values of one token of one head):
   // q/out row = b*q_bs + h*q_hs + i*q_ts, key row = b*kv_bs + slot*kv_hs + j*kv_ts.
   // BHLc: (H*L, L, 1); BLHc (the layout of the flash-attention call): (L*H, 1, H).
@@ -1463,9 +1464,11 @@ struct FewQLds {
   static constexpr int kQ = 0;                                         // [8][64] 16-byte Q^T operands
   static constexpr int kVt = kQ + 8 * 64 * 16;                         // [FQ_NW][D][FQ_VTS] bf16
   static constexpr int kPar = kVt + FQ_NW * FQ_D * FQ_VTS * 2;         // [FQ_NW][2][32] fp32
-  static constexpr int kMl = kPar + FQ_NW * 2 * 32 * 4;                // [2][32][2] fp32 (merge)
-  static constexpr int kBytes = kMl + 2 * 32 * 2 * 4;
-  static_assert(2 * 64 * 64 * 4 <= FQ_NW * FQ_D * FQ_VTS * 2, "the merge slots reuse the V^T tiles");
+  static constexpr int kMl = kPar + FQ_NW * 2 * 32 * 4;                // [FQ_NW][32][2] fp32 (merge)
+  static constexpr int kBytes = kMl + FQ_NW * 32 * 2 * 4;
+  // the merge slots -- for every wavefront, a quarter of each other wavefront's accumulators --
+  // reuse the Q^T operands and the V^T tiles
+  static_assert(FQ_NW * (FQ_NW - 1) * 16 * 64 * 4 <= kPar - kQ, "room for the merge slots");
 };
 
 template <int BITS>
@@ -1478,6 +1481,7 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   constexpr int WPU = BITS == 8 ? 2 : 1;      // words per unit
   constexpr int OPU = BITS == 2 ? 2 : 1;      // octets per unit
   constexpr int IPL = 16 * UPR / 64;          // V items (two keys x one unit) per lane and block
+  static_assert(NDB == FQ_NW, "the merge gives every wavefront one 32-channel block of the output");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u32x4_t *const lds_q = reinterpret_cast<u32x4_t *>(lds_raw + FewQLds::kQ);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1486,18 +1490,105 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   float *const par = reinterpret_cast<float *>(lds_raw + FewQLds::kPar) + wave * 2 * 32;
   float *const lds_ml = reinterpret_cast<float *>(lds_raw + FewQLds::kMl);
 
-  // workgroup -> (batch * head, query tile, share), ids congruent mod 8 (one L2) for one (batch, head)
-  const int wg = blockIdx.x;
-  const int xcd = wg & 7, slot_s = wg >> 3;
-  const int split = slot_s % p.nsplit, slot = slot_s / p.nsplit;
-  const int bh = (slot / p.q_tiles) * 8 + xcd;
-  const int qt = slot % p.q_tiles;
+  // workgroup -> (batch * head, query tile, share) without a division: the grid is (8, shares,
+  // groups of eight (batch, head) x query tiles); x runs fastest in the dispatch order, so the
+  // workgroups of one (batch, head) sit on one XCD (one L2), as in the kernel above.
+  static_assert(kFewQueries <= 64, "at most two query tiles");
+  const int xcd = blockIdx.x, split = blockIdx.y, slot = blockIdx.z;
+  const int qt = p.q_tiles == 2 ? (slot & 1) : 0;
+  const int bh = (p.q_tiles == 2 ? (slot >> 1) : slot) * 8 + xcd;
   if (bh >= p.bh_total) return;
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
   const int hq = p.head_map ? p.head_map[hs] : hs;
 
+  const int qrow = qt * 32 + col;
+  const bool q_live = qrow < p.Lq;
+  int limit = p.kv_limit ? min(p.kv_limit[min(qrow, p.Lq - 1)], p.Lk) : p.Lk;
+  if (limit < 0) limit = 0;
+  // every wavefront holds the same queries: the largest and smallest limit need no exchange between them
+  int kv_end = q_live ? limit : 0, minlim = q_live ? limit : p.Lk;
+  if (p.kv_limit) {
+    for (int off = 1; off < 64; off <<= 1) {
+      kv_end = max(kv_end, __shfl_xor(kv_end, off, 64));
+      minlim = min(minlim, __shfl_xor(minlim, off, 64));
+    }
+  } else {
+    kv_end = p.Lk; minlim = p.Lk;   // (some query of the tile is live)
+  }
+  // the share's blocks: a fixed number per share (set by the host from Lk), cut at the tile's last key
+  const int nb = (kv_end + FQ_BK - 1) / FQ_BK;
+  const int b_begin = split * p.fq_share_blocks, b_end = min(b_begin + p.fq_share_blocks, nb);
+  // Block j of the share goes to wavefront (j + rot) % 4: the wavefront that gets the odd block
+  // more differs between the workgroups that are likely to sit on one compute unit.
+  const int slot_s = slot * p.nsplit + split;
+  const int rot = (slot_s + (slot_s >> 5)) & 3;
+  const int blk0 = b_begin + ((wave - rot) & 3);
+
+  u32 kmask = KCodec<BITS>::kMask;
+  asm volatile("" : "+v"(kmask));
+
+  // Packed words and parameters of a block as loaded.  The registers are refilled with the
+  // wavefront's next block as soon as the current one has used them: K after S^T, V after the
+  // V^T tile is written.  The requests are issued without conditions around them (past the end
+  // they re-read the last key row; a missing zero-point array reads the scales instead): with a
+  // branch around a load the compiler no longer knows how many loads are in flight and waits for
+  // all of them where it needs the oldest.
+  // Addresses: the (batch, head) bases are uniform; a lane keeps 32-bit byte offsets of its rows
+  // from them, advanced by four blocks per request and clamped at the last key (the host checks
+  // that they fit) -- an add and a min per stream instead of the products of key and strides.
+  const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
+  const char *const kw_base = reinterpret_cast<const char *>(p.k_words + kv_row0 * WPR);
+  const char *const vw_base = reinterpret_cast<const char *>(p.v_words + kv_row0 * WPR);
+  const char *const ks_base = reinterpret_cast<const char *>(p.k_scale + kv_row0);
+  const char *const kz_base = reinterpret_cast<const char *>((p.k_zp ? p.k_zp : p.k_scale) + kv_row0);
+  const char *const vs_base = reinterpret_cast<const char *>(p.v_scale + kv_row0);
+  const char *const vz_base = reinterpret_cast<const char *>((p.v_zp ? p.v_zp : p.v_scale) + kv_row0);
+  const bool has_kzp = p.k_zp != nullptr, has_vzp = p.v_zp != nullptr;
+  const u32 row_b = (u32)p.kv_ts * (WPR * 4), par_b = (u32)p.kv_ts * 4;   // bytes from one key to the next
+  const u32 par_last = (u32)(p.Lk - 1) * par_b;
+  const u32 k_lane = half * (HW * 4), v_lane = (lane >> 4) * (WPU * 4);     // this lane's place inside a row
+  const u32 k_row_last = (u32)(p.Lk - 1) * row_b + k_lane, v_row_last = (u32)(p.Lk - 1) * row_b + v_lane;
+  const u32 row_step = FQ_NW * FQ_BK * row_b, par_step = FQ_NW * FQ_BK * par_b;
+  // MFMA row `col` carries key kperm(col) of the block; V: item = lane + 64 i covers keys 2 kp, 2 kp + 1
+  // (kp = lane & 15: the lanes of a tile row write 16 adjacent banks) and unit (lane >> 4) + 4 i
+  u32 ok_row = (u32)(blk0 * FQ_BK + kperm(col)) * row_b + k_lane, ok_par = (u32)(blk0 * FQ_BK + kperm(col)) * par_b;
+  u32 ov_row = (u32)(blk0 * FQ_BK + 2 * (lane & 15)) * row_b + v_lane, ov_par = (u32)(blk0 * FQ_BK + col) * par_b;
+  u32x4_t kraw[KP];
+  u32 vraw[IPL][2][WPU];
+  float ksc, kzp, vsc, vzp;
+  auto umin = [](u32 x, u32 y) { return x < y ? x : y; };
+  auto request_k = [&]() {   // the wavefront's next block
+    const u32 orow = umin(ok_row, k_row_last), opar = umin(ok_par, par_last);
+    ok_row += row_step; ok_par += par_step;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) kraw[i] = *reinterpret_cast<const u32x4_t *>(kw_base + orow + 16 * i);
+    ksc = *reinterpret_cast<const float *>(ks_base + opar);
+    kzp = *reinterpret_cast<const float *>(kz_base + opar);
+  };
+  auto request_v = [&]() {
+    const u32 orow[2] = {umin(ov_row, v_row_last), umin(ov_row + row_b, v_row_last)};
+    const u32 opar = umin(ov_par, par_last);
+    ov_row += row_step; ov_par += par_step;
+#pragma unroll
+    for (int i = 0; i < IPL; ++i)
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const char *src = vw_base + orow[r] + i * (4 * WPU * 4);
+        if constexpr (WPU == 2) { const uint2 t = *reinterpret_cast<const uint2 *>(src); vraw[i][r][0] = t.x; vraw[i][r][1] = t.y; }
+        else vraw[i][r][0] = *reinterpret_cast<const u32 *>(src);
+      }
+    vsc = *reinterpret_cast<const float *>(vs_base + opar);
+    vzp = *reinterpret_cast<const float *>(vz_base + opar);
+  };
+  // the first block is on its way while the queries are staged
+  request_k();
+  request_v();
+
   // ---- the workgroup's 32 queries: Q^T operands to LDS, in the slot order of the K codec ----
-  for (int e = tid; e < NCH * 64; e += FQ_NW * 64) {
+  static_assert(NCH * 64 % (FQ_NW * 64) == 0, "whole passes");
+#pragma unroll
+  for (int it = 0; it < NCH * 64 / (FQ_NW * 64); ++it) {
+    const int e = tid + it * FQ_NW * 64;
     const int ch = e >> 6, l = e & 63;
     const int qr = min(qt * 32 + (l & 31), p.Lq - 1);
     const __bf16 *qp = p.q + (b * p.q_bs + hq * p.q_hs + qr * p.q_ts) * D + ((l >> 5) * 8 + ch) * 8;
@@ -1511,26 +1602,7 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
     }
     lds_q[e] = o;
   }
-  const int qrow = qt * 32 + col;
-  const bool q_live = qrow < p.Lq;
-  int limit = p.kv_limit ? min(p.kv_limit[min(qrow, p.Lq - 1)], p.Lk) : p.Lk;
-  if (limit < 0) limit = 0;
-  // every wavefront holds the same queries: the largest and smallest limit need no exchange between them
-  int kv_end = q_live ? limit : 0, minlim = q_live ? limit : p.Lk;
-  for (int off = 1; off < 64; off <<= 1) {
-    kv_end = max(kv_end, __shfl_xor(kv_end, off, 64));
-    minlim = min(minlim, __shfl_xor(minlim, off, 64));
-  }
-  const int nb = (kv_end + FQ_BK - 1) / FQ_BK;
-  const int b_begin = (int)((int64_t)nb * split / p.nsplit), b_end = (int)((int64_t)nb * (split + 1) / p.nsplit);
   __syncthreads();   // Q^T operands written
-
-  const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
-  const int64_t kv_ts = p.kv_ts;
-  const u32 *kw = p.k_words + kv_row0 * WPR;
-  const u32 *vw = p.v_words + kv_row0 * WPR;
-  u32 kmask = KCodec<BITS>::kMask;
-  asm volatile("" : "+v"(kmask));
 
   floatx16_t oacc[NDB];
 #pragma unroll
@@ -1540,65 +1612,16 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   float m_ref = 0.f, l_part = 0.f;
   bool first = true;
 
-  // packed words and parameters of one block, as loaded
-  u32x4_t kraw[KP];
-  u32 vraw[IPL][2][WPU];
-  float ksc, kzp, vsc, vzp;
-  auto request = [&](int blk) {
+  // One block of 32 keys.  BYTES: 4-bit codes through bytes (see byte_bias4), with the bias ka4
+  // of this lane's K row; V goes through bytes too if its zero-points fit.  The block's V words
+  // and parameters are not touched before its softmax is done: they were requested last.
+  auto block = [&](const int blk, auto bytes_tag, const u32 ka4) {
+    constexpr bool BYTES = decltype(bytes_tag)::value;
     const int t0 = blk * FQ_BK;
-    const int key = min(t0 + kperm(col), p.Lk - 1);       // MFMA row `col` carries key kperm(col) of the block
-    const u32 *src = kw + key * kv_ts * WPR + half * HW;
-#pragma unroll
-    for (int i = 0; i < KP; ++i) kraw[i] = *reinterpret_cast<const u32x4_t *>(src + 4 * i);
-    const int64_t g = kv_row0 + key * kv_ts;
-    ksc = p.k_scale[g];
-    kzp = p.k_zp ? p.k_zp[g] : 0.f;
-#pragma unroll
-    for (int i = 0; i < IPL; ++i) {
-      const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
-#pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const int vkey = min(t0 + 2 * kp + r, p.Lk - 1);
-        const u32 *vs_ = vw + vkey * kv_ts * WPR + u * WPU;
-        if constexpr (WPU == 2) { const uint2 t = *reinterpret_cast<const uint2 *>(vs_); vraw[i][r][0] = t.x; vraw[i][r][1] = t.y; }
-        else vraw[i][r][0] = vs_[0];
-      }
-    }
-    const int64_t gv = kv_row0 + min(t0 + col, p.Lk - 1) * kv_ts;
-    vsc = p.v_scale[gv];
-    vzp = p.v_zp ? p.v_zp[gv] : 0.f;
-  };
-
-  int blk = b_begin + wave;
-  if (blk < b_end) request(blk);
-  for (; blk < b_end; blk += FQ_NW) {
-    const int t0 = blk * FQ_BK;
-    // this block's operands out of the request registers (which the next block's request refills)
-    u32x4_t kcur[KP];
-    u32 vcur[IPL][2][WPU];
-#pragma unroll
-    for (int i = 0; i < KP; ++i) kcur[i] = kraw[i];
-#pragma unroll
-    for (int i = 0; i < IPL; ++i)
-#pragma unroll
-      for (int r = 0; r < 2; ++r)
-#pragma unroll
-        for (int w = 0; w < WPU; ++w) vcur[i][r][w] = vraw[i][r][w];
     // (code - zp) * scale = (raw - (zp + kOff) / kMul) * (kMul * scale) for the code image `raw`
-    const float zk = (kzp + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), sk = ksc * KCodec<BITS>::kMul;
-    // 4-bit codes: through bytes (see byte_bias4) unless a zero-point of the block does not fit
-    u32 ka4 = 0, va4 = 0;
-    bool bytes = false;
-    if constexpr (BITS == 4) {
-      const bool okk = byte_bias4(kzp, ka4), okv = byte_bias4(vzp, va4);
-      bytes = !__any(!(okk && okv));
-    }
+    const float kz = has_kzp ? kzp : 0.f;
+    const float zk = (kz + KCodec<BITS>::kOff) * (1.f / KCodec<BITS>::kMul), sk = ksc * KCodec<BITS>::kMul;
     const float ks_plain = ksc, kc = -128.f * ksc;
-    if (half == 0) {
-      par[col] = bytes ? u2f(va4) : (vzp + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
-      par[32 + col] = bytes ? vsc : vsc * VCodec<BITS>::kMul;
-    }
-    if (blk + FQ_NW < b_end) request(blk + FQ_NW);
 
     // ---- S^T = K Q^T, K dequantized in registers ----
     floatx16_t sacc;
@@ -1609,9 +1632,9 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
       const int pc = ch / OPQ, j = ch % OPQ;
       u32 q4[4];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) q4[w] = kcur[pc][w] ^ KCodec<BITS>::kStageXor;
+      for (int w = 0; w < 4; ++w) q4[w] = kraw[pc][w] ^ KCodec<BITS>::kStageXor;
       u32x4_t a;
-      if (BITS == 4 && bytes) {
+      if constexpr (BYTES) {
         const u32 e = (q4[j] & 0x0f0f0f0fu) + ka4, o = ((q4[j] >> 4) & 0x0f0f0f0fu) + ka4;
         // operand slots (2m, 2m+1) hold channels (m, m+4): bytes 0 and 2 of e are channels 0 and 4, ...
         a[0] = pack_bf16_rne(__builtin_fmaf(ubyte_f32(e, 0), ks_plain, kc), __builtin_fmaf(ubyte_f32(e, 2), ks_plain, kc));
@@ -1626,56 +1649,83 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
       }
       sacc = mfma_32x32x16<false>(a, lds_q[ch * 64 + lane], sacc);
     }
+    request_k();
 
     // ---- softmax of the block: register i <-> key t0 + 16*(i/8) + 8*half + i%8 ----
+    // The logits are taken against the reference as it stands (log2 domain) and the reference
+    // moves only when a weight would exceed 2^16, which the block's sum of weights shows -- the
+    // denominator needs that sum anyway, and the common block then has no search for the row
+    // maximum and no rescaling of the 64 output accumulators.
     float z[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) z[i] = p.scale_log2e * sacc[i];
+    for (int i = 0; i < 16; ++i) z[i] = __builtin_fmaf(p.scale_log2e, sacc[i], -m_ref);
     if (t0 + FQ_BK > minlim) {
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (t0 + 16 * (i >> 3) + 8 * half + (i & 7) >= limit) z[i] = -INFINITY;
     }
-    float zmax = z[0];
+    // Moves the reference to the row's current maximum: up only once something has been
+    // accumulated; the first block takes its maximum as it is (the accumulators are zero).
+    auto move_reference = [&]() {
+      float zmax = z[0];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
-    {
-      const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
-      zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
-    }
-    // the reference follows the running maximum; the accumulators are rescaled in every block
-    // (64 multiplications, mostly by one): a branch around them makes the compiler copy the
-    // accumulators at its join, which costs more
-    {
-      const float m_new = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(m_ref, zmax);
-      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
-      m_ref = m_new;
-      first = false;
-      l_part *= alpha;
+      for (int i = 1; i < 16; ++i) zmax = fmaxf(zmax, z[i]);
+      {
+        const auto sw = __builtin_amdgcn_permlane32_swap(f2u(zmax), f2u(zmax), false, false);
+        zmax = fmaxf(u2f(sw[0]), u2f(sw[1]));
+      }
+      const float delta = first ? ((zmax == -INFINITY) ? 0.f : zmax) : fmaxf(zmax, 0.f);
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      m_ref += delta;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] -= delta;
 #pragma unroll
       for (int d = 0; d < NDB; ++d)
 #pragma unroll
         for (int j = 0; j < 16; ++j) oacc[d][j] *= alpha;
-    }
+      l_part *= alpha;
+    };
     u32 pop[2][4];
+    float bsum = 0.f;
+    auto weights = [&]() {
+      bsum = 0.f;
 #pragma unroll
-    for (int i2 = 0; i2 < 8; ++i2) {
-      const int i = 2 * i2;
-      const u32 w = pack_bf16_rne(__builtin_amdgcn_exp2f(z[i] - m_ref), __builtin_amdgcn_exp2f(z[i + 1] - m_ref));
-      pop[i >> 3][(i & 7) >> 1] = w;
-      typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-      l_part = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), l_part, false);
+      for (int i2 = 0; i2 < 8; ++i2) {
+        const int i = 2 * i2;
+        const u32 w = pack_bf16_rne(__builtin_amdgcn_exp2f(z[i]), __builtin_amdgcn_exp2f(z[i + 1]));
+        pop[i >> 3][(i & 7) >> 1] = w;
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        bsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), bsum, false);
+      }
+    };
+    if (first) move_reference();
+    weights();
+    if (!first && __any(!(bsum <= 65536.f))) {
+      move_reference();
+      weights();
     }
+    l_part += bsum;
+    first = false;
 
     // ---- V of the block -> V^T tile of this wavefront (bf16 values) ----
+    bool vbytes = false;
+    {
+      u32 va4 = 0;
+      const float vz = has_vzp ? vzp : 0.f, vsc_ = vsc;
+      if constexpr (BYTES) vbytes = !__any(!byte_bias4(vz, va4));
+      if (half == 0) {
+        par[col] = vbytes ? u2f(va4) : (vz + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+        par[32 + col] = vbytes ? vsc_ : vsc_ * VCodec<BITS>::kMul;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < IPL; ++i) {
       const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
       u32 r0[WPU], r1[WPU];
 #pragma unroll
-      for (int w = 0; w < WPU; ++w) { r0[w] = vcur[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vcur[i][1][w] ^ VCodec<BITS>::kStageXor; }
+      for (int w = 0; w < WPU; ++w) { r0[w] = vraw[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vraw[i][1][w] ^ VCodec<BITS>::kStageXor; }
       const float2 z2 = *reinterpret_cast<const float2 *>(par + 2 * kp), s2 = *reinterpret_cast<const float2 *>(par + 32 + 2 * kp);
-      if (BITS == 4 && bytes) {
+      if (BYTES && vbytes) {
         // (z2 holds the two keys' byte biases, s2 their plain scales)
         const u32 e0 = (r0[0] & 0x0f0f0f0fu) + f2u(z2.x), o0 = ((r0[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.x);
         const u32 e1 = (r1[0] & 0x0f0f0f0fu) + f2u(z2.y), o1 = ((r1[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.y);
@@ -1687,18 +1737,20 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
           *reinterpret_cast<u32 *>(&vt[(u * 8 + 2 * j2 + 1) * FQ_VTS + kp * 2]) =
               pack_bf16_rne(__builtin_fmaf(ubyte_f32(o0, j2), s2.x, c0), __builtin_fmaf(ubyte_f32(o1, j2), s2.y, c1));
         }
-        continue;
-      }
+      } else {
 #pragma unroll
-      for (int o = 0; o < OPU; ++o) {
-        float f0[8], f1[8];
-        v_pair_values<BITS>(r0, r1, o, kmask, f0, f1);
-        const int oct = u * OPU + o;
+        for (int o = 0; o < OPU; ++o) {
+          float f0[8], f1[8];
+          v_pair_values<BITS>(r0, r1, o, kmask, f0, f1);
+          const int oct = u * OPU + o;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * FQ_VTS + kp * 2]) = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
+          for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * FQ_VTS + kp * 2]) = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
+        }
       }
     }
+    request_v();
+
     // ---- O^T += V^T P^T ----
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -1709,60 +1761,104 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
         oacc[d] = mfma_32x32x16<false>(av, bv, oacc[d]);
       }
     }
-  }
+  };
 
-  // ---- merge the wavefronts' partial results: 2 and 3 into 0 and 1, then 1 into 0 ----
-  float l_sum = l_part + __shfl_xor(l_part, 32, 64);
-  float *const slots = reinterpret_cast<float *>(lds_raw + FewQLds::kVt);   // [2][64 registers][64 lanes]
-#pragma unroll
-  for (int stride = 2; stride >= 1; stride >>= 1) {
-    __syncthreads();   // (first round: every wavefront is done with its V^T tile)
-    if (wave >= stride && wave < 2 * stride) {
-      float *dst = slots + (wave - stride) * 64 * 64;
-#pragma unroll
-      for (int d = 0; d < NDB; ++d)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) dst[(d * 16 + j) * 64 + lane] = oacc[d][j];
-      if (half == 0) { lds_ml[((wave - stride) * 32 + col) * 2] = m_ref; lds_ml[((wave - stride) * 32 + col) * 2 + 1] = l_sum; }
-    }
-    __syncthreads();
-    if (wave < stride) {
-      const float *src = slots + wave * 64 * 64;
-      const float mb = lds_ml[(wave * 32 + col) * 2], lb = lds_ml[(wave * 32 + col) * 2 + 1];
-      const bool has_a = l_sum > 0.f, has_b = lb > 0.f;
-      const float M = (has_a && has_b) ? fmaxf(m_ref, mb) : has_b ? mb : m_ref;
-      const float wa = has_a ? __builtin_amdgcn_exp2f(m_ref - M) : 0.f, wb = has_b ? __builtin_amdgcn_exp2f(mb - M) : 0.f;
-#pragma unroll
-      for (int d = 0; d < NDB; ++d)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) oacc[d][j] = oacc[d][j] * wa + src[(d * 16 + j) * 64 + lane] * wb;
-      l_sum = l_sum * wa + lb * wb;
-      m_ref = M;
+  // 4-bit codes go through bytes until a K zero-point of a block does not fit; from there on (and
+  // for the other widths) the general form.  Two loops one after the other rather than two arms
+  // inside one: arms that both update the output accumulators make the compiler copy them at
+  // the join, twice per block.
+  int blk = blk0;
+  if constexpr (BITS == 4) {
+    for (; blk < b_end; blk += FQ_NW) {
+      u32 ka4 = 0;
+      if (__any(!byte_bias4(has_kzp ? kzp : 0.f, ka4))) break;
+      block(blk, std::true_type{}, ka4);
     }
   }
-  if (wave != 0 || !q_live) return;
+  for (; blk < b_end; blk += FQ_NW) block(blk, std::false_type{}, 0u);
+
+  // ---- merge the wavefronts' partial results: wavefront t ends up with channels 32t .. 32t+31 ----
+  // Every wavefront hands the other three their quarters of its accumulators through LDS (one
+  // barrier on each side), forms the four weights from everyone's (m, l) and sums its quarter.
+  const float l_own = l_part + __shfl_xor(l_part, 32, 64);
+  float *const slots = reinterpret_cast<float *>(lds_raw + FewQLds::kQ);   // [target][source - target - 1 mod 4][16 registers][64 lanes]
+  __syncthreads();   // every wavefront is done with the Q^T operands and its V^T tile
+#pragma unroll
+  for (int t = 0; t < FQ_NW; ++t) {
+    if (t == wave) continue;
+    float *dst = slots + ((t * 3 + ((wave - t - 1) & 3)) * 16) * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) dst[j * 64] = oacc[t][j];
+  }
+  if (half == 0) *reinterpret_cast<float2 *>(lds_ml + (wave * 32 + col) * 2) = make_float2(m_ref, l_own);
+  __syncthreads();
+  // (the partial results are addressed through LDS, not through register arrays with a run-time index)
+  float M = 0.f;
+  bool any_live = false;
+#pragma unroll
+  for (int w = 0; w < FQ_NW; ++w) {
+    const float2 ml = *reinterpret_cast<const float2 *>(lds_ml + (w * 32 + col) * 2);
+    if (ml.y > 0.f) { M = any_live ? fmaxf(M, ml.x) : ml.x; any_live = true; }
+  }
+  auto weight_of = [&](int w, float &l_w) {
+    const float2 ml = *reinterpret_cast<const float2 *>(lds_ml + (w * 32 + col) * 2);
+    l_w = ml.y;
+    return ml.y > 0.f ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;
+  };
+  float l_sum = 0.f;   // (summed in the same order by every wavefront)
+#pragma unroll
+  for (int w = 0; w < FQ_NW; ++w) {
+    float l_w;
+    const float wt = weight_of(w, l_w);
+    l_sum = __builtin_fmaf(l_w, wt, l_sum);
+  }
+  float mine[16];
+  {
+    float l_w;
+    const float w_own = weight_of(wave, l_w);
+#pragma unroll
+    for (int t = 0; t < FQ_NW; ++t)
+      if (t == wave) {   // (a wavefront-uniform choice among the four accumulator blocks)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) mine[j] = oacc[t][j] * w_own;
+      }
+  }
+#pragma unroll
+  for (int s = 0; s < FQ_NW - 1; ++s) {
+    float l_w;
+    const float ws = weight_of((wave + 1 + s) & 3, l_w);
+    const float *src = slots + ((wave * 3 + s) * 16) * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) mine[j] = __builtin_fmaf(src[j * 64], ws, mine[j]);
+  }
+  if (!q_live) return;
   const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
-  __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D;
-  const bool shared_out = p.nsplit > 1;
-  const int64_t prow = ((int64_t)split * p.bh_total + bh) * p.Lq + qrow;
-  float *wptr = p.ws_o + prow * D;
-  if (shared_out && half == 0) *reinterpret_cast<float2 *>(p.ws_ml + prow * 2) = make_float2(m_ref, l_sum);
+  // registers 4*g4 .. 4*g4+3 are rows 32*wave + 8*g4 + 4*half + 0..3 of O^T
+  if (p.nsplit > 1) {
+    const int64_t prow = ((int64_t)split * p.bh_total + bh) * p.Lq + qrow;
+    float *wptr = p.ws_o + prow * D + wave * 32 + 4 * half;
+    if (wave == 0 && half == 0) *reinterpret_cast<float2 *>(p.ws_ml + prow * 2) = make_float2(M, l_sum);
 #pragma unroll
-  for (int d = 0; d < NDB; ++d)
+    for (int g4 = 0; g4 < 4; ++g4)
+      *reinterpret_cast<float4 *>(wptr + 8 * g4) = make_float4(mine[4 * g4] * inv, mine[4 * g4 + 1] * inv, mine[4 * g4 + 2] * inv, mine[4 * g4 + 3] * inv);
+  } else {
+    __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D + wave * 32 + 4 * half;
 #pragma unroll
-    for (int g4 = 0; g4 < 4; ++g4) {
-      // registers 4*g4 .. 4*g4+3 are rows d*32 + 8*g4 + 4*half + 0..3 of O^T
-      const float o0 = oacc[d][4 * g4 + 0] * inv, o1 = oacc[d][4 * g4 + 1] * inv, o2 = oacc[d][4 * g4 + 2] * inv, o3 = oacc[d][4 * g4 + 3] * inv;
-      if (shared_out) *reinterpret_cast<float4 *>(wptr + d * 32 + 8 * g4 + 4 * half) = make_float4(o0, o1, o2, o3);
-      else *reinterpret_cast<uint2 *>(optr + d * 32 + 8 * g4 + 4 * half) = make_uint2(pack_bf16_rne(o0, o1), pack_bf16_rne(o2, o3));
-    }
+    for (int g4 = 0; g4 < 4; ++g4)
+      *reinterpret_cast<uint2 *>(optr + 8 * g4) =
+          make_uint2(pack_bf16_rne(mine[4 * g4] * inv, mine[4 * g4 + 1] * inv), pack_bf16_rne(mine[4 * g4 + 2] * inv, mine[4 * g4 + 3] * inv));
+  }
 }
 
 // Whether a launch takes the few-queries kernel, and over how many workgroups the keys of a
 // (batch, head, 32 queries) are shared out then: enough for the two resident workgroups per
 // compute unit (the kernel holds ~200 registers), at least eight blocks per workgroup.
-bool fewq_eligible(int Lq, int Lk, int D, int k_group, int v_group) {
-  return D == FQ_D && k_group == D && v_group == D && Lq > 0 && Lq <= kFewQueries && Lk >= kFewQMinKeys;
+bool fewq_eligible(int B, int Hkv, int Lq, int Lk, int D, int k_group, int v_group) {
+  // (the kernel keeps 32-bit byte offsets inside one (batch, head): rows of up to D bytes, up to
+  // Hkv rows from one key to the next, a few blocks of overshoot before the clamp)
+  return D == FQ_D && k_group == D && v_group == D && Lq > 0 && Lq <= kFewQueries && Lk >= kFewQMinKeys &&
+         ((int64_t)Lk + 8 * FQ_BK) * Hkv * D < (1ll << 32) &&
+         ((int64_t)B * Hkv + 7) / 8 * ((Lq + 31) / 32) <= 65535;   // (the grid's z extent)
 }
 int fewq_shares(int bh_total, int Lq, int Lk) {
   const int64_t tiles = (int64_t)((bh_total + 7) / 8 * 8) * ((Lq + 31) / 32);
@@ -1775,7 +1871,7 @@ int fewq_shares(int bh_total, int Lq, int Lk) {
 
 template <int BITS> void launch_fewq(const AttnParams &p, hipStream_t st) {
   const int bh_pad = (p.bh_total + 7) / 8 * 8;
-  dim3 grid((unsigned)(bh_pad * p.q_tiles * p.nsplit));
+  dim3 grid(8, (unsigned)p.nsplit, (unsigned)(bh_pad / 8 * p.q_tiles));
   hipLaunchKernelGGL((fused_attn_fewq_kernel<BITS>), grid, dim3(FQ_NW * 64), FewQLds::kBytes, st, p);
   if (p.nsplit > 1) {
     const int64_t rows = (int64_t)p.bh_total * p.Lq;
@@ -1793,13 +1889,13 @@ extern "C" size_t varq_fused_attn_workspace_bytes(int B, int Hkv, int Lq, int Lk
   int n = splits ? splits : choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), tiles, rows, D);
   // (the group sizes are not known here: room for the few-queries kernel's shares whenever the
   // other sizes would admit it)
-  if (splits == 0 && fewq_eligible(Lq, Lk, D, D, D)) n = max(n, fewq_shares(B * Hkv, Lq, Lk));
+  if (splits == 0 && fewq_eligible(B, Hkv, Lq, Lk, D, D, D)) n = max(n, fewq_shares(B * Hkv, Lq, Lk));
   return split_workspace_bytes(n, rows, D);
 }
 
 extern "C" int varq_fused_attn_key_shares(int B, int Hkv, int Lq, int Lk, int D, int k_group, int v_group) {
   if (B <= 0 || Hkv <= 0 || Lq <= 0 || Lk <= 0 || (D != 64 && D != 128)) return 0;
-  if (fewq_eligible(Lq, Lk, D, k_group, v_group)) return fewq_shares(B * Hkv, Lq, Lk);
+  if (fewq_eligible(B, Hkv, Lq, Lk, D, k_group, v_group)) return fewq_shares(B * Hkv, Lq, Lk);
   return choose_splits((int64_t)B * Hkv * ((Lq + BM - 1) / BM), (Lk + BN - 1) / BN, (int64_t)B * Hkv * Lq, D);
 }
 
@@ -1845,18 +1941,20 @@ extern "C" int varq_fused_attn(const void *q, void *out,
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
+  p.fq_share_blocks = 0;
   p.scale_log2e = softmax_scale * kLog2e;
   p.f16 = io_dtype == VARQ_F16;
   p.exact_codes = operand_form == VARQ_ATTN_EXACT_CODES && !p.f16;
   if (int e = set_layout(p, layout, "fused_attn")) return e;
   hipStream_t st = (hipStream_t)stream;
   // few queries over a long cache, left to the library: the kernel whose wavefronts share the keys
-  if (splits == 0 && !p.f16 && !p.exact_codes && fewq_eligible(Lq, Lk, D, k_group, v_group)) {
+  if (splits == 0 && !p.f16 && !p.exact_codes && fewq_eligible(B, Hkv, Lq, Lk, D, k_group, v_group)) {
     const int64_t rows = (int64_t)p.bh_total * Lq;
     int n = fewq_shares(p.bh_total, Lq, Lk);
     while (n > 1 && (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < split_workspace_bytes(n, rows, D))) --n;
     p.q_tiles = (Lq + 31) / 32;
     p.nsplit = n;
+    p.fq_share_blocks = ((Lk + FQ_BK - 1) / FQ_BK + n - 1) / n;
     p.ws_o = n > 1 ? reinterpret_cast<float *>(workspace) : nullptr;
     p.ws_ml = n > 1 ? p.ws_o + (size_t)n * (size_t)rows * (size_t)D : nullptr;
     if (k_bits == 4) launch_fewq<4>(p, st);
@@ -1935,6 +2033,7 @@ extern "C" int varq_fused_attn_channel(const void *q, void *out,
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.Lstride = Lk_stride;
   p.q_tiles = (Lq + BM - 1) / BM;
   p.bh_total = B * Hkv;
+  p.fq_share_blocks = 0;
   p.scale_log2e = softmax_scale * kLog2e;
   p.f16 = io_dtype == VARQ_F16;
   p.exact_codes = 0;
