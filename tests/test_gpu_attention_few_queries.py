@@ -129,3 +129,84 @@ def test_seeded_random_shapes(dev, seed):
         heads = sorted(set(r(0, H - 1) for _ in range(2)))
     _case(dev, B, H, Lq, Lk, bits, seed=700 + seed, dist=('normal', 'student4')[seed % 2], limit=seed % 3 == 0,
           layout=('BHLc', 'BLHc')[(seed // 2) % 2] if heads is None else 'BHLc', Lstride=Lk + r(1, 200) if seed % 5 == 2 else None, heads=heads)
+
+
+@pytest.mark.parametrize('bits', [4, 8])
+def test_zero_points_outside_the_byte_form(dev, bits):
+    """4-bit codes are dequantized through bytes while the zero-points are integers of small
+    size and through the general form from the first block on where a K zero-point is not (and
+    per block for V): fractional and large zero-points set in here and there along the keys,
+    against the oracle's dequantization with the same parameters."""
+    B, H, Lq, Lk, D, g = 1, 2, 24, 3000, 128, 128
+    gen = torch.Generator().manual_seed(321 + bits)
+    k, v = O.synth_kv((B, H, Lk, D), 5, 'normal').bfloat16(), O.synth_kv((B, H, Lk, D), 6, 'normal').bfloat16()
+    q = torch.randn(B, H, Lq, D, generator=gen).bfloat16()
+    kq, ks, kz = O.quant_groupwise(k, g, bits, True)
+    vq, vs, vz = O.quant_groupwise(v, g, bits, True)
+    kz, vz = kz.clone(), vz.clone()
+    kz[:, 0, 1700:] += 0.5          # head 0: every wavefront reaches a fractional K zero-point on its way
+    kz[:, 1, 2999] = 300.0          # head 1: only the last key's, far outside a byte
+    vz[:, 0, 40:45] -= 0.25         # V: a few keys of one block ...
+    vz[:, 1, 1000:2000] = -200.0    # ... and a long run of blocks
+    kd, vd = O.dequant_groupwise(kq, ks, kz, g), O.dequant_groupwise(vq, vs, vz, g)
+    scale = 1.0 / math.sqrt(D)
+    note('few queries, zero-points outside the byte form', bits)
+    put = lambda t: t.to(dev)
+    args = [put(O.pack_last_dim(kq, bits)[0]), put(ks), put(kz), put(O.pack_last_dim(vq, bits)[0]), put(vs), put(vz)]
+    assert _lib.load().varq_fused_attn_key_shares(B, H, Lq, Lk, D, g, g) > 1
+    out = ops.fused_attn(put(q), *args, bits, bits, Lk, scale)
+    general = ops.fused_attn(put(q), *args, bits, bits, Lk, scale, splits=1)
+    torch.cuda.synchronize()
+    _compare(out, O.attention_ref(q, kd, vd, scale, None), _exact_fp64(q, kd, vd, scale, None, dev), f'few queries, odd zero-points, int{bits}')
+    span = max(1.0, float(general.float().abs().max()))
+    assert float((out.float() - general.float()).abs().max()) <= span * 2 ** -6
+
+
+def _range_profile(name, Lk):
+    t = torch.arange(Lk, dtype=torch.float32) / (Lk - 1)
+    if name == 'up':
+        return 4 * t - 2
+    if name == 'down':
+        return 2 - 4 * t
+    if name == 'step':                       # one jump in the middle of a 32-key block
+        return torch.where(torch.arange(Lk) < 1113, -2.0, 2.0)
+    if name == 'saw':                        # up in five teeth, each higher than the last
+        return (5 * t).frac() * 1.5 - 2 + 2.5 * t
+    if name == 'late':                       # flat, then the last key alone far above the rest
+        c = torch.full((Lk,), -1.0)
+        c[-1] = 2.0
+        return c
+    raise ValueError(name)
+
+
+@pytest.mark.parametrize('prof', ['up', 'down', 'step', 'saw', 'late'])
+@pytest.mark.parametrize('bits,limit', [(4, False), (8, True)])
+def test_softmax_range(dev, prof, bits, limit):
+    """Logits that rise, fall, jump or zig-zag by up to ~200 octaves along the keys, with queries of
+    both signs and several gains side by side: the softmax reference of the kernel moves in some
+    lanes and not in others, once or many times (the yardstick is that of
+    test_gpu_attention_softmax_range.py)."""
+    from test_gpu_attention_softmax_range import _check
+    B, H, Lq, Lk, D, g = 1, 2, 50, 1500, 128, 128
+    gen = torch.Generator().manual_seed(77 + bits)
+    w = torch.where(torch.rand(D, generator=gen) < 0.5, -1.0, 1.0)
+    c = _range_profile(prof, Lk)
+    k = (c[:, None] * w[None, :] + 0.2 * torch.randn(H, Lk, D, generator=gen)).unsqueeze(0).bfloat16()
+    v = torch.randn(B, H, Lk, D, generator=gen).bfloat16()
+    gain = torch.tensor([1.0, -1.0, 0.3, -0.3, 0.05, 0.0, 0.7])[torch.arange(Lq) % 7]
+    q = (3.0 * gain[:, None] * w[None, :] + 0.1 * torch.randn(H, Lq, D, generator=gen)).unsqueeze(0).bfloat16()
+    lim = bias = None
+    if limit:
+        lim = torch.randint(1, Lk + 1, (Lq,), generator=gen).int()
+        bias = torch.zeros(Lq, Lk)
+        bias[torch.arange(Lk)[None, :] >= lim[:, None].long()] = float('-inf')
+    kw, ks, kz, kd = _quantize(k, g, bits)
+    vw, vs, vz, vd = _quantize(v, g, bits)
+    scale = 1.0 / math.sqrt(D)
+    note('few queries, softmax range', prof, bits, limit)
+    put = lambda t: None if t is None else t.to(dev)
+    assert _lib.load().varq_fused_attn_key_shares(B, H, Lq, Lk, D, g, g) > 1
+    out = ops.fused_attn(put(q), put(kw), put(ks), put(kz), put(vw), put(vs), put(vz), bits, bits, Lk, scale, kv_limit=put(lim))
+    torch.cuda.synchronize()
+    _check(out, O.attention_ref(q, kd, vd, scale, bias), O.attention_exact(q.float(), kd, vd, scale, bias),
+           f'few queries, softmax range {prof} int{bits}' + (' limit' if limit else ''))

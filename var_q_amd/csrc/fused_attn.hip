@@ -1448,10 +1448,13 @@ int set_splits(AttnParams &p, int D, int tiles, int splits, void *workspace, siz
 //  * V: a lane widens items of two adjacent keys x 8 channels into a wavefront-private V^T tile
 //    in LDS (the second contraction runs over keys), read back as MFMA A operands by the same
 //    wavefront -- LDS requests of one wavefront are served in order, so no barrier is needed;
-//  * online softmax per lane against the running maximum;
-//  * the next block's packed words are requested before the current block's arithmetic.
-// The wavefronts' partial results are merged through LDS (two rounds), the workgroups' shares
-// through the workspace and combine_splits_kernel, as for the kernel above.
+//  * online softmax per lane against a reference that moves only when a weight would pass 2^16;
+//  * a block runs S^T, then the V^T tile (under the S^T MFMAs), then the softmax, then O^T; the
+//    wavefront's next block is requested piece by piece as the current one frees its registers
+//    (K after S^T, V after the tile), each about a block's time ahead of its use.
+// The wavefronts' partial results are merged through LDS (each wavefront ends up with a quarter
+// of the channels), the workgroups' shares through the workspace and combine_splits_kernel, as
+// for the kernel above.
 // One scale group per key (group = D = 128), bf16, any layout, key limits, head maps.
 constexpr int FQ_NW = 4;             // wavefronts per workgroup
 constexpr int FQ_BK = 32;            // keys per block: one 32-row MFMA block
@@ -1613,8 +1616,7 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   bool first = true;
 
   // One block of 32 keys.  BYTES: 4-bit codes through bytes (see byte_bias4), with the bias ka4
-  // of this lane's K row; V goes through bytes too if its zero-points fit.  The block's V words
-  // and parameters are not touched before its softmax is done: they were requested last.
+  // of this lane's K row; V goes through bytes too if its zero-points fit.
   auto block = [&](const int blk, auto bytes_tag, const u32 ka4) {
     constexpr bool BYTES = decltype(bytes_tag)::value;
     const int t0 = blk * FQ_BK;
@@ -1650,6 +1652,50 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
       sacc = mfma_32x32x16<false>(a, lds_q[ch * 64 + lane], sacc);
     }
     request_k();
+
+    // ---- V of the block -> V^T tile of this wavefront (bf16 values) ----
+    bool vbytes = false;
+    {
+      u32 va4 = 0;
+      const float vz = has_vzp ? vzp : 0.f, vsc_ = vsc;
+      if constexpr (BYTES) vbytes = !__any(!byte_bias4(vz, va4));
+      if (half == 0) {
+        par[col] = vbytes ? u2f(va4) : (vz + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+        par[32 + col] = vbytes ? vsc_ : vsc_ * VCodec<BITS>::kMul;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < IPL; ++i) {
+      const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
+      u32 r0[WPU], r1[WPU];
+#pragma unroll
+      for (int w = 0; w < WPU; ++w) { r0[w] = vraw[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vraw[i][1][w] ^ VCodec<BITS>::kStageXor; }
+      const float2 z2 = *reinterpret_cast<const float2 *>(par + 2 * kp), s2 = *reinterpret_cast<const float2 *>(par + 32 + 2 * kp);
+      if (BYTES && vbytes) {
+        // (z2 holds the two keys' byte biases, s2 their plain scales)
+        const u32 e0 = (r0[0] & 0x0f0f0f0fu) + f2u(z2.x), o0 = ((r0[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.x);
+        const u32 e1 = (r1[0] & 0x0f0f0f0fu) + f2u(z2.y), o1 = ((r1[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.y);
+        const float c0 = -128.f * s2.x, c1 = -128.f * s2.y;
+#pragma unroll
+        for (int j2 = 0; j2 < 4; ++j2) {
+          *reinterpret_cast<u32 *>(&vt[(u * 8 + 2 * j2) * FQ_VTS + kp * 2]) =
+              pack_bf16_rne(__builtin_fmaf(ubyte_f32(e0, j2), s2.x, c0), __builtin_fmaf(ubyte_f32(e1, j2), s2.y, c1));
+          *reinterpret_cast<u32 *>(&vt[(u * 8 + 2 * j2 + 1) * FQ_VTS + kp * 2]) =
+              pack_bf16_rne(__builtin_fmaf(ubyte_f32(o0, j2), s2.x, c0), __builtin_fmaf(ubyte_f32(o1, j2), s2.y, c1));
+        }
+      } else {
+#pragma unroll
+        for (int o = 0; o < OPU; ++o) {
+          float f0[8], f1[8];
+          v_pair_values<BITS>(r0, r1, o, kmask, f0, f1);
+          const int oct = u * OPU + o;
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * FQ_VTS + kp * 2]) = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
+        }
+      }
+    }
+    request_v();
 
     // ---- softmax of the block: register i <-> key t0 + 16*(i/8) + 8*half + i%8 ----
     // The logits are taken against the reference as it stands (log2 domain) and the reference
@@ -1706,50 +1752,6 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
     }
     l_part += bsum;
     first = false;
-
-    // ---- V of the block -> V^T tile of this wavefront (bf16 values) ----
-    bool vbytes = false;
-    {
-      u32 va4 = 0;
-      const float vz = has_vzp ? vzp : 0.f, vsc_ = vsc;
-      if constexpr (BYTES) vbytes = !__any(!byte_bias4(vz, va4));
-      if (half == 0) {
-        par[col] = vbytes ? u2f(va4) : (vz + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
-        par[32 + col] = vbytes ? vsc_ : vsc_ * VCodec<BITS>::kMul;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < IPL; ++i) {
-      const int item = lane + 64 * i, kp = item & 15, u = item >> 4;   // (key pair fastest: the lanes of a row write 16 adjacent banks)
-      u32 r0[WPU], r1[WPU];
-#pragma unroll
-      for (int w = 0; w < WPU; ++w) { r0[w] = vraw[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vraw[i][1][w] ^ VCodec<BITS>::kStageXor; }
-      const float2 z2 = *reinterpret_cast<const float2 *>(par + 2 * kp), s2 = *reinterpret_cast<const float2 *>(par + 32 + 2 * kp);
-      if (BYTES && vbytes) {
-        // (z2 holds the two keys' byte biases, s2 their plain scales)
-        const u32 e0 = (r0[0] & 0x0f0f0f0fu) + f2u(z2.x), o0 = ((r0[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.x);
-        const u32 e1 = (r1[0] & 0x0f0f0f0fu) + f2u(z2.y), o1 = ((r1[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.y);
-        const float c0 = -128.f * s2.x, c1 = -128.f * s2.y;
-#pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) {
-          *reinterpret_cast<u32 *>(&vt[(u * 8 + 2 * j2) * FQ_VTS + kp * 2]) =
-              pack_bf16_rne(__builtin_fmaf(ubyte_f32(e0, j2), s2.x, c0), __builtin_fmaf(ubyte_f32(e1, j2), s2.y, c1));
-          *reinterpret_cast<u32 *>(&vt[(u * 8 + 2 * j2 + 1) * FQ_VTS + kp * 2]) =
-              pack_bf16_rne(__builtin_fmaf(ubyte_f32(o0, j2), s2.x, c0), __builtin_fmaf(ubyte_f32(o1, j2), s2.y, c1));
-        }
-      } else {
-#pragma unroll
-        for (int o = 0; o < OPU; ++o) {
-          float f0[8], f1[8];
-          v_pair_values<BITS>(r0, r1, o, kmask, f0, f1);
-          const int oct = u * OPU + o;
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<u32 *>(&vt[(oct * 8 + j) * FQ_VTS + kp * 2]) = pack_bf16_rne((f0[j] - z2.x) * s2.x, (f1[j] - z2.y) * s2.y);
-        }
-      }
-    }
-    request_v();
 
     // ---- O^T += V^T P^T ----
 #pragma unroll
