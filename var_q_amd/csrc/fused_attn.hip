@@ -1464,14 +1464,12 @@ constexpr int kFewQueries = 64;      // launches with at most this many queries 
 constexpr int kFewQMinKeys = 1024;   // ... over at least this many keys take this kernel
 constexpr int kMaxKeyShares = kMaxKeyShares_v;
 struct FewQLds {
-  static constexpr int kQ = 0;                                         // [8][64] 16-byte Q^T operands
-  static constexpr int kVt = kQ + 8 * 64 * 16;                         // [FQ_NW][D][FQ_VTS] bf16
-  static constexpr int kPar = kVt + FQ_NW * FQ_D * FQ_VTS * 2;         // [FQ_NW][2][32] fp32
-  static constexpr int kMl = kPar + FQ_NW * 2 * 32 * 4;                // [FQ_NW][32][2] fp32 (merge)
-  static constexpr int kBytes = kMl + FQ_NW * 32 * 2 * 4;
+  static constexpr int kVt = 0;                                        // [FQ_NW][D][FQ_VTS] bf16
   // the merge slots -- for every wavefront, a quarter of each other wavefront's accumulators --
-  // reuse the Q^T operands and the V^T tiles
-  static_assert(FQ_NW * (FQ_NW - 1) * 16 * 64 * 4 <= kPar - kQ, "room for the merge slots");
+  // start at the V^T tiles and need a little more
+  static constexpr int kSlotBytes = FQ_NW * (FQ_NW - 1) * 16 * 64 * 4;
+  static constexpr int kMl = kVt + (FQ_NW * FQ_D * FQ_VTS * 2 > kSlotBytes ? FQ_NW * FQ_D * FQ_VTS * 2 : kSlotBytes);   // [FQ_NW][32][2] fp32 (merge)
+  static constexpr int kBytes = kMl + FQ_NW * 32 * 2 * 4;
 };
 
 template <int BITS>
@@ -1486,11 +1484,9 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   constexpr int IPL = 16 * UPR / 64;          // V items (two keys x one unit) per lane and block
   static_assert(NDB == FQ_NW, "the merge gives every wavefront one 32-channel block of the output");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  u32x4_t *const lds_q = reinterpret_cast<u32x4_t *>(lds_raw + FewQLds::kQ);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, half = lane >> 5;
   uint16_t *const vt = reinterpret_cast<uint16_t *>(lds_raw + FewQLds::kVt) + wave * D * FQ_VTS;
-  float *const par = reinterpret_cast<float *>(lds_raw + FewQLds::kPar) + wave * 2 * 32;
   float *const lds_ml = reinterpret_cast<float *>(lds_raw + FewQLds::kMl);
 
   // workgroup -> (batch * head, query tile, share) without a division: the grid is (8, shares,
@@ -1555,10 +1551,10 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   // MFMA row `col` carries key kperm(col) of the block; V: item = lane + 64 i covers keys 2 kp, 2 kp + 1
   // (kp = lane & 15: the lanes of a tile row write 16 adjacent banks) and unit (lane >> 4) + 4 i
   u32 ok_row = (u32)(blk0 * FQ_BK + kperm(col)) * row_b + k_lane, ok_par = (u32)(blk0 * FQ_BK + kperm(col)) * par_b;
-  u32 ov_row = (u32)(blk0 * FQ_BK + 2 * (lane & 15)) * row_b + v_lane, ov_par = (u32)(blk0 * FQ_BK + col) * par_b;
+  u32 ov_row = (u32)(blk0 * FQ_BK + 2 * (lane & 15)) * row_b + v_lane, ov_par = (u32)(blk0 * FQ_BK + 2 * (lane & 15)) * par_b;
   u32x4_t kraw[KP];
   u32 vraw[IPL][2][WPU];
-  float ksc, kzp, vsc, vzp;
+  float ksc, kzp, vsc[2], vzp[2];   // (V: of this lane's two keys)
   auto umin = [](u32 x, u32 y) { return x < y ? x : y; };
   auto request_k = [&]() {   // the wavefront's next block
     const u32 orow = umin(ok_row, k_row_last), opar = umin(ok_par, par_last);
@@ -1570,8 +1566,13 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   };
   auto request_v = [&]() {
     const u32 orow[2] = {umin(ov_row, v_row_last), umin(ov_row + row_b, v_row_last)};
-    const u32 opar = umin(ov_par, par_last);
+    const u32 opar[2] = {umin(ov_par, par_last), umin(ov_par + par_b, par_last)};
     ov_row += row_step; ov_par += par_step;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {   // (the parameters first: the block's V work starts with them)
+      vsc[r] = *reinterpret_cast<const float *>(vs_base + opar[r]);
+      vzp[r] = *reinterpret_cast<const float *>(vz_base + opar[r]);
+    }
 #pragma unroll
     for (int i = 0; i < IPL; ++i)
 #pragma unroll
@@ -1580,32 +1581,32 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
         if constexpr (WPU == 2) { const uint2 t = *reinterpret_cast<const uint2 *>(src); vraw[i][r][0] = t.x; vraw[i][r][1] = t.y; }
         else vraw[i][r][0] = *reinterpret_cast<const u32 *>(src);
       }
-    vsc = *reinterpret_cast<const float *>(vs_base + opar);
-    vzp = *reinterpret_cast<const float *>(vz_base + opar);
   };
-  // the first block is on its way while the queries are staged
-  request_k();
-  request_v();
-
-  // ---- the workgroup's 32 queries: Q^T operands to LDS, in the slot order of the K codec ----
-  static_assert(NCH * 64 % (FQ_NW * 64) == 0, "whole passes");
+  // ---- this lane's query: the eight Q^T operands (channels in the slot order of the K codec)
+  // stay in registers for the whole key loop; the loads go out ahead of the first block's ----
+  u32x4_t qop[NCH];
+  {
+    const __bf16 *qp = p.q + (b * p.q_bs + hq * p.q_hs + min(qrow, p.Lq - 1) * p.q_ts) * D + half * 64;
 #pragma unroll
-  for (int it = 0; it < NCH * 64 / (FQ_NW * 64); ++it) {
-    const int e = tid + it * FQ_NW * 64;
-    const int ch = e >> 6, l = e & 63;
-    const int qr = min(qt * 32 + (l & 31), p.Lq - 1);
-    const __bf16 *qp = p.q + (b * p.q_bs + hq * p.q_hs + qr * p.q_ts) * D + ((l >> 5) * 8 + ch) * 8;
-    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(qp);
-    u32x4_t o;
+    for (int ch = 0; ch < NCH; ++ch) qop[ch] = *reinterpret_cast<const u32x4_t *>(qp + ch * 8);
+  }
+  // (the loads keep this order -- queries, K, V: the compiler's count of loads in flight on the
+  // way into the key loop becomes what it waits for inside it)
+  __builtin_amdgcn_sched_barrier(0);
+  request_k();
+  __builtin_amdgcn_sched_barrier(0);
+  request_v();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int ch = 0; ch < NCH; ++ch) {
+    const u32x4_t raw = qop[ch];
 #pragma unroll
     for (int j2 = 0; j2 < 4; ++j2) {
       const int d0 = KCodec<BITS>::slot_d(2 * j2), d1 = KCodec<BITS>::slot_d(2 * j2 + 1);
       const u32 lo = (raw[d0 >> 1] >> (16 * (d0 & 1))) & 0xffffu, hi = (raw[d1 >> 1] >> (16 * (d1 & 1))) << 16;
-      o[j2] = lo | hi;
+      qop[ch][j2] = lo | hi;
     }
-    lds_q[e] = o;
   }
-  __syncthreads();   // Q^T operands written
 
   floatx16_t oacc[NDB];
 #pragma unroll
@@ -1649,20 +1650,25 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
 #pragma unroll
         for (int m = 0; m < 4; ++m) a[m] = pack_bf16_rne((f[2 * m] - zk) * sk, (f[2 * m + 1] - zk) * sk);
       }
-      sacc = mfma_32x32x16<false>(a, lds_q[ch * 64 + lane], sacc);
+      sacc = mfma_32x32x16<false>(a, qop[ch], sacc);
     }
     request_k();
 
     // ---- V of the block -> V^T tile of this wavefront (bf16 values) ----
+    // (z2, s2: byte biases and plain scales of the lane's two keys, or the general form's parameters)
     bool vbytes = false;
+    float2 z2, s2;
     {
-      u32 va4 = 0;
-      const float vz = has_vzp ? vzp : 0.f, vsc_ = vsc;
-      if constexpr (BYTES) vbytes = !__any(!byte_bias4(vz, va4));
-      if (half == 0) {
-        par[col] = vbytes ? u2f(va4) : (vz + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
-        par[32 + col] = vbytes ? vsc_ : vsc_ * VCodec<BITS>::kMul;
+      u32 va0 = 0, va1 = 0;
+      const float vz0 = has_vzp ? vzp[0] : 0.f, vz1 = has_vzp ? vzp[1] : 0.f;
+      if constexpr (BYTES) {
+        const bool ok0 = byte_bias4(vz0, va0), ok1 = byte_bias4(vz1, va1);
+        vbytes = !__any(!(ok0 && ok1));
       }
+      z2.x = vbytes ? u2f(va0) : (vz0 + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+      z2.y = vbytes ? u2f(va1) : (vz1 + VCodec<BITS>::kOff) * (1.f / VCodec<BITS>::kMul);
+      s2.x = vbytes ? vsc[0] : vsc[0] * VCodec<BITS>::kMul;
+      s2.y = vbytes ? vsc[1] : vsc[1] * VCodec<BITS>::kMul;
     }
 #pragma unroll
     for (int i = 0; i < IPL; ++i) {
@@ -1670,7 +1676,6 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
       u32 r0[WPU], r1[WPU];
 #pragma unroll
       for (int w = 0; w < WPU; ++w) { r0[w] = vraw[i][0][w] ^ VCodec<BITS>::kStageXor; r1[w] = vraw[i][1][w] ^ VCodec<BITS>::kStageXor; }
-      const float2 z2 = *reinterpret_cast<const float2 *>(par + 2 * kp), s2 = *reinterpret_cast<const float2 *>(par + 32 + 2 * kp);
       if (BYTES && vbytes) {
         // (z2 holds the two keys' byte biases, s2 their plain scales)
         const u32 e0 = (r0[0] & 0x0f0f0f0fu) + f2u(z2.x), o0 = ((r0[0] >> 4) & 0x0f0f0f0fu) + f2u(z2.x);
@@ -1783,8 +1788,8 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   // Every wavefront hands the other three their quarters of its accumulators through LDS (one
   // barrier on each side), forms the four weights from everyone's (m, l) and sums its quarter.
   const float l_own = l_part + __shfl_xor(l_part, 32, 64);
-  float *const slots = reinterpret_cast<float *>(lds_raw + FewQLds::kQ);   // [target][source - target - 1 mod 4][16 registers][64 lanes]
-  __syncthreads();   // every wavefront is done with the Q^T operands and its V^T tile
+  float *const slots = reinterpret_cast<float *>(lds_raw + FewQLds::kVt);   // [target][source - target - 1 mod 4][16 registers][64 lanes]
+  __syncthreads();   // every wavefront is done with its V^T tile
 #pragma unroll
   for (int t = 0; t < FQ_NW; ++t) {
     if (t == wave) continue;
