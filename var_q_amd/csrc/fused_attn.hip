@@ -1779,6 +1779,17 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
     for (; blk < b_end; blk += FQ_NW) {
       u32 ka4 = 0;
       if (__any(!byte_bias4(has_kzp ? kzp : 0.f, ka4))) break;
+      // Two workgroups share a compute unit and the SIMD's arbiter prefers the older wavefront:
+      // left alone, the older workgroup finishes about a quarter earlier and the younger one
+      // then runs its rest at one wavefront per SIMD.  Priority by the quarter of its own
+      // blocks a wavefront is in lets the one that is behind catch up.
+      {
+        const int q4 = (blk - blk0) * 4 / max(b_end - blk0, 1);
+        if (q4 == 0) __builtin_amdgcn_s_setprio(3);
+        else if (q4 == 1) __builtin_amdgcn_s_setprio(2);
+        else if (q4 == 2) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
       block(blk, std::true_type{}, ka4);
     }
   }
