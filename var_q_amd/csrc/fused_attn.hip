@@ -1533,8 +1533,10 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   // branch around a load the compiler no longer knows how many loads are in flight and waits for
   // all of them where it needs the oldest.
   // Addresses: the (batch, head) bases are uniform; a lane keeps 32-bit byte offsets of its rows
-  // from them, advanced by four blocks per request and clamped at the last key (the host checks
-  // that they fit) -- an add and a min per stream instead of the products of key and strides.
+  // from them, advanced by four blocks per request and clamped at the last key of the wavefront's
+  // own last block (the host checks that they fit) -- an add and a min per stream instead of the
+  // products of key and strides; the one request past the wavefront's blocks re-reads that row
+  // instead of fetching a block of another wavefront's.
   const int64_t kv_row0 = b * p.kv_bs + hs * p.kv_hs;
   const char *const kw_base = reinterpret_cast<const char *>(p.k_words + kv_row0 * WPR);
   const char *const vw_base = reinterpret_cast<const char *>(p.v_words + kv_row0 * WPR);
@@ -1544,9 +1546,12 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   const char *const vz_base = reinterpret_cast<const char *>((p.v_zp ? p.v_zp : p.v_scale) + kv_row0);
   const bool has_kzp = p.k_zp != nullptr, has_vzp = p.v_zp != nullptr;
   const u32 row_b = (u32)p.kv_ts * (WPR * 4), par_b = (u32)p.kv_ts * 4;   // bytes from one key to the next
-  const u32 par_last = (u32)(p.Lk - 1) * par_b;
+  static_assert(FQ_NW == 4, "a wavefront's blocks are four apart");
+  const int last_blk = blk0 + ((max(b_end - 1 - blk0, 0) >> 2) << 2);   // (this wavefront's last block, if it has any)
+  const u32 last_key = (u32)min(last_blk * FQ_BK + FQ_BK - 1, p.Lk - 1);
+  const u32 par_last = last_key * par_b;
   const u32 k_lane = half * (HW * 4), v_lane = (lane >> 4) * (WPU * 4);     // this lane's place inside a row
-  const u32 k_row_last = (u32)(p.Lk - 1) * row_b + k_lane, v_row_last = (u32)(p.Lk - 1) * row_b + v_lane;
+  const u32 k_row_last = last_key * row_b + k_lane, v_row_last = last_key * row_b + v_lane;
   const u32 row_step = FQ_NW * FQ_BK * row_b, par_step = FQ_NW * FQ_BK * par_b;
   // MFMA row `col` carries key kperm(col) of the block; V: item = lane + 64 i covers keys 2 kp, 2 kp + 1
   // (kp = lane & 15: the lanes of a tile row write 16 adjacent banks) and unit (lane >> 4) + 4 i
