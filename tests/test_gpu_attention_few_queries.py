@@ -210,3 +210,33 @@ def test_softmax_range(dev, prof, bits, limit):
     torch.cuda.synchronize()
     _check(out, O.attention_ref(q, kd, vd, scale, bias), O.attention_exact(q.float(), kd, vd, scale, bias),
            f'few queries, softmax range {prof} int{bits}' + (' limit' if limit else ''))
+
+
+def test_workspace_missing_or_short(dev):
+    """The key shares are cut down to what the caller's workspace holds: no workspace at all (one
+    workgroup per (batch, head) walks the whole cache) and one that is too small for the shares
+    the library would like, through the C ABI, against the call with the full workspace."""
+    from var_q_amd._lib import check
+    B, H, Lq, Lk, D, bits, g = 1, 3, 20, 4100, 128, 4, 128
+    gen = torch.Generator(device=dev).manual_seed(606)
+    k = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    v = torch.randn(B, H, Lk, D, device=dev, generator=gen).bfloat16()
+    q = torch.randn(B, H, Lq, D, device=dev, generator=gen).bfloat16()
+    (kw, ks, kz), (vw, vs, vz) = ops.quant_pack_rows(k, g, bits, True), ops.quant_pack_rows(v, g, bits, True)
+    scale = 1 / math.sqrt(D)
+    lib = _lib.load()
+    full = int(lib.varq_fused_attn_workspace_bytes(B, H, Lq, Lk, D, 1, 0))
+    shares = int(lib.varq_fused_attn_key_shares(B, H, Lq, Lk, D, g, g))
+    assert shares > 4 and full > 0
+    want = ops.fused_attn(q, kw, ks, kz, vw, vs, vz, bits, bits, Lk, scale)
+    span = max(1.0, float(want.float().abs().max()))
+    for nbytes in (0, full // 3):
+        note('few queries, workspace of', nbytes, 'bytes where', full, 'are asked for')
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        out = torch.zeros_like(q)
+        check(lib.varq_fused_attn(q.data_ptr(), out.data_ptr(), kw.data_ptr(), ks.data_ptr(), kz.data_ptr(), bits, g,
+                                  vw.data_ptr(), vs.data_ptr(), vz.data_ptr(), bits, g, B, H, H, None, Lq, Lk, Lk, D, None,
+                                  float(scale), 0, 1, 0, ws.data_ptr() if nbytes else None, nbytes, 0,
+                                  torch.cuda.current_stream().cuda_stream), 'varq_fused_attn')
+        torch.cuda.synchronize()
+        assert float((out.float() - want.float()).abs().max()) <= span * 2 ** -6
