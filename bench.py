@@ -498,6 +498,29 @@ def hbm_regime_rates(torch, dev, kv_sets):
                             'kv_read_frac_hbm_peak': round(kv_bytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
                             'TFLOPs': round(flops / dt / 1e12, 1),
                             'key_shares': int(lib.varq_fused_attn_key_shares(B, H, lq, L, D, GROUP, GROUP))}
+    # the same 16 queries over a cache four times as long (synthetic, same format): how the rate
+    # grows once the costs that do not depend on the cache length weigh less
+    L4 = 4 * L
+    long_sets = []
+    for _ in range(4):
+        k4, v4 = (torch.randn(B, H, L4, D, device=dev, generator=gd).bfloat16() for _ in range(2))
+        (kw, ks, kz), (vw, vs, vz) = ops.quant_pack_rows(k4, GROUP, BITS, True), ops.quant_pack_rows(v4, GROUP, BITS, True)
+        long_sets.append((kw, ks, kz, vw, vs, vz))
+        del k4, v4
+    q = torch.randn(B, H, 16, D, device=dev, generator=gd).bfloat16()
+    o = torch.empty_like(q)
+    j = [0]
+
+    def fn4():
+        t = long_sets[j[0] % 4]
+        j[0] += 1
+        ops.fused_attn(q, *t, BITS, BITS, L4, scale, out=o)
+    dt = timed_launches(torch, fn4, reps=40, warm=8)
+    out['Lq16_four_times_the_keys'] = {'keys': L4, 'kv_MB': round(4 * kv_bytes / 1e6, 2), 'us': round(dt * 1e6, 1),
+                                       'kv_read_GBps': round(4 * kv_bytes / dt / 1e9, 1),
+                                       'kv_read_frac_hbm_peak': round(4 * kv_bytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                                       'key_shares': int(lib.varq_fused_attn_key_shares(B, H, 16, L4, D, GROUP, GROUP))}
+    del long_sets
     out['config5_early_scales'] = c5_early_scales(torch, dev)
     return out
 

@@ -63,6 +63,8 @@ def test_classes_on_side_streams_equal_one_stream(dev):
     q = torch.randn(B, H, 300, D, generator=gen).bfloat16().to(dev)
     cache.append(k, v)
     cache.splits = 1     # (on one stream the library would share the keys out; same arithmetic wanted here)
+    assert cache.concurrent_min_flops > 0     # (the default keeps a call of this size on one stream ...)
+    cache.concurrent_min_flops = 0            # (... so the streams are forced here)
     outs = {}
     for mode in (False, True, True):
         cache.concurrent_classes = mode

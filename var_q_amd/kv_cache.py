@@ -38,7 +38,12 @@ class PackedKVCache:
         self.B, self.H, self.Lmax, self.D, self.group = B, H, Lmax, D, group_size
         self.per_head_bits, self.symmetric, self.eps = per_head, symmetric, eps
         self.len = 0
-        self.concurrent_classes = True   # attend(): one stream per bit-width class
+        self.concurrent_classes = True   # attend(): one stream per bit-width class ...
+        # ... once the call is large enough: forking and joining the streams costs the host about
+        # 50 us, more than the classes of a small step gain by running side by side (measured on
+        # the 13-scale schedule at B=8, H=16: side streams win from 576 queries over 1 497 keys
+        # on).  While a graph is being recorded there is no such cost and the streams are always used.
+        self.concurrent_min_flops = 4e10
         self.splits = 0                  # attend() on one stream: shares of a query block's keys (0 = library's choice)
         self._side = self._fork = self._join = None
         self.classes: List[_BitClass] = [
@@ -178,7 +183,9 @@ class PackedKVCache:
         asym = not self.symmetric
         many = len(self.classes) > 1
         main = torch.cuda.current_stream(q.device)
-        side = self._side_streams(q.device) if many and self.concurrent_classes else None
+        worth = (torch.cuda.is_current_stream_capturing()
+                 or 4.0 * q.shape[0] * q.shape[1] * q.shape[2] * self.len * self.D >= self.concurrent_min_flops)
+        side = self._side_streams(q.device) if many and self.concurrent_classes and worth else None
         if side:
             self._fork.record(main)
         for i, c in enumerate(self.classes):
@@ -192,7 +199,8 @@ class PackedKVCache:
                                c.v_words, c.v_scale, c.v_zp if asym else None,
                                c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
                                head_map=c.head_map if many else None, out=out,
-                               splits=1 if side else self.splits, exact_codes=exact_codes)   # classes side by side fill the device already
+                               splits=1 if many and self.concurrent_classes else self.splits,   # classes side by side fill the device already; the
+                               exact_codes=exact_codes)                                         # same rule on one stream, so both ways add up alike
             if stream is not main:
                 self._join[i - 1].record(stream)
                 main.wait_event(self._join[i - 1])
