@@ -521,6 +521,24 @@ def hbm_regime_rates(torch, dev, kv_sets):
                                        'kv_read_frac_hbm_peak': round(4 * kv_bytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
                                        'key_shares': int(lib.varq_fused_attn_key_shares(B, H, 16, L4, D, GROUP, GROUP))}
     del long_sets
+    # and over an INT8 group-128 cache of configuration 4's shape (twice the bytes per key, the same number of codes)
+    sets8 = []
+    for _ in range(4):
+        k8, v8 = (torch.randn(B, H, L, D, device=dev, generator=gd).bfloat16() for _ in range(2))
+        sets8.append((*ops.quant_pack_rows(k8, GROUP, 8, True), *ops.quant_pack_rows(v8, GROUP, 8, True)))
+        del k8, v8
+    kv8 = 2 * (B * H * L * D + B * H * L * (D // GROUP) * 8)
+    j[0] = 0
+
+    def fn8():
+        t = sets8[j[0] % 4]
+        j[0] += 1
+        ops.fused_attn(q, *t, 8, 8, L, scale, out=o)
+    dt = timed_launches(torch, fn8, reps=40, warm=8)
+    out['Lq16_int8_cache'] = {'kv_MB': round(kv8 / 1e6, 2), 'us': round(dt * 1e6, 1), 'kv_read_GBps': round(kv8 / dt / 1e9, 1),
+                              'kv_read_frac_hbm_peak': round(kv8 / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                              'key_shares': int(lib.varq_fused_attn_key_shares(B, H, 16, L, D, GROUP, GROUP))}
+    del sets8
     out['config5_early_scales'] = c5_early_scales(torch, dev)
     return out
 
