@@ -88,6 +88,19 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert lib.varq_fused_attn_workspace_bytes(2, 16, 4096, 10521, 128, 1, 0) == 0
     assert lib.varq_fused_attn_workspace_bytes(2, 16, 400, 921, 128, 8, 0) > 0
     assert lib.varq_fused_attn_workspace_bytes(2, 16, 400, 921, 128, 8, 1) == 0
+    # the kernel for few queries over a long cache (D = 128, one group per key, at most 64 queries,
+    # at least 1024 keys, a (batch, head) slice within 4 GB): its share counts on 256 compute units
+    # (what the library assumes without a device), its workspace, and who is not taken
+    ks = lib.varq_fused_attn_key_shares
+    assert ks(2, 16, 16, 10521, 128, 128, 128) == 16 and ks(2, 16, 64, 10521, 128, 128, 128) == 8
+    assert ks(8, 128, 16, 1024, 128, 128, 128) == 1            # enough (batch, head) pairs already
+    assert ks(1, 1, 16, 100000, 128, 128, 128) == 64           # capped
+    assert ks(1, 2, 16, 1056, 128, 128, 128) == 4              # at least eight 32-key blocks per share
+    assert lib.varq_fused_attn_workspace_bytes(2, 16, 16, 10521, 128, 1, 0) == 16 * (2 * 16 * 16) * (128 + 2) * 4
+    for args in ((2, 16, 65, 10521, 128, 128, 128), (2, 16, 16, 1000, 128, 128, 128), (2, 16, 16, 10521, 64, 64, 64),
+                 (2, 16, 16, 10521, 128, 64, 128), (1, 64, 16, 1 << 20, 128, 128, 128)):
+        shares = ks(*args)
+        assert 1 <= shares <= 8, args                           # the general kernel's sharing, or none
     # per-channel attention: segment table checks
     i32 = lambda v: (ctypes.c_int32 * len(v))(*v)
     chan = lambda nseg, ends, Lk=16, D=128: lib.varq_fused_attn_channel(
