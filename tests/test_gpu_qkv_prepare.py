@@ -132,3 +132,46 @@ def test_zero_points_around_the_rounding_shortcuts_limit(dev, bits):
     cq, cs, cz = O.quant_groupwise(v_ref, c, bits, True)
     assert torch.equal(vs.cpu(), cs) and torch.equal(vz.cpu(), cz)
     assert torch.equal(vw.cpu(), O.pack_last_dim(cq, bits)[0])
+
+
+def test_more_token_tiles_than_one_grid_plane(dev):
+    """One head of 524 328 tokens at c = 128 is 32 771 tiles of 16 tokens, past the 32 768 that lie
+    along one grid dimension: the whole launch equals two launches over its halves (bit for bit,
+    every output), and its last tokens equal the oracle's."""
+    B, L, H, c, bits, group = 1, 32768 * 16 + 40, 1, 128, 4, 128
+    g = torch.Generator(device=dev).manual_seed(77)
+    qkv = torch.randn(B, L, 3, H, c, device=dev, generator=g).bfloat16()
+    mul = torch.tensor([1.75], device=dev)
+
+    def run(x, outs, off):
+        n = x.shape[1]
+        rowmap = [B, n, H, H * L, 1, L, off, -1]
+        q_out = torch.empty(B, H, n, c, dtype=torch.bfloat16, device=dev)
+        ops.qkv_prepare_append(x, q_out, group, bits, True, 1e-12, *outs, rowmap, None, mul, True, 1e-12, None, 0)
+        return q_out
+
+    def buffers():
+        mk = lambda last, dt: torch.full((B, H, L, last), 7, dtype=dt, device=dev)
+        W = c * bits // 32
+        return (mk(W, torch.int32), mk(1, torch.float32), mk(1, torch.float32),
+                mk(W, torch.int32), mk(1, torch.float32), mk(1, torch.float32))
+
+    note('qkv_prepare 32771 tiles, one launch')
+    whole = buffers()
+    q_whole = run(qkv, whole, 0)
+    note('qkv_prepare 32771 tiles, two launches')
+    halves = buffers()
+    Lh = L // 2 + 3
+    q_a = run(qkv[:, :Lh].contiguous(), halves, 0)
+    q_b = run(qkv[:, Lh:].contiguous(), halves, Lh)
+    torch.cuda.synchronize()
+    assert torch.equal(q_whole, torch.cat([q_a, q_b], dim=2))
+    for a, b in zip(whole, halves):
+        assert torch.equal(a, b)
+    tail = 48
+    q_ref, k_ref, v_ref = O.prepare_qkv(qkv[:, -tail:].cpu(), mul.cpu(), True, 1e-12, None, 0)
+    assert torch.equal(q_whole[:, :, -tail:].cpu().view(torch.int16), q_ref.view(torch.int16))
+    for x, (w, s, z) in ((k_ref, whole[:3]), (v_ref, whole[3:])):
+        cq, cs, cz = O.quant_groupwise(x, group, bits, True)
+        assert torch.equal(s[:, :, -tail:].cpu(), cs) and torch.equal(z[:, :, -tail:].cpu(), cz)
+        assert torch.equal(w[:, :, -tail:].cpu(), O.pack_last_dim(cq, bits)[0])

@@ -39,6 +39,9 @@ struct PrepParams {
   int64_t rows;                // B*L*H
 };
 
+// the token tiles of a launch lie along grid y, and along z beyond this many
+constexpr int kTilesPerPlane = 32768;
+
 template <int LANES> __device__ __forceinline__ float group_allsum(float v) {
   // after each step the partners hold the same value, so the mirrored steps pair equal halves
   if (LANES >= 2) v = v + dpp_f<0xB1>(v);
@@ -153,12 +156,15 @@ __device__ __forceinline__ float pair_swap(float v) { return dpp_f<0xB1>(v); }
 // One lane = 8 channels of one (b, l, h); LR = c/8 lanes form the row, LG = group/8 a group.
 template <int DT, int BITS, bool ASYM, int LR, int LG>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
-  // grid = (tiles of 256/LR tokens, B*H): lanes walk the (b, h, l) order of the outputs, so the
+  // grid = (B*H, tiles of 256/LR tokens): lanes walk the (b, h, l) order of the outputs, so the
   // prepared q, the packed words and the scales of a wavefront are contiguous; the reads are
   // whole 16*LR-byte rows either way.  (b, h) is uniform for the workgroup: no vector divisions.
-  const int bh = blockIdx.y;
+  // The head is the fastest grid dimension: the workgroups that are in flight together then read
+  // all heads of the same tokens, whole 6*H*c-byte stretches of the input between them, instead
+  // of one 2*c-byte piece out of every token row (8 % of the kernel's time at H=16, c=128).
+  const int bh = blockIdx.x;
   const int h = bh % p.H, b = bh / p.H;
-  const int o = blockIdx.x * 256 + threadIdx.x;
+  const int o = (blockIdx.z * kTilesPerPlane + blockIdx.y) * 256 + threadIdx.x;
   const int lt = o / LR;                              // (LR is a power of two)
   const int col = o - lt * LR;
   const bool live = lt < p.L;
@@ -172,6 +178,13 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
   const bool odd = col & 1;
 
   float q[8], k[8], v[8];
+  // the rotation's factors are requested with the row, long before the rotation needs them;
+  // without a table the requests read the first 16 bytes of the input and nothing uses them
+  const float *cos_base = p.cos ? p.cos : reinterpret_cast<const float *>(p.qkv);
+  const float *sin_base = p.cos ? p.sin : reinterpret_cast<const float *>(p.qkv);
+  const int t = p.cos ? (p.token_start + l) * (c / 2) + col * 4 : 0;   // (fits 32 bits: checked on the host)
+  const float4 cs = *reinterpret_cast<const float4 *>(cos_base + t);
+  const float4 sn = *reinterpret_cast<const float4 *>(sin_base + t);
   In8<DT>::load(p.qkv, base_bh + lane_off, q);
   In8<DT>::load(p.qkv, base_bh + lane_off + tstride, k);
   In8<DT>::load(p.qkv, base_bh + lane_off + 2 * tstride, v);
@@ -205,9 +218,6 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
     }
   }
   if (p.cos) {
-    const int t = (p.token_start + l) * (c / 2) + col * 4;     // (fits 32 bits: checked on the host)
-    const float4 cs = *reinterpret_cast<const float4 *>(p.cos + t);
-    const float4 sn = *reinterpret_cast<const float4 *>(p.sin + t);
     const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -364,8 +374,10 @@ extern "C" int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int 
   p.norm_eps = norm_eps; p.eps = eps; p.rows = rows;
   p.slow_levels = !(eps >= 0x1p-80f);
   const int64_t tiles = ((int64_t)L * p.c8 + 255) / 256;
-  VARQ_CHECK_ARG(tiles < (1ll << 31) && (int64_t)B * H <= 65535, "qkv_prepare: B*H must not exceed 65535");
-  dim3 grid((unsigned)tiles, (unsigned)(B * H));
+  const int64_t planes = (tiles + kTilesPerPlane - 1) / kTilesPerPlane;
+  VARQ_CHECK_ARG(planes <= 65535 && (int64_t)B * H < (1ll << 31), "qkv_prepare: tensor too large");
+  // (tiles past the last token in the last plane find no live lane and store nothing)
+  dim3 grid((unsigned)(B * H), (unsigned)(tiles < kTilesPerPlane ? tiles : kTilesPerPlane), (unsigned)planes);
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (x_dtype == VARQ_F32) rc = launch_dt<VARQ_F32>(p, bits, asym, p.c8, group / 8, grid, st);
