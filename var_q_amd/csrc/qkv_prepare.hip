@@ -44,10 +44,7 @@ constexpr int kTilesPerPlane = 32768;
 
 template <int LANES> __device__ __forceinline__ float group_allsum(float v) {
   // after each step the partners hold the same value, so the mirrored steps pair equal halves
-  if (LANES >= 2) v = v + dpp_f<0xB1>(v);
-  if (LANES >= 4) v = v + dpp_f<0x4E>(v);
-  if (LANES >= 8) v = v + dpp_f<0x141>(v);
-  if (LANES >= 16) v = v + dpp_f<0x140>(v);
+  v = row_fold_add<(LANES < 16 ? LANES : 16)>(v);
   if (LANES >= 32) v = v + __shfl_xor(v, 16, 64);
   return v;
 }

@@ -157,14 +157,40 @@ __device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
 // Cross-lane all-reduce over aligned groups of LANES lanes (power of two).
 // Stages inside a 16-lane row use DPP, wider stages a lane permute.
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
-  return u2f((u32)__builtin_amdgcn_update_dpp((int)f2u(v), (int)f2u(v), CTRL, 0xf, 0xf, false));
+  // (every lane of these controls has a source lane, so no old value is needed)
+  return u2f((u32)__builtin_amdgcn_mov_dpp((int)f2u(v), CTRL, 0xf, 0xf, false));
 }
+
+// A fold over aligned groups of up to 16 lanes as one DPP instruction per step, v = OP(v of
+// the partner lane, v).  Written as assembly because the compiler's sequence for the same
+// step through the intrinsic is four instructions (a copy, a DPP move, a canonicalising max
+// of the moved value with itself, the operation).  A DPP read needs two idle cycles after a
+// vector write of its source: the s_nop in front of every step provides them whatever wrote
+// the source, the one at the end covers a DPP read of the result by whatever follows.
+// v_max_f32 / v_min_f32 return the other operand when one is a quiet NaN, like fmaxf / fminf.
+#define VARQ_DPP_FOLD_STEP(op, ctrl) "s_nop 1\n\t" op "_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
+#define VARQ_DPP_FOLD(NAME, OP)                                                                     \
+  template <int LANES> __device__ __forceinline__ float NAME(float v) {                             \
+    static_assert(LANES == 1 || LANES == 2 || LANES == 4 || LANES == 8 || LANES == 16, "one row");  \
+    if (LANES == 2) asm(VARQ_DPP_FOLD_STEP(OP, "quad_perm:[1,0,3,2]") "s_nop 1" : "+v"(v));         \
+    if (LANES == 4)                                                                                 \
+      asm(VARQ_DPP_FOLD_STEP(OP, "quad_perm:[1,0,3,2]") VARQ_DPP_FOLD_STEP(OP, "quad_perm:[2,3,0,1]") "s_nop 1" : "+v"(v)); \
+    if (LANES == 8)                                                                                 \
+      asm(VARQ_DPP_FOLD_STEP(OP, "quad_perm:[1,0,3,2]") VARQ_DPP_FOLD_STEP(OP, "quad_perm:[2,3,0,1]")  \
+          VARQ_DPP_FOLD_STEP(OP, "row_half_mirror") "s_nop 1" : "+v"(v));                           \
+    if (LANES == 16)                                                                                \
+      asm(VARQ_DPP_FOLD_STEP(OP, "quad_perm:[1,0,3,2]") VARQ_DPP_FOLD_STEP(OP, "quad_perm:[2,3,0,1]")  \
+          VARQ_DPP_FOLD_STEP(OP, "row_half_mirror") VARQ_DPP_FOLD_STEP(OP, "row_mirror") "s_nop 1" : "+v"(v)); \
+    return v;                                                                                       \
+  }
+VARQ_DPP_FOLD(row_fold_max, "v_max_f32")
+VARQ_DPP_FOLD(row_fold_min, "v_min_f32")
+VARQ_DPP_FOLD(row_fold_add, "v_add_f32")
+#undef VARQ_DPP_FOLD
+
 template <int LANES, bool IS_MAX> __device__ __forceinline__ float group_allreduce(float v) {
 #define VARQ_COMBINE(a, b) (IS_MAX ? fmaxf((a), (b)) : fminf((a), (b)))
-  if (LANES >= 2) v = VARQ_COMBINE(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
-  if (LANES >= 4) v = VARQ_COMBINE(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
-  if (LANES >= 8) v = VARQ_COMBINE(v, dpp_f<0x141>(v));  // row_half_mirror
-  if (LANES >= 16) v = VARQ_COMBINE(v, dpp_f<0x140>(v)); // row_mirror
+  v = IS_MAX ? row_fold_max<(LANES < 16 ? LANES : 16)>(v) : row_fold_min<(LANES < 16 ? LANES : 16)>(v);
   if (LANES >= 32) v = VARQ_COMBINE(v, __shfl_xor(v, 16, 64));
   if (LANES >= 64) v = VARQ_COMBINE(v, __shfl_xor(v, 32, 64));
 #undef VARQ_COMBINE
