@@ -134,10 +134,10 @@ def test_zero_points_around_the_rounding_shortcuts_limit(dev, bits):
     assert torch.equal(vw.cpu(), O.pack_last_dim(cq, bits)[0])
 
 
-def test_more_token_tiles_than_one_grid_plane(dev):
-    """One head of 524 328 tokens at c = 128 is 32 771 tiles of 16 tokens, past the 32 768 that lie
-    along one grid dimension: the whole launch equals two launches over its halves (bit for bit,
-    every output), and its last tokens equal the oracle's."""
+def test_half_a_million_tokens_of_one_head(dev):
+    """One head of 524 328 tokens at c = 128 (32 771 tiles of 16 tokens, not a multiple of the eight
+    that the workgroup order deals out together): the whole launch equals two launches over its
+    halves (bit for bit, every output), and its last tokens equal the oracle's."""
     B, L, H, c, bits, group = 1, 32768 * 16 + 40, 1, 128, 4, 128
     g = torch.Generator(device=dev).manual_seed(77)
     qkv = torch.randn(B, L, 3, H, c, device=dev, generator=g).bfloat16()
@@ -156,10 +156,10 @@ def test_more_token_tiles_than_one_grid_plane(dev):
         return (mk(W, torch.int32), mk(1, torch.float32), mk(1, torch.float32),
                 mk(W, torch.int32), mk(1, torch.float32), mk(1, torch.float32))
 
-    note('qkv_prepare 32771 tiles, one launch')
+    note('qkv_prepare 524328 tokens, one launch')
     whole = buffers()
     q_whole = run(qkv, whole, 0)
-    note('qkv_prepare 32771 tiles, two launches')
+    note('qkv_prepare 524328 tokens, two launches')
     halves = buffers()
     Lh = L // 2 + 3
     q_a = run(qkv[:, :Lh].contiguous(), halves, 0)

@@ -39,9 +39,6 @@ struct PrepParams {
   int64_t rows;                // B*L*H
 };
 
-// the token tiles of a launch lie along grid y, and along z beyond this many
-constexpr int kTilesPerPlane = 32768;
-
 template <int LANES> __device__ __forceinline__ float group_allsum(float v) {
   // after each step the partners hold the same value, so the mirrored steps pair equal halves
   v = row_fold_add<(LANES < 16 ? LANES : 16)>(v);
@@ -153,15 +150,20 @@ __device__ __forceinline__ float pair_swap(float v) { return dpp_f<0xB1>(v); }
 // One lane = 8 channels of one (b, l, h); LR = c/8 lanes form the row, LG = group/8 a group.
 template <int DT, int BITS, bool ASYM, int LR, int LG>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
-  // grid = (B*H, tiles of 256/LR tokens): lanes walk the (b, h, l) order of the outputs, so the
-  // prepared q, the packed words and the scales of a wavefront are contiguous; the reads are
-  // whole 16*LR-byte rows either way.  (b, h) is uniform for the workgroup: no vector divisions.
-  // The head is the fastest grid dimension: the workgroups that are in flight together then read
-  // all heads of the same tokens, whole 6*H*c-byte stretches of the input between them, instead
-  // of one 2*c-byte piece out of every token row (8 % of the kernel's time at H=16, c=128).
-  const int bh = blockIdx.x;
+  // One workgroup = one tile of 256/LR tokens of one (b, h): lanes walk the (b, h, l) order of the
+  // outputs, so the prepared q, the packed words and the scales of a wavefront are contiguous; the
+  // reads are whole 16*LR-byte rows either way.  (b, h) is uniform for the workgroup: no vector
+  // divisions.  Order of the workgroups (1-D grid; consecutive ids go to consecutive XCDs):
+  // id = ((tile / 8) * B*H + bh) * 8 + tile % 8.  The workgroups in flight together then read all
+  // heads of the same few tokens, whole 6*H*c-byte stretches of the input between them, instead
+  // of one 2*c-byte piece out of every token row (8 % of the kernel's time at H=16, c=128), and
+  // the B*H workgroups of one tile run on one XCD, whose L2 fetches that tile's rotary factors once.
+  const u32 id = blockIdx.x, j = id >> 3;
+  const u32 BH = (u32)(p.B * p.H);
+  const u32 tile8 = j / BH;                           // (uniform: scalar arithmetic)
+  const int bh = (int)(j - tile8 * BH);
   const int h = bh % p.H, b = bh / p.H;
-  const int o = (blockIdx.z * kTilesPerPlane + blockIdx.y) * 256 + threadIdx.x;
+  const int o = (int)(tile8 * 8u + (id & 7u)) * 256 + threadIdx.x;
   const int lt = o / LR;                              // (LR is a power of two)
   const int col = o - lt * LR;
   const bool live = lt < p.L;
@@ -371,10 +373,10 @@ extern "C" int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int 
   p.norm_eps = norm_eps; p.eps = eps; p.rows = rows;
   p.slow_levels = !(eps >= 0x1p-80f);
   const int64_t tiles = ((int64_t)L * p.c8 + 255) / 256;
-  const int64_t planes = (tiles + kTilesPerPlane - 1) / kTilesPerPlane;
-  VARQ_CHECK_ARG(planes <= 65535 && (int64_t)B * H < (1ll << 31), "qkv_prepare: tensor too large");
-  // (tiles past the last token in the last plane find no live lane and store nothing)
-  dim3 grid((unsigned)(B * H), (unsigned)(tiles < kTilesPerPlane ? tiles : kTilesPerPlane), (unsigned)planes);
+  // (tiles are dealt out in eights; those past the last token find no live lane and store nothing)
+  const int64_t wgs = (tiles + 7) / 8 * 8 * ((int64_t)B * H);
+  VARQ_CHECK_ARG(wgs < (1ll << 31), "qkv_prepare: tensor too large");
+  dim3 grid((unsigned)wgs);
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (x_dtype == VARQ_F32) rc = launch_dt<VARQ_F32>(p, bits, asym, p.c8, group / 8, grid, st);
