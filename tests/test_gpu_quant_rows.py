@@ -209,3 +209,47 @@ def _offset_rows(c):
 def test_zero_points_around_the_rounding_shortcuts_limit(dev, bits, c, group):
     note('quant_rows zero-point limit', bits, c, group)
     _check(_offset_rows(c), group, bits, True, dev)
+
+
+@pytest.mark.parametrize('bits,group,asym,dtype', [(4, 128, True, torch.bfloat16), (8, 64, False, torch.float32),
+                                                    (2, 32, True, torch.float16), (4, 16, True, torch.bfloat16),
+                                                    (8, 8, True, torch.bfloat16)])
+@pytest.mark.parametrize('n', [1, 3, 5, 37, 300])
+def test_token_major_input_into_a_head_major_cache(dev, bits, group, asym, dtype, n):
+    """K and V as the Infinity block holds them, [B, L, H, c], written into a [B, heads, Lmax]
+    cache through a row map over (B, L, H) with a slot table over the heads
+    (VAR_Q/quant.py:196-201 behind the transpose of Infinity/infinity/models/basic.py:330).
+    With at least as many tokens as heads the kernel walks the tokens of one head, otherwise the
+    heads of one token; either way the cache must hold what the head-major order of the same
+    values gives, which in turn equals the oracle."""
+    B, H, D, Lmax, start = 2, 5, 128, 320, 11
+    heads = [3, 0, 4]
+    g = torch.Generator().manual_seed(bits * 7 + group + n)
+    k = (torch.randn(B, n, H, D, generator=g) * 3).to(dtype)
+    v = (torch.randn(B, n, H, D, generator=g) * 3).to(dtype)
+    slot = torch.full((H,), -1, dtype=torch.int32)
+    for i, h in enumerate(heads):
+        slot[h] = i
+    slot = slot.to(dev)
+    hc, W, ng = len(heads), D * bits // 32, D // group
+    map_blhc = [B, n, H, hc * Lmax, 1, Lmax, start, 2]
+    map_bhlc = [B, H, n, hc * Lmax, Lmax, 1, start, 1]
+
+    def bufs():
+        return (torch.full((B, hc, Lmax, W), 7, dtype=torch.int32, device=dev),
+                torch.full((B, hc, Lmax, ng), 7.0, device=dev), torch.full((B, hc, Lmax, ng), 7.0, device=dev) if asym else None)
+    a_k, a_v, b_k, b_v, c_k = bufs(), bufs(), bufs(), bufs(), bufs()
+    note('quant_pack_rows token-major', bits, group, asym, dtype, n)
+    ops.quant_pack_rows_pair_into(k.to(dev), v.to(dev), group, bits, asym, 1e-12, a_k, a_v, map_blhc, slot)
+    ops.quant_pack_rows_into(k.to(dev), group, bits, asym, 1e-12, *c_k, map_blhc, slot)
+    kt, vt = k.transpose(1, 2).contiguous(), v.transpose(1, 2).contiguous()
+    ops.quant_pack_rows_pair_into(kt.to(dev), vt.to(dev), group, bits, asym, 1e-12, b_k, b_v, map_bhlc, slot)
+    torch.cuda.synchronize()
+    for x, y in zip(a_k + a_v + a_k, b_k + b_v + c_k):
+        if x is not None:
+            assert torch.equal(x, y)
+    q, s, z = O.quant_groupwise(kt[:, heads], group, bits, asym)
+    sl = slice(start, start + n)
+    assert torch.equal(a_k[0][:, :, sl].cpu(), O.pack_last_dim(q, bits)[0])
+    assert torch.equal(a_k[1][:, :, sl].cpu(), s) and (not asym or torch.equal(a_k[2][:, :, sl].cpu(), z))
+    assert bool((a_k[0][:, :, :start] == 7).all()) and bool((a_k[0][:, :, start + n:] == 7).all())

@@ -12,6 +12,17 @@
 // the min/max reduction is a DPP butterfly inside the wavefront and never
 // touches LDS.  A block covers octets of one (i0,i1) pair of the row map so
 // that the output row offset is block-uniform.
+//
+// Which of the map's inner two dims is the block-uniform one is the launcher's
+// choice: the rows a block walks should be the ones that lie next to each other
+// in the OUTPUT.  For K and V in [B, L, H, c] order going into a [B, H, Lmax]
+// cache (VAR_Q/quant.py:196-201 after the transpose of
+// Infinity/infinity/models/basic.py:330) a block therefore takes tokens l.. of
+// one head - 2c-byte pieces H*2c bytes apart on the input side, whole
+// contiguous stretches of packed words, scales and zero-points on the output
+// side - instead of the H heads of one token, whose packed rows lie Lmax rows
+// apart (64-byte stores all over the cache, a quarter of the lanes at work for
+// H = 16: 0.34 of HBM peak where the other order reaches 0.72).
 #include <type_traits>
 #include "varq_common.h"
 
@@ -29,7 +40,12 @@ struct RowsParams {
   float *scale1;
   float *zp1;
   const int32_t *slot;
-  RowMap map;
+  RowMap map;                // as the kernel walks it: n1 is uniform per workgroup, n2 the rows inside
+  // element offset of row (i0, i1, i2) of the input: i0 * in_s0 + i1 * in_s1 + i2 * in_s2.  For an
+  // input in the order of the map, in_s2 = c; when the launcher has swapped the roles of the map's
+  // inner two dims (below), the rows of a workgroup lie in_s2 > c elements apart.
+  int64_t in_s0, in_s1, in_s2;
+  bool strided;              // in_s2 != c
   int64_t octets_per_pair;   // n2 * c8
   int64_t blocks_per_pair;
   int c8;                    // octets per row
@@ -88,7 +104,6 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   float *pscale = second ? p.scale1 : p.scale;
   float *pzp = second ? p.zp1 : p.zp;
   const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
-  const int64_t pair = i0 * p.map.n1 + i1;
   const int tile = blockIdx.x;
 
   int64_t s0 = i0, s1 = i1;
@@ -100,7 +115,9 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   const int o = tile * 256 + (int)threadIdx.x;      // octet index inside the pair
   const bool live = o < (int)p.octets_per_pair;
   const int oc = live ? o : 0;                        // clamp: dead lanes still join the DPP
-  const int64_t in_elem = (pair * p.octets_per_pair + oc) * 8;
+  int64_t in_elem = i0 * p.in_s0 + i1 * p.in_s1;
+  if (p.strided) in_elem += (oc >> p.c8_shift) * (int)p.in_s2 + (oc & (p.c8 - 1)) * 8;   // (c8 is a power of two, the extent fits 31 bits)
+  else in_elem += (int64_t)oc * 8;
 
   float v[8];
   In8<DT>::load(px, in_elem, v);
@@ -185,13 +202,12 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   float *pscale = second ? p.scale1 : p.scale;
   float *pzp = second ? p.zp1 : p.zp;
   const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
-  const int64_t pair = i0 * p.map.n1 + i1;
   int64_t s0 = i0, s1 = i1;
   if (p.map.slot_dim == 0) s0 = p.slot[i0];
   if (p.map.slot_dim == 1) s1 = p.slot[i1];
   if (s0 < 0 || s1 < 0) return;
   const int64_t out_base = s0 * p.map.os0 + s1 * p.map.os1 + p.map.off;
-  const int64_t pair_elem0 = pair * p.octets_per_pair * 8;
+  const int64_t pair_elem0 = i0 * p.in_s0 + i1 * p.in_s1;
 
   const int n_oct = (int)p.octets_per_pair;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -199,13 +215,28 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   constexpr float kMin = (float)QRange<BITS>::kMin, kMax = (float)QRange<BITS>::kMax;
   const int w0 = blockIdx.x * 1024 + wv * 256;       // first octet of this wave's window, inside the pair
 
-  // 1 KiB contiguous per load instruction
+  // 1 KiB per load instruction: contiguous, or whole rows in_s2 elements apart.  Only the
+  // offsets are formed under the (launch-uniform) branch; the four loads follow it together.
+  int64_t e[4];
+  if (!p.strided) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int o = w0 + k * 64 + lane;
+      e[k] = (int64_t)(o < n_oct ? o : 0) * 8;          // past the end: re-read octet 0, never stored
+    }
+  } else {
+    const int s2 = (int)p.in_s2;                        // (the pair's extent fits 31 bits: checked on the host)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      int o = w0 + k * 64 + lane;
+      o = o < n_oct ? o : 0;
+      e[k] = (o >> p.c8_shift) * s2 + (o & (p.c8 - 1)) * 8;
+    }
+  }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    int o = w0 + k * 64 + lane;
-    o = o < n_oct ? o : 0;                            // past the end: re-read octet 0, never stored
     Raw8<DT> r;
-    r.load(px, pair_elem0 + (int64_t)o * 8);
+    r.load(px, pair_elem0 + e[k]);
     stage[k * 64 + lane] = r;
   }
   __builtin_amdgcn_wave_barrier();
@@ -443,10 +474,23 @@ static int quant_pack_rows_launch(const char *who, const void *x, const void *x1
   if (n_rows == 0) return VARQ_OK;
 
   RowsParams p;
-  p.x = x; p.words = words; p.scale = scale; p.zp = zp; p.slot = slot; p.map = m;
+  p.x = x; p.words = words; p.scale = scale; p.zp = zp; p.slot = slot;
   p.x1 = x1; p.words1 = words1; p.scale1 = scale1; p.zp1 = zp1;
   p.c8 = c / 8;
   p.c8_shift = varq_log2_exact(p.c8);
+  p.in_s0 = m.n1 * m.n2 * c; p.in_s1 = m.n2 * c; p.in_s2 = c;
+  // The rows a workgroup walks should be neighbours in the output: if those are the rows along
+  // the map's middle dim (and there are at least as many of them as along the inner one), the
+  // two dims change roles and the workgroup reads its rows n2 * c elements apart.
+  if (m.os1 == 1 && m.os2 != 1 && m.slot_dim != 1 && p.c8_shift >= 0 && m.n1 >= m.n2 && m.n1 * m.n2 * c < (1ll << 31)) {
+    RowMap t = m;
+    t.n1 = m.n2; t.n2 = m.n1; t.os1 = m.os2; t.os2 = m.os1;
+    t.slot_dim = m.slot_dim == 2 ? 1 : m.slot_dim;
+    p.in_s1 = c; p.in_s2 = m.n2 * c;
+    m = t;
+  }
+  p.strided = p.in_s2 != c;
+  p.map = m;
   p.nseg = c / group;
   p.eps = eps;
   p.octets_per_pair = m.n2 * p.c8;
