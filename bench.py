@@ -357,7 +357,7 @@ def prepare_rates(torch, dev):
             'tokens_per_s': round(Bp * Lp / dt, 1), 'algorithmic_MB': round(nbytes / 1e6, 2)}
 
 
-def pack_unpack_rates(torch, dev):
+def pack_unpack_rates(torch, dev, token_major=True):
     """The pack and unpack kernels on their own (the reference's pack_last_dim_to_int32 /
     unpack_last_dim_from_int32 on int8 codes): configuration-4 shape [2,16,10521,128], INT4, INT2
     and INT8, 40 back-to-back launches through the C ABI between one event pair; four sets of
@@ -397,7 +397,43 @@ def pack_unpack_rates(torch, dev):
                                'unpack_us': round(t_u * 1e6, 1), 'unpack_GBps': round(nbytes / t_u / 1e9, 1),
                                'unpack_frac_hbm_peak': round(nbytes / t_u / 1e9 / HBM_PEAK_GBPS, 4), 'algorithmic_MB': round(nbytes / 1e6, 2)}
         del codes, words, back
+    if token_major:
+        out['quantize_token_major_input'] = token_major_quantize_rate(torch, dev)
     return out
+
+
+def token_major_quantize_rate(torch, dev):
+    """The quantize+pack kernel on K and V in the order the Infinity block holds them,
+    [B, L, H, c] = [2, 10521, 16, 128] (bf16), written into the head-major cache [B, H, L, ...]
+    through a row map over (B, L, H): INT4 group 128 asymmetric, K and V in one launch, four
+    input sets cycled.  Bytes: both inputs once, packed words, scales and zero-points once."""
+    from var_q_amd import ops
+    gd = torch.Generator(device=dev).manual_seed(8008)
+    W = D * BITS // 32
+    xs = [(torch.randn(B, L, H, D, device=dev, generator=gd).bfloat16(), torch.randn(B, L, H, D, device=dev, generator=gd).bfloat16())
+          for _ in range(4)]
+    mk = lambda last, dt: torch.empty((B, H, L, last), dtype=dt, device=dev)
+    outs = [[(mk(W, torch.int32), mk(D // GROUP, torch.float32), mk(D // GROUP, torch.float32)) for _ in range(2)] for _ in range(4)]
+    rowmap = [B, L, H, H * L, 1, L, 0, -1]
+    i = [0]
+
+    def fn():
+        i[0] += 1
+        k, v = xs[i[0] % 4]
+        o = outs[i[0] % 4]
+        ops.quant_pack_rows_pair_into(k, v, GROUP, BITS, True, 1e-12, o[0], o[1], rowmap, None)
+    dt = timed_launches(torch, fn, reps=40, warm=8)
+    # the same values in head-major order must give the same cache
+    k, v = xs[1]
+    ref = ops.quant_pack_rows(k.transpose(1, 2).contiguous(), GROUP, BITS, True)
+    i[0] = 0
+    fn()
+    torch.cuda.synchronize()
+    same = all(torch.equal(a, b) for a, b in zip(ref, outs[1][0]))
+    nbytes = 2 * (B * H * L * D * 2 + B * H * L * (W * 4 + 2 * (D // GROUP) * 4))
+    return {'workload': 'K and V [2,10521,16,128] bf16 (token-major) -> INT4 g128 in the head-major cache, one launch',
+            'us': round(dt * 1e6, 1), 'GBps': round(nbytes / dt / 1e9, 1), 'frac_hbm_peak': round(nbytes / dt / 1e9 / HBM_PEAK_GBPS, 4),
+            'algorithmic_MB': round(nbytes / 1e6, 2), 'equals_head_major_input': bool(same)}
 
 
 def shipped_rule_latency(torch, dev, passes=5, warm=2):
@@ -603,6 +639,8 @@ def main():
     ap.add_argument('--no-prepare', action='store_true', help='skip the producer-side (qkv_prepare) leg (profiling runs)')
     ap.add_argument('--no-hbm', action='store_true', help='skip the few-queries-over-a-long-cache leg (profiling runs)')
     ap.add_argument('--no-pack', action='store_true', help='skip the standalone pack / unpack leg (profiling runs)')
+    ap.add_argument('--no-token-major', action='store_true',
+                    help='skip the token-major quantize leg (profiling runs: its launches are the headline pack kernel on the same grid)')
     ap.add_argument('--calib', action='store_true',
                     help='also launch a plain 256 MiB device copy 4 times: known traffic to scale the rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE counters by')
@@ -833,7 +871,7 @@ def main():
         'config5_latency': None if args.no_c5 else c5_latency(torch, dev, check=not args.no_cpu),
         'config3_rates': None if args.no_c3 else c3_rates(torch, dev),
         'qkv_prepare_rates': None if args.no_prepare else prepare_rates(torch, dev),
-        'pack_unpack_rates': None if args.no_pack else pack_unpack_rates(torch, dev),
+        'pack_unpack_rates': None if args.no_pack else pack_unpack_rates(torch, dev, not args.no_token_major),
         'shipped_rule_latency': None if args.no_rule else shipped_rule_latency(torch, dev),
     }
     print(json.dumps(line), flush=True)

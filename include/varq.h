@@ -72,6 +72,9 @@ const char *varq_last_error(void);
  * offset L0 of a [B,H',Lmax,...] cache, optionally only the heads of one
  * bit-width class.  It replaces the torch.cat growth of VAR_Q/quant.py:200-201.
  * Passed as 8 host int64: {n0,n1,n2,os0,os1,os2,off,slot_dim(-1 = none)}.
+ * A token-major step [B,n,H,c] goes into the same cache with the map
+ * {B,n,H, H'*Lmax,1,Lmax, L0, 2}: the quantizer walks whichever of the inner two
+ * dims has output stride 1, so both orders store whole contiguous stretches.
  */
 
 /*
