@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define VARQ_ABI_VERSION 7
+#define VARQ_ABI_VERSION 8
 
 enum varq_status {
   VARQ_OK = 0,
@@ -299,6 +299,9 @@ int varq_fused_attn_channel(const void *q, void *out,
  *   - quantizes k (normalised, rotated) and v group-wise (as varq_quant_pack_rows) into
  *     their cache rows: input row (b, l, h) goes to the row the map gives for
  *     (n0, n1, n2) = (B, L, H).
+ * With a slot table over the heads (slot_dim = 2: one call per bit-width class of a
+ * mixed cache) a head whose slot is negative is left out altogether, its q included:
+ * the calls of the classes share out the heads and between them write all of q.
  * c in {32, 64, 128}; group a power of two in [8, c] (>= 16 for 2-bit codes).
  */
 int varq_qkv_prepare_append(const void *qkv, int x_dtype, int B, int L, int H, int c,

@@ -25,7 +25,7 @@ def test_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f'{n} is declared in varq.h but not exported'
     assert sorted(_lib.SYMBOLS) == names, 'ctypes table and header disagree'
-    assert lib.varq_abi_version() == _lib.ABI_VERSION == 7
+    assert lib.varq_abi_version() == _lib.ABI_VERSION == 8
 
 
 def test_invalid_arguments_are_rejected_on_the_host():

@@ -175,3 +175,35 @@ def test_half_a_million_tokens_of_one_head(dev):
         cq, cs, cz = O.quant_groupwise(x, group, bits, True)
         assert torch.equal(s[:, :, -tail:].cpu(), cs) and torch.equal(z[:, :, -tail:].cpu(), cz)
         assert torch.equal(w[:, :, -tail:].cpu(), O.pack_last_dim(cq, bits)[0])
+
+
+def test_slot_table_over_heads_leaves_other_heads_alone(dev):
+    """One call per bit-width class of a mixed cache: the heads of the class get q, k and v, the
+    others nothing (their q included), so that the calls of all classes write every head once."""
+    B, L, H, c, bits, group, Lmax = 2, 21, 5, 128, 4, 64, 32
+    heads = [3, 0, 4]
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, L, 3, H, c, generator=g).bfloat16()
+    rope = hooks.rope2d_tables(c, [(3, 3), (4, 4)])
+    q_ref, k_ref, v_ref = O.prepare_qkv(qkv, None, True, 1e-12, rope, 0)
+    slot = torch.full((H,), -1, dtype=torch.int32)
+    for i, h in enumerate(heads):
+        slot[h] = i
+    hc, W, ns = len(heads), c * bits // 32, c // group
+    mk = lambda last, dt: torch.full((B, hc, Lmax, last), 7, dtype=dt, device=dev)
+    kw, vw = mk(W, torch.int32), mk(W, torch.int32)
+    ks, kz, vs, vz = (mk(ns, torch.float32) for _ in range(4))
+    q_out = torch.full((B, H, L, c), 7.0, dtype=torch.bfloat16, device=dev)
+    note('qkv_prepare slot table over heads')
+    ops.qkv_prepare_append(qkv.to(dev), q_out, group, bits, True, 1e-12, kw, ks, kz, vw, vs, vz,
+                           [B, L, H, hc * Lmax, 1, Lmax, 3, 2], slot.to(dev), None, True, 1e-12,
+                           (rope[0].to(dev), rope[1].to(dev)), 0)
+    torch.cuda.synchronize()
+    others = [h for h in range(H) if h not in heads]
+    assert bool((q_out[:, others] == 7.0).all()), 'q of a head outside the class was written'
+    assert torch.equal(q_out[:, heads].cpu().view(torch.int16), q_ref[:, heads].view(torch.int16))
+    for x, w, s, z in ((k_ref, kw, ks, kz), (v_ref, vw, vs, vz)):
+        cq, cs, cz = O.quant_groupwise(x[:, heads], group, bits, True)
+        assert torch.equal(w[:, :, 3:3 + L].cpu(), O.pack_last_dim(cq, bits)[0])
+        assert torch.equal(s[:, :, 3:3 + L].cpu(), cs) and torch.equal(z[:, :, 3:3 + L].cpu(), cz)
+        assert bool((w[:, :, :3] == 7).all()) and bool((w[:, :, 3 + L:] == 7).all())

@@ -7,7 +7,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, 'libvarq_hip.so')
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 SYMBOLS = {
     'varq_abi_version': (c_int, []),

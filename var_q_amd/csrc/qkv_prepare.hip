@@ -163,6 +163,13 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
   const u32 tile8 = j / BH;                           // (uniform: scalar arithmetic)
   const int bh = (int)(j - tile8 * BH);
   const int h = bh % p.H, b = bh / p.H;
+  // a slot table over the heads (one launch per bit-width class of a mixed cache): the heads of
+  // the other classes are theirs altogether, q included, so that the launches share out the work
+  int head_slot = h;
+  if (p.map.slot_dim == 2) {
+    head_slot = p.slot[h];
+    if (head_slot < 0) return;                        // (uniform for the workgroup)
+  }
   const int o = (int)(tile8 * 8u + (id & 7u)) * 256 + threadIdx.x;
   const int lt = o / LR;                              // (LR is a power of two)
   const int col = o - lt * LR;
@@ -260,10 +267,9 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepParams p) {
   pack_octet<BITS, ASYM>(v, vs, vr, vz, fast, vw0, vw1);
 
   // cache row of (b, l, h)
-  int64_t s0 = b, s1 = l, s2 = h;
+  int64_t s0 = b, s1 = l, s2 = head_slot;
   if (p.map.slot_dim == 0) s0 = p.slot[b];
   if (p.map.slot_dim == 1) s1 = p.slot[l];
-  if (p.map.slot_dim == 2) s2 = p.slot[h];
   const bool stored = live && s0 >= 0 && s1 >= 0 && s2 >= 0;
   const int64_t row = s0 * p.map.os0 + s1 * p.map.os1 + s2 * p.map.os2 + p.map.off;
 
