@@ -130,3 +130,28 @@ def test_csv_report_appends_rows(tmp_path):
     rows = rep.rows()
     assert [r['tag'] for r in rows] == ['k', 'v'] and rows[0]['l2_norm_error'] == '0.125' and rows[1]['bits'] == '2'
     assert list(rows[0].keys()) == FIELDS
+
+
+def test_cache_buffer_validation_of_the_row_map_calls():
+    """The quantize-into-cache calls refuse buffers whose row lengths do not match
+    (c, bits, group) or that the row map would overrun, before anything is launched."""
+    import torch
+    from var_q_amd import ops
+    from var_q_amd._lib import VarqError
+    B, H, L, D, bits, g = 2, 3, 5, 64, 4, 32
+    W = D * bits // 32
+    words = torch.zeros(B, H, L, W, dtype=torch.int32)
+    dense = [B, H, L, H * L, L, 1, 0, -1]
+    one = torch.zeros(B, H, L, 1)
+    with pytest.raises(VarqError, match='expected 8 / 2'):
+        ops._check_cache_buffers(D, g, bits, True, words, one, one.clone(), dense, 't')
+    two = torch.zeros(B, H, L, 2)
+    ops._check_cache_buffers(D, g, bits, True, words, two, two.clone(), dense, 't')
+    ops._check_cache_buffers(D, g, bits, False, words, two, None, dense, 't')
+    with pytest.raises(VarqError, match='zp buffer'):
+        ops._check_cache_buffers(D, g, bits, True, words, two, None, dense, 't')
+    with pytest.raises(VarqError, match='reaches row 30'):
+        ops._check_cache_buffers(D, g, bits, True, words, two, two.clone(), [B, H, L, H * L, L, 1, 1, -1], 't')
+    # a slot table over the heads: that dim counts from its first slot
+    ops._check_cache_buffers(D, g, bits, True, words[:, :1].contiguous(), two[:, :1].contiguous(), two[:, :1].contiguous(),
+                             [B, H, L, 1 * L, L, 1, 0, 1], 't')

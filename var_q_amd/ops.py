@@ -68,6 +68,23 @@ def _dt(t: torch.Tensor) -> int:
 # ---------------------------------------------------------------------------
 # row-local (group-wise along the last dim) quantize + pack
 # ---------------------------------------------------------------------------
+def _check_cache_buffers(c: int, group: int, bits: int, asym: bool, words: torch.Tensor, scale: torch.Tensor,
+                         zp: Optional[torch.Tensor], rowmap: Sequence[int], what: str) -> None:
+    """The kernels trust the row map: make sure the buffers it points into have the row
+    lengths the call implies and enough rows for the map's last row (dims addressed
+    through a slot table count from their first slot)."""
+    W, ng = c * bits // 32, c // group
+    if words.shape[-1] != W or scale.shape[-1] != ng:
+        raise VarqError(f'{what}: words / scale rows of {words.shape[-1]} / {scale.shape[-1]} entries, expected {W} / {ng}')
+    if asym and (zp is None or zp.shape != scale.shape or zp.dtype != torch.float32 or not zp.is_contiguous()):
+        raise VarqError(f'{what}: asym needs a contiguous fp32 zp buffer of the shape of scale')
+    n, os_, off, slot_dim = rowmap[0:3], rowmap[3:6], rowmap[6], rowmap[7]
+    last = off + sum((n[d] - 1) * os_[d] for d in range(3) if d != slot_dim and n[d] > 0)
+    rows = min(words.numel() // W, scale.numel() // ng)
+    if min(n) > 0 and not 0 <= last < rows:
+        raise VarqError(f'{what}: the row map reaches row {last} of buffers that hold {rows} rows')
+
+
 def quant_pack_rows(x: torch.Tensor, group: int, bits: int, asym: bool = True, eps: float = 1e-12
                     ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """One-pass quantize+pack with one (scale[, zp]) per `group` contiguous
@@ -98,6 +115,7 @@ def quant_pack_rows_into(x: torch.Tensor, group: int, bits: int, asym: bool, eps
     c = x.shape[-1]
     n_rows = x.numel() // c
     assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
+    _check_cache_buffers(c, group, bits, asym, words, scale, zp, rowmap, 'quant_pack_rows_into')
     lib = _lib.load()
     with _on_device(x.device):
         check(lib.varq_quant_pack_rows(x.data_ptr(), _dt(x), n_rows, c, group, bits, int(asym), eps, i64arr(rowmap),
@@ -119,6 +137,8 @@ def quant_pack_rows_pair_into(x0: torch.Tensor, x1: torch.Tensor, group: int, bi
     c = x0.shape[-1]
     n_rows = x0.numel() // c
     assert rowmap[0] * rowmap[1] * rowmap[2] == n_rows
+    for w, s_, z in (out0, out1):
+        _check_cache_buffers(c, group, bits, asym, w, s_, z, rowmap, 'quant_pack_rows_pair_into')
     lib = _lib.load()
     with _on_device(x0.device):
         check(lib.varq_quant_pack_rows2(x0.data_ptr(), x1.data_ptr(), _dt(x0), n_rows, c, group, bits, int(asym), eps,
@@ -333,6 +353,10 @@ def qkv_prepare_append(qkv: torch.Tensor, q_out: torch.Tensor, group: int, bits:
     B, L, _, H, c = qkv.shape
     assert q_out.shape == (B, H, L, c) and q_out.dtype == torch.bfloat16 and q_out.is_contiguous()
     assert list(rowmap[:3]) == [B, L, H]
+    for w, s_, z in ((k_words, k_scale, k_zp), (v_words, v_scale, v_zp)):
+        _gpu(w, 'words'); _gpu(s_, 'scale')
+        assert w.is_contiguous() and s_.is_contiguous() and w.dtype == torch.int32 and s_.dtype == torch.float32
+        _check_cache_buffers(c, group, bits, asym, w, s_, z, rowmap, 'qkv_prepare_append')
     cos = sin = None
     if rope is not None:
         cos, sin = rope
