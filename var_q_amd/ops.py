@@ -432,9 +432,16 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     assert Wk * 32 == D * k_bits and v_words.shape[3] * 32 == D * v_bits
     assert k_scale.shape[:3] == k_words.shape[:3] and v_scale.shape[:3] == k_words.shape[:3]
     k_group, v_group = D // k_scale.shape[3], D // v_scale.shape[3]
+    for z, sc, n in ((k_zp, k_scale, 'k_zp'), (v_zp, v_scale, 'v_zp')):
+        if z is not None:
+            _gpu(z, n)
+            assert z.shape == sc.shape and z.dtype == torch.float32 and z.is_contiguous(), f'{n} must look like its scale'
+    assert k_scale.dtype == torch.float32 and v_scale.dtype == torch.float32 and k_words.dtype == torch.int32 \
+        and v_words.dtype == torch.int32
+    assert 0 <= Lk <= Lstride, f'Lk={Lk} outside the cache of {Lstride} tokens'
     if out is None:
         out = torch.empty_like(q)
-    assert out.dtype == q.dtype, 'out must have the dtype of q'
+    assert out.dtype == q.dtype and out.shape == q.shape and out.is_contiguous(), 'out must look like q'
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
@@ -491,9 +498,11 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
             _gpu(t, n)
             assert t.dtype == torch.float32 and t.numel() >= nseg * Hkv * D and t.is_contiguous(), \
                 f'{n} must be fp32 [nseg, Hkv, D] (more tables than segments are allowed)'
+    assert k_words.dtype == torch.int32 and v_words.dtype == torch.int32
+    assert 0 <= Lk <= Lstride, f'Lk={Lk} outside the cache of {Lstride} tokens'
     if out is None:
         out = torch.empty_like(q)
-    assert out.dtype == q.dtype, 'out must have the dtype of q'
+    assert out.dtype == q.dtype and out.shape == q.shape and out.is_contiguous(), 'out must look like q'
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
