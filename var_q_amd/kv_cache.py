@@ -182,28 +182,32 @@ class PackedKVCache:
             out = torch.empty_like(q)
         asym = not self.symmetric
         many = len(self.classes) > 1
-        main = torch.cuda.current_stream(q.device)
-        worth = (torch.cuda.is_current_stream_capturing()
-                 or 4.0 * q.shape[0] * q.shape[1] * q.shape[2] * self.len * self.D >= self.concurrent_min_flops)
-        side = self._side_streams(q.device) if many and self.concurrent_classes and worth else None
-        if side:
+        # side streams for the bit-width classes only where the call is large enough to gain from
+        # them (or a graph is being recorded); small calls stay on the caller's stream and skip
+        # every stream lookup
+        side = None
+        if many and self.concurrent_classes and (
+                4.0 * q.shape[0] * q.shape[1] * q.shape[2] * self.len * self.D >= self.concurrent_min_flops
+                or torch.cuda.is_current_stream_capturing()):
+            side = self._side_streams(q.device)
+            main = torch.cuda.current_stream(q.device)
             self._fork.record(main)
-        for i, c in enumerate(self.classes):
+        splits = 1 if many and self.concurrent_classes else self.splits   # classes side by side fill the device already;
+        for i, c in enumerate(self.classes):                              # the same rule on one stream, so both ways add up alike
             # classes cover disjoint heads and disjoint rows of `out`: with side streams their
             # launches share the GPU instead of queueing behind each other half-empty
-            stream = side[i - 1] if side and i else main
-            if stream is not main:
+            args = (q, c.k_words, c.k_scale, c.k_zp if asym else None, c.v_words, c.v_scale, c.v_zp if asym else None,
+                    c.bits, c.bits, self.len, softmax_scale)
+            kw = dict(kv_limit=kv_limit, head_map=c.head_map if many else None, out=out, splits=splits, exact_codes=exact_codes)
+            if side and i:
+                stream = side[i - 1]
                 stream.wait_event(self._fork)
-            with torch.cuda.stream(stream):
-                ops.fused_attn(q, c.k_words, c.k_scale, c.k_zp if asym else None,
-                               c.v_words, c.v_scale, c.v_zp if asym else None,
-                               c.bits, c.bits, self.len, softmax_scale, kv_limit=kv_limit,
-                               head_map=c.head_map if many else None, out=out,
-                               splits=1 if many and self.concurrent_classes else self.splits,   # classes side by side fill the device already; the
-                               exact_codes=exact_codes)                                         # same rule on one stream, so both ways add up alike
-            if stream is not main:
+                with torch.cuda.stream(stream):
+                    ops.fused_attn(*args, **kw)
                 self._join[i - 1].record(stream)
                 main.wait_event(self._join[i - 1])
+            else:
+                ops.fused_attn(*args, **kw)
         return out
 
     def _side_streams(self, device):
