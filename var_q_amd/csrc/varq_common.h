@@ -157,8 +157,8 @@ __device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
 // Cross-lane all-reduce over aligned groups of LANES lanes (power of two).
 // Stages inside a 16-lane row use DPP, wider stages a lane permute.
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
-  // (every lane of these controls has a source lane, so no old value is needed)
-  return u2f((u32)__builtin_amdgcn_mov_dpp((int)f2u(v), CTRL, 0xf, 0xf, false));
+  // (a lane whose partner is switched off keeps its own value)
+  return u2f((u32)__builtin_amdgcn_update_dpp((int)f2u(v), (int)f2u(v), CTRL, 0xf, 0xf, false));
 }
 
 // A fold over aligned groups of up to 16 lanes as one DPP instruction per step, v = OP(v of
@@ -168,6 +168,7 @@ template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
 // vector write of its source: the s_nop in front of every step provides them whatever wrote
 // the source, the one at the end covers a DPP read of the result by whatever follows.
 // v_max_f32 / v_min_f32 return the other operand when one is a quiet NaN, like fmaxf / fminf.
+// A lane whose partner is switched off is not written by the step and so keeps its value.
 #define VARQ_DPP_FOLD_STEP(op, ctrl) "s_nop 1\n\t" op "_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
 #define VARQ_DPP_FOLD(NAME, OP)                                                                     \
   template <int LANES> __device__ __forceinline__ float NAME(float v) {                             \
