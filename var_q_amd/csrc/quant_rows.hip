@@ -103,8 +103,9 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(RowsParams p) {
   int32_t *pwords = second ? p.words1 : p.words;
   float *pscale = second ? p.scale1 : p.scale;
   float *pzp = second ? p.zp1 : p.zp;
-  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
-  const int tile = blockIdx.x;
+  // (strided input: the pair index is the fastest grid dim, see the launcher)
+  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = p.strided ? blockIdx.x : blockIdx.y;
+  const int tile = p.strided ? blockIdx.y : blockIdx.x;
 
   int64_t s0 = i0, s1 = i1;
   if (p.map.slot_dim == 0) s0 = p.slot[i0];
@@ -201,7 +202,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   int32_t *pwords = second ? p.words1 : p.words;
   float *pscale = second ? p.scale1 : p.scale;
   float *pzp = second ? p.zp1 : p.zp;
-  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = blockIdx.y;
+  const int64_t i0 = blockIdx.z - (second ? (unsigned)p.map.n0 : 0u), i1 = p.strided ? blockIdx.x : blockIdx.y;
+  const int tile = p.strided ? blockIdx.y : blockIdx.x;
   int64_t s0 = i0, s1 = i1;
   if (p.map.slot_dim == 0) s0 = p.slot[i0];
   if (p.map.slot_dim == 1) s1 = p.slot[i1];
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   Raw8<DT> *stage = lds_stage[wv];
   constexpr float kMin = (float)QRange<BITS>::kMin, kMax = (float)QRange<BITS>::kMax;
-  const int w0 = blockIdx.x * 1024 + wv * 256;       // first octet of this wave's window, inside the pair
+  const int w0 = tile * 1024 + wv * 256;             // first octet of this wave's window, inside the pair
 
   // 1 KiB per load instruction: contiguous, or whole rows in_s2 elements apart.  Only the
   // offsets are formed under the (launch-uniform) branch; the four loads follow it together.
@@ -419,7 +421,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows32_kernel(RowsParams p) {
 template <int DT, int BITS, bool ASYM>
 int launch_lpg(const RowsParams &p, int lpg, dim3 grid, hipStream_t st) {
   if (lpg >= 4) {   // groups of >= 32 channels: 4 octets per lane, 1024 octets per workgroup
-    dim3 g32((unsigned)((p.octets_per_pair + 1023) / 1024), grid.y, grid.z);
+    const unsigned t32 = (unsigned)((p.octets_per_pair + 1023) / 1024);
+    dim3 g32(p.strided ? grid.x : t32, p.strided ? t32 : grid.y, grid.z);
     const bool dense = (p.map.os2 == 1) && (p.map.slot_dim != 2);
     switch (lpg / 4) {
 #define VARQ_CASE32(L)                                                                                            \
@@ -482,7 +485,8 @@ static int quant_pack_rows_launch(const char *who, const void *x, const void *x1
   // The rows a workgroup walks should be neighbours in the output: if those are the rows along
   // the map's middle dim (and there are at least as many of them as along the inner one), the
   // two dims change roles and the workgroup reads its rows n2 * c elements apart.
-  if (m.os1 == 1 && m.os2 != 1 && m.slot_dim != 1 && p.c8_shift >= 0 && m.n1 >= m.n2 && m.n1 * m.n2 * c < (1ll << 31)) {
+  if (m.os1 == 1 && m.os2 != 1 && m.slot_dim != 1 && p.c8_shift >= 0 && m.n1 >= m.n2 && m.n1 * m.n2 * c < (1ll << 31) &&
+      (m.n1 * p.c8 + 255) / 256 <= 65535) {
     RowMap t = m;
     t.n1 = m.n2; t.n2 = m.n1; t.os1 = m.os2; t.os2 = m.os1;
     t.slot_dim = m.slot_dim == 2 ? 1 : m.slot_dim;
@@ -497,7 +501,11 @@ static int quant_pack_rows_launch(const char *who, const void *x, const void *x1
   p.blocks_per_pair = (p.octets_per_pair + 255) / 256;
   VARQ_CHECK_ARG(p.octets_per_pair < (1ll << 31) - 256, "%s: more than 2^31 octets per (i0,i1) pair", who);
   VARQ_CHECK_ARG(m.n1 <= 65535 && m.n0 * (two ? 2 : 1) <= 65535, "%s: n0 (times the number of tensors) and n1 of the row map must be <= 65535", who);
+  // strided input: the workgroups in flight together should read whole stretches of the input
+  // between them, so the pair index (the head, for [B, L, H, c] input) is the fastest grid dim
+  // and the tiles of tokens lie along y (their count was bounded where the roles were swapped)
   dim3 grid((unsigned)p.blocks_per_pair, (unsigned)m.n1, (unsigned)(m.n0 * (two ? 2 : 1)));
+  if (p.strided) grid = dim3((unsigned)m.n1, (unsigned)p.blocks_per_pair, grid.z);
   hipStream_t st = (hipStream_t)stream;
   int rc = -1;
   if (x_dtype == VARQ_F32) rc = launch_dt<VARQ_F32>(p, bits, asym, lpg, grid, st);
