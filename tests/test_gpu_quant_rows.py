@@ -253,3 +253,50 @@ def test_token_major_input_into_a_head_major_cache(dev, bits, group, asym, dtype
     assert torch.equal(a_k[0][:, :, sl].cpu(), O.pack_last_dim(q, bits)[0])
     assert torch.equal(a_k[1][:, :, sl].cpu(), s) and (not asym or torch.equal(a_k[2][:, :, sl].cpu(), z))
     assert bool((a_k[0][:, :, :start] == 7).all()) and bool((a_k[0][:, :, start + n:] == 7).all())
+
+
+def test_token_major_seeded_random_shapes(dev):
+    """Forty seeded random shapes of a token-major step into a head-major cache (rows of 32 to
+    256 channels, also 96: twelve octets per row, not a power of two; one to seventy tokens against one to nine heads;
+    every width and dtype; with and without a slot table over the heads): the cache equals the
+    oracle's codes, scales and zero-points at the step's rows and is untouched elsewhere."""
+    import random
+    rnd = random.Random(20240607)
+    for case in range(40):
+        c = rnd.choice([32, 64, 96, 128, 256])
+        bits = rnd.choice([2, 4, 8])
+        groups = [g for g in (8, 16, 32, 64, 128, 256) if c % g == 0 and (g // 8) & (g // 8 - 1) == 0 and (bits != 2 or g >= 16)]
+        group = rnd.choice(groups)
+        asym = rnd.random() < 0.6
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        B, n, H = rnd.randint(1, 3), rnd.randint(1, 70), rnd.randint(1, 9)
+        start = rnd.randint(0, 5)
+        Lmax = start + n + rnd.randint(0, 4)
+        with_slot = H > 1 and rnd.random() < 0.5
+        heads = list(range(H))
+        if with_slot:
+            heads = rnd.sample(range(H), rnd.randint(1, H))     # (in any order: the slot table maps head -> place)
+        g = torch.Generator().manual_seed(1000 + case)
+        x = (torch.randn(B, n, H, c, generator=g) * rnd.choice([0.01, 1.0, 30.0])).to(dtype)
+        slot = None
+        if with_slot:
+            slot = torch.full((H,), -1, dtype=torch.int32)
+            for i, h in enumerate(heads):
+                slot[h] = i
+            slot = slot.to(dev)
+        hc, W, ng = len(heads), c * bits // 32, c // group
+        words = torch.full((B, hc, Lmax, W), 7, dtype=torch.int32, device=dev)
+        scale = torch.full((B, hc, Lmax, ng), 7.0, device=dev)
+        zp = torch.full((B, hc, Lmax, ng), 7.0, device=dev) if asym else None
+        note('quant_pack_rows token-major random', case, (B, n, H, c), bits, group, asym, dtype, 'slot' if with_slot else 'all heads')
+        ops.quant_pack_rows_into(x.to(dev), group, bits, asym, 1e-12, words, scale, zp,
+                                 [B, n, H, hc * Lmax, 1, Lmax, start, 2 if with_slot else -1], slot)
+        torch.cuda.synchronize()
+        q, s, z = O.quant_groupwise(x.transpose(1, 2)[:, heads].contiguous(), group, bits, asym)
+        sl = slice(start, start + n)
+        assert torch.equal(words[:, :, sl].cpu(), O.pack_last_dim(q, bits)[0]), f'case {case}: packed words differ'
+        assert torch.equal(scale[:, :, sl].cpu(), s), f'case {case}: scales differ'
+        if asym:
+            assert torch.equal(zp[:, :, sl].cpu(), z), f'case {case}: zero-points differ'
+        assert bool((words[:, :, :start] == 7).all()) and bool((words[:, :, start + n:] == 7).all()), f'case {case}: rows outside the step written'
+        assert bool((scale[:, :, :start] == 7).all()) and bool((scale[:, :, start + n:] == 7).all())
