@@ -207,3 +207,45 @@ def test_slot_table_over_heads_leaves_other_heads_alone(dev):
         assert torch.equal(w[:, :, 3:3 + L].cpu(), O.pack_last_dim(cq, bits)[0])
         assert torch.equal(s[:, :, 3:3 + L].cpu(), cs) and torch.equal(z[:, :, 3:3 + L].cpu(), cz)
         assert bool((w[:, :, :3] == 7).all()) and bool((w[:, :, 3 + L:] == 7).all())
+
+
+def test_seeded_random_shapes(dev):
+    """Thirty seeded random calls: one to 300 tokens (up to 19 tiles of 16 tokens at c = 128, so
+    tile counts on either side of the eight that one round of the workgroup order deals out),
+    one to three batch entries, one to seven heads, every head dim, width and input type, each
+    stage of the pipeline on or off."""
+    import random
+    rnd = random.Random(777)
+    for case in range(30):
+        c = rnd.choice([32, 64, 128])
+        bits = rnd.choice([2, 4, 8])
+        group = rnd.choice([g for g in (8, 16, 32, 64, 128) if g <= c and (bits != 2 or g >= 16)])
+        asym = rnd.random() < 0.7
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        B, L, H = rnd.randint(1, 3), rnd.randint(1, 300), rnd.randint(1, 7)
+        l2norm, with_mul, with_rope = rnd.random() < 0.7, rnd.random() < 0.5, rnd.random() < 0.6
+        start, off = rnd.randint(0, 30), rnd.randint(0, 3)
+        g = torch.Generator().manual_seed(5000 + case)
+        qkv = (torch.randn(B, L, 3, H, c, generator=g) * rnd.choice([0.05, 1.0, 20.0])).to(dtype)
+        mul = (torch.rand(H, generator=g) * 5 + 0.5) if with_mul else None
+        rope = hooks.rope2d_tables(c, [(19, 19)]) if with_rope else None      # 361 rows >= start + L
+        qo, ko, vo = O.prepare_qkv(qkv, mul, l2norm, 1e-12, rope, start)
+        Lmax, W, ns = L + off + rnd.randint(0, 2), c * bits // 32, c // group
+        mk = lambda last, dt: torch.full((B, H, Lmax, last), 7, dtype=dt, device=dev)
+        kw, vw = mk(W, torch.int32), mk(W, torch.int32)
+        ks, kz, vs, vz = (mk(ns, torch.float32) for _ in range(4))
+        q_out = torch.empty(B, H, L, c, dtype=torch.bfloat16, device=dev)
+        note('qkv_prepare random', case, (B, L, H, c), bits, group, asym, dtype, l2norm, with_mul, with_rope, start, off)
+        ops.qkv_prepare_append(qkv.to(dev), q_out, group, bits, asym, 1e-12, kw, ks, kz if asym else None,
+                               vw, vs, vz if asym else None, [B, L, H, H * Lmax, 1, Lmax, off, -1], None,
+                               None if mul is None else mul.to(dev), l2norm, 1e-12,
+                               None if rope is None else (rope[0].to(dev), rope[1].to(dev)), start)
+        torch.cuda.synchronize()
+        assert torch.equal(q_out.cpu().view(torch.int16), qo.view(torch.int16)), f'case {case}: prepared q differs'
+        sl = slice(off, off + L)
+        for name, x, w, s, z in (('k', ko, kw, ks, kz), ('v', vo, vw, vs, vz)):
+            cq, cs, cz = O.quant_groupwise(x, group, bits, asym)
+            assert torch.equal(s[:, :, sl].cpu(), cs), f'case {case}: {name} scale differs'
+            assert not asym or torch.equal(z[:, :, sl].cpu(), cz), f'case {case}: {name} zero-point differs'
+            assert torch.equal(w[:, :, sl].cpu(), O.pack_last_dim(cq, bits)[0]), f'case {case}: {name} packed words differ'
+            assert bool((w[:, :, :off] == 7).all()) and bool((w[:, :, off + L:] == 7).all()), f'case {case}: rows outside the step written'
