@@ -141,3 +141,30 @@ def test_pack_unpack_word_tails_and_unaligned_words(dev, bits, rows, c, word_off
     _lib.check(lib.varq_unpack(words.data_ptr(), rows, c, bits, back.data_ptr(), st), 'varq_unpack')
     torch.cuda.synchronize()
     assert torch.equal(back[:rows * c].cpu().reshape(rows, c), q) and int(back[rows * c]) == 99
+
+
+@pytest.mark.parametrize('bits', [2, 4, 8])
+@pytest.mark.parametrize('H,c', [(16, 128), (8, 64), (4, 32), (2, 16), (16, 64)])
+def test_dequant_table_over_the_inner_rows(dev, bits, H, c):
+    """One scale per (head, channel) of a token-major tensor [B,L,H,c] (the reference's default
+    method in layout BLHc, VAR_Q/quant.py:84-88): the call reads the H rows of a token as one
+    long row of H*c channels where that is a power-of-two number of octets up to 256.  Dense
+    tensor and a window of a longer cache, symmetric and affine, fp32 and bf16 out."""
+    g = torch.Generator().manual_seed(bits * 100 + H + c)
+    lo, hi = O.qrange(bits)
+    B, L, Lcap, first = 2, 301, 340, 17
+    q = torch.randint(lo, hi + 1, (B, Lcap, H, c), generator=g, dtype=torch.int8)
+    words, _ = O.pack_last_dim(q, bits)
+    s = torch.rand(1, 1, H, c, generator=g) + 0.01
+    z = torch.randint(-9, 9, (1, 1, H, c), generator=g).float()
+    W = words.shape[-1]
+    for asym in (False, True):
+        for out_dtype in (torch.float32, torch.bfloat16):
+            note('dequant table over the inner rows', bits, H, c, asym, out_dtype)
+            zz = z if asym else None
+            want = (O.dequant_asym(q, s, z) if asym else O.dequant_sym(q, s)).to(out_dtype)
+            got = ops.dequant(words.to(dev), s.to(dev), None if zz is None else zz.to(dev), c, bits, out_dtype)
+            assert torch.equal(got.cpu(), want)
+            win = ops.dequant_window(words.to(dev), s.to(dev), None if zz is None else zz.to(dev), (B, L, H, c), [0, 0, c, 1],
+                                     1, bits, [B, L, H, Lcap * H, H, 1, first * H, -1], out_dtype)
+            assert torch.equal(win.cpu(), want[:, first:first + L])

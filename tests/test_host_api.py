@@ -155,3 +155,25 @@ def test_cache_buffer_validation_of_the_row_map_calls():
     # a slot table over the heads: that dim counts from its first slot
     ops._check_cache_buffers(D, g, bits, True, words[:, :1].contiguous(), two[:, :1].contiguous(), two[:, :1].contiguous(),
                              [B, H, L, 1 * L, L, 1, 0, 1], 't')
+
+
+def test_rows_read_as_channels_for_per_row_tables():
+    """The host-side rewrite of a [n0,n1,n2,c] dequantization with one scale per (i2, channel)
+    into long rows applies only where the bytes allow it."""
+    from var_q_amd import ops
+    f = ops._rows_as_channels
+    # [B,L,H,c] = [2,100,16,128], table [1,1,H,c]: long rows of 2048 channels = 256 octets
+    assert f(True, [2, 100, 16, 128], [0, 0, 128, 1], 1, 4, None) == ([1, 2, 100, 2048], [0, 0, 0, 1], None)
+    # a window of a cache with room for 160 tokens per batch entry
+    window = f(True, [2, 100, 16, 128], [0, 0, 128, 1], 1, 8, [2, 100, 16, 160 * 16, 16, 1, 32, -1])
+    assert window == ([1, 2, 100, 2048], [0, 0, 0, 1], [1, 2, 100, 0, 160, 1, 2, -1])
+    same = lambda *a: f(*a) == (a[1], a[2], a[5])
+    assert same(True, [2, 100, 30, 64], [0, 0, 64, 1], 1, 8, None)          # 240 octets: not a power of two
+    assert same(True, [2, 100, 32, 128], [0, 0, 128, 1], 1, 8, None)        # 512 octets: too long
+    assert same(True, [2, 100, 3, 30], [0, 0, 30, 1], 1, 8, None)           # rows that are not whole octets
+    assert same(True, [2, 100, 2, 8], [0, 0, 8, 1], 1, 2, None)             # 2-bit rows that are not whole words
+    assert same(False, [2, 100, 16, 128], [0, 0, 128, 1], 1, 8, None)       # int8 codes, not packed words
+    assert same(True, [2, 100, 16, 128], [0, 128 * 16, 128, 1], 1, 8, None) # the scale depends on i1 too
+    assert same(True, [2, 100, 16, 128], [0, 0, 4, 1], 32, 4, None)         # group-wise scales
+    assert same(True, [2, 100, 16, 128], [0, 0, 128, 1], 1, 8, [2, 100, 16, 100 * 16, 1, 100, 0, -1])   # rows of a pair apart
+    assert same(True, [2, 100, 16, 128], [0, 0, 128, 1], 1, 8, [2, 100, 16, 160 * 16, 16, 1, 8, -1])    # window starts mid-row

@@ -311,6 +311,7 @@ def dequant(q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor], c:
         shape = [1, 1, n0 * n1 * n2, c]
     elif strides[0] == 0 and strides[1] == 0:
         pass
+    shape, strides, _ = _rows_as_channels(packed, shape, strides, group, bits, None)
     with _on_device(q.device):
         check(lib.varq_dequant(q.data_ptr() if packed else None, None if packed else q.data_ptr(),
                                scale.data_ptr(), _ptr(zp), i64arr(shape), i64arr(strides), group, bits, None,
@@ -327,13 +328,34 @@ def dequant_window(words: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.
     packed = words.dtype == torch.int32
     assert packed or words.dtype == torch.int8
     out = torch.empty(tuple(shape4), dtype=out_dtype, device=words.device)
+    shape4, scale_strides4, in_rowmap = _rows_as_channels(packed, shape4, scale_strides4, group, bits, in_rowmap)
     lib = _lib.load()
     with _on_device(words.device):
         check(lib.varq_dequant(words.data_ptr() if packed else None, None if packed else words.data_ptr(),
                                scale.data_ptr(), _ptr(zp), i64arr(shape4),
-                               i64arr(scale_strides4), group, bits, i64arr(in_rowmap), out.data_ptr(),
-                               _DT[out_dtype], _stream(words)), 'varq_dequant')
+                               i64arr(scale_strides4), group, bits, None if in_rowmap is None else i64arr(in_rowmap),
+                               out.data_ptr(), _DT[out_dtype], _stream(words)), 'varq_dequant')
     return out
+
+
+def _rows_as_channels(packed: bool, shape4, strides4, group: int, bits: int, rowmap):
+    """One scale per (i2, channel) whatever i0 and i1 (the per-(head, channel) table of a
+    [B,L,H,c] tensor: VAR_Q/quant.py:84-88 in layout BLHc), the n2 rows of an (i0, i1) pair next
+    to each other in the window: the same bytes read as [1, n0, n1, n2*c] with one scale per
+    channel of the long rows, which is the form the kernel has its table path for (a lane keeps
+    one vector of eight scales for all its pieces instead of loading eight per piece).  The
+    long rows must be a power-of-two number of octets, at most 256, and every row whole words."""
+    n0, n1, n2, c = [int(v) for v in shape4]
+    c8l = n2 * c // 8
+    if not packed or group != 1 or n2 <= 1 or c % 8 or (c * bits) % 32 or list(strides4) != [0, 0, c, 1] \
+            or c8l > 256 or c8l & (c8l - 1):
+        return shape4, strides4, rowmap
+    if rowmap is None:
+        return [1, n0, n1, n2 * c], [0, 0, 0, 1], None
+    rn0, rn1, rn2, os0, os1, os2, off, slot_dim = [int(v) for v in rowmap]
+    if (rn0, rn1, rn2) != (n0, n1, n2) or os2 != 1 or slot_dim >= 0 or os0 % n2 or os1 % n2 or off % n2:
+        return shape4, strides4, rowmap
+    return [1, n0, n1, n2 * c], [0, 0, 0, 1], [1, n0, n1, 0, os0 // n2, os1 // n2, off // n2, -1]
 
 
 # ---------------------------------------------------------------------------
