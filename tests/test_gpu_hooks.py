@@ -12,7 +12,7 @@ import torch
 
 import varq_oracle as O
 from gpu_util import note
-from var_q_amd import hooks
+from var_q_amd import VAR_Q, hooks
 
 pytestmark = pytest.mark.gpu
 
@@ -259,3 +259,38 @@ def test_var_module_in_fp16_the_dtype_of_its_autocast(dev, backend, layout):
         rng = a.abs().max().item()
         assert (a - b).abs().max().item() <= 2e-2 * max(rng, 1.0), (p, (a - b).abs().max().item(), rng)
         assert _cos(a, b) >= 0.9995
+
+
+class _PlainProtocol:
+    """The package's quantizer behind the reference's call signature only (no out_dtype): the
+    drop-in module then casts the fp32 result itself, as the reference's modules do."""
+
+    def __init__(self, **kw):
+        self.q = VAR_Q(**kw)
+
+    def use_var_q(self, item):
+        return self.q.use_var_q(item)
+
+    def __getattr__(self, name):
+        return getattr(self.q, name)
+
+
+@pytest.mark.parametrize('layout,method', [('BLHc', 'G_SCALE_HEAD_DIM'), ('BHLc', 'G_SCALE_HEAD_DIM'), ('BLHc', 'G_TOKEN_HEAD')])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_dropin_module_dequantizes_into_the_attention_dtype(dev, layout, method, dtype):
+    """fused=False with this package's quantizer: K and V come back in the module's compute
+    dtype directly; the module's output is bit for bit the one it gives when the quantizer
+    returns fp32 and the module casts."""
+    torch.manual_seed(9)
+    C, H = 256, 4
+    kw = dict(embed_dim=C, num_heads=H, layout=layout, q_bits=8, quant_method=method, enable_quantization=True, max_tokens=40)
+    a_mod = hooks.VarSelfAttention(0, fused=False, **kw).to(dev).to(dtype)
+    b_mod = hooks.VarSelfAttention(0, fused=False, quantizer_factory=_PlainProtocol, **kw).to(dev).to(dtype)
+    b_mod.load_state_dict(a_mod.state_dict())
+    a_mod.kv_caching(True)
+    b_mod.kv_caching(True)
+    for n in (1, 4, 9, 16):
+        note('hooks dropin into attention dtype', layout, method, dtype, n)
+        x = torch.randn(2, n, C, device=dev, dtype=dtype)
+        assert torch.equal(a_mod(x), b_mod(x))
+    assert isinstance(a_mod.k_quant, VAR_Q) and not isinstance(b_mod.k_quant, VAR_Q)

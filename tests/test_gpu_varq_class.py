@@ -280,6 +280,26 @@ def test_use_var_q_keeps_the_dequantized_prefix(dev, fmt, method, keep):
 
 
 @pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
+@pytest.mark.parametrize('method', ['G_SCALE_HEAD_DIM', 'G_TOKEN', 'G_HEAD_DIM', 'G_TENSOR', 'G_TOKEN_HEAD', 'G_SCALE'])
+@pytest.mark.parametrize('bits,pack', [(8, True), (4, True), (8, False)])
+def test_use_var_q_into_the_attention_dtype(dev, fmt, method, bits, pack):
+    """use_var_q(x, out_dtype=...) and dequant_all(out_dtype) give the fp32 result of the
+    reference's protocol rounded once to that type, i.e. what the attention module's own cast of
+    the fp32 tensor gives (VAR/models/basic_var.py:158), at every step."""
+    note('VAR_Q dequantized into the attention dtype', fmt, method, bits, pack)
+    ref = O.OracleVARQ(bits, fmt, method, pack_to_int32=pack)
+    for out_dtype in (torch.bfloat16, torch.float16):
+        gpu = VAR_Q(bits, fmt, method, pack_to_int32=pack)
+        ref = O.OracleVARQ(bits, fmt, method, pack_to_int32=pack)
+        for i, x in enumerate(_steps(fmt, torch.float32, seed=31)):
+            want = ref.use_var_q(x).to(out_dtype)
+            got = gpu.use_var_q(x.to(dev), out_dtype=out_dtype)
+            assert got.dtype == out_dtype and torch.equal(got.cpu(), want), f'step {i} {out_dtype}'
+            assert torch.equal(gpu.dequant_all(out_dtype).cpu(), want)
+            assert gpu.dequant_all().dtype == torch.float32
+
+
+@pytest.mark.parametrize('fmt', ['BLHc', 'BHLc'])
 @pytest.mark.parametrize('method', ['G_SCALE_HEAD_DIM', 'G_TOKEN_HEAD', 'G_TOKEN'])
 def test_empty_step_is_refused_and_changes_nothing(dev, fmt, method):
     """A step without tokens: the reference fails in its amax over an empty dim

@@ -194,8 +194,16 @@ class _QuantizedSelfAttention(nn.Module):
             return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
         if self.caching:
             if self.enable_quantization:
-                k = self.k_quant.use_var_q(k)
-                v = self.v_quant.use_var_q(v)
+                # (dequantized straight into the attention's dtype: the values `.to(out_dtype)` of
+                # the reference's fp32 result would have)
+                # (only this package's quantizer takes the argument; any other factory's is called
+                # as the reference calls it)
+                if out_dtype in (torch.bfloat16, torch.float16) and isinstance(self.k_quant, VAR_Q):
+                    k = self.k_quant.use_var_q(k, out_dtype=out_dtype)
+                    v = self.v_quant.use_var_q(v, out_dtype=out_dtype)
+                else:
+                    k = self.k_quant.use_var_q(k)
+                    v = self.v_quant.use_var_q(v)
             elif self.cached_k is None:
                 self.cached_k, self.cached_v = k, v
             else:

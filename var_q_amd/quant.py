@@ -434,25 +434,31 @@ class VAR_Q:
                 self._tok_zp.append(self.zp.expand(*shape))
 
     # ---------------- dequantize ----------------
-    def _dequant(self, q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor]) -> torch.Tensor:
+    def _dequant(self, q: torch.Tensor, scale: torch.Tensor, zp: Optional[torch.Tensor],
+                 out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
         if self.pack_to_int32:
             assert self._pack_meta is not None, "pack meta is missing"
             c = self._pack_meta['orig_c']
         else:
             c = q.shape[-1]
-        return _dequant_views(q, scale, zp, c, self.quant_bits)
+        return _dequant_views(q, scale, zp, c, self.quant_bits, out_dtype)
 
-    def dequant_current(self) -> torch.Tensor:
-        return self._dequant(self.quantized_item, self.scale, self.zp)
+    def dequant_current(self, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        return self._dequant(self.quantized_item, self.scale, self.zp, out_dtype)
 
-    def dequant_all(self) -> torch.Tensor:
+    def dequant_all(self, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The whole cache dequantized (VAR_Q/quant.py:216-224: fp32).  out_dtype bfloat16 / float16
+        gives the fp32 product rounded once to that type -- bit for bit what `.to(out_dtype)` of the
+        fp32 result is, without writing and re-reading the fp32 tensor."""
         if self.cached_item is None:
-            return self.dequant_current()
-        return self._dequant(self.cached_item, self.cached_scale, self.cached_zp)
+            return self.dequant_current(out_dtype)
+        return self._dequant(self.cached_item, self.cached_scale, self.cached_zp, out_dtype)
 
-    def use_var_q(self, item: torch.Tensor) -> torch.Tensor:
+    def use_var_q(self, item: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         """quant + cache + dequant_all (VAR_Q/quant.py:226-230).  Like the reference, the whole
         cache is dequantized into a fresh fp32 tensor at every step and nothing of it is kept.
+        out_dtype (an addition): the type the caller would cast the result to anyway (the attention
+        modules do, VAR/models/basic_var.py:158); see dequant_all.  Ignored with keep_dequantized.
 
         With `keep_dequantized=True` (constructor) the fp32 values are kept from step to step
         instead: under the appending methods the codes and scales of earlier steps never change,
@@ -466,7 +472,7 @@ class VAR_Q:
         self.quant(item)
         self.cache()
         if not self.keep_dequantized:
-            return self.dequant_all()
+            return self.dequant_all(out_dtype or torch.float32)
         d, n = self._c_deq, self.quantized_item.size(self.dim_cat)
         if self.quant_method == 'G_HEAD_DIM' or self._c_item.buf is None or d.dim != self.dim_cat or d.len + n != self._c_item.len:
             # (the replacing method; or the kept values are not those of the cache's earlier steps:
