@@ -445,7 +445,10 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
   const int xcd = wg & 7, slot_s = wg >> 3;
   const int split = p.nsplit > 1 ? slot_s % p.nsplit : 0;
   const int slot = p.nsplit > 1 ? slot_s / p.nsplit : slot_s;
-  const int bh = (slot / p.q_tiles) * 8 + xcd;
+  // (a token-major cache: the key rows of neighbouring heads share cache lines, so an XCD takes a
+  // run of consecutive (batch, head) pairs there instead of every eighth)
+  const int grp = slot / p.q_tiles;
+  const int bh = p.kv_hs == 1 && p.kv_ts > 1 ? xcd * ((p.bh_total + 7) >> 3) + grp : grp * 8 + xcd;
   const int qt = slot % p.q_tiles;
   if (bh >= p.bh_total) return;
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
@@ -1495,7 +1498,8 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   static_assert(kFewQueries <= 64, "at most two query tiles");
   const int xcd = blockIdx.x, split = blockIdx.y, slot = blockIdx.z;
   const int qt = p.q_tiles == 2 ? (slot & 1) : 0;
-  const int bh = (p.q_tiles == 2 ? (slot >> 1) : slot) * 8 + xcd;
+  const int grp = p.q_tiles == 2 ? (slot >> 1) : slot;
+  const int bh = p.kv_hs == 1 && p.kv_ts > 1 ? xcd * ((p.bh_total + 7) >> 3) + grp : grp * 8 + xcd;   // (as in the kernel above)
   if (bh >= p.bh_total) return;
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
   const int hq = p.head_map ? p.head_map[hs] : hs;
@@ -1518,8 +1522,10 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
   const int nb = (kv_end + FQ_BK - 1) / FQ_BK;
   const int b_begin = split * p.fq_share_blocks, b_end = min(b_begin + p.fq_share_blocks, nb);
   // Block j of the share goes to wavefront (j + rot) % 4: the wavefront that gets the odd block
-  // more differs between the workgroups that are likely to sit on one compute unit.
-  const int slot_s = slot * p.nsplit + split;
+  // more differs between the workgroups that are likely to sit on one compute unit.  (A function
+  // of the (batch, head) pair, the query tile and the share only, not of where the workgroup
+  // sits in the grid: the two cache layouts add up in the same order.)
+  const int slot_s = ((p.q_tiles == 2 ? ((bh >> 3) << 1) | qt : (bh >> 3))) * p.nsplit + split;
   const int rot = (slot_s + (slot_s >> 5)) & 3;
   const int blk0 = b_begin + ((wave - rot) & 3);
 
