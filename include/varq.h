@@ -41,7 +41,9 @@ enum varq_status {
 enum varq_dtype { VARQ_F32 = 0, VARQ_BF16 = 1, VARQ_F16 = 2 };
 
 /* K/V tensor layouts of the reference's quantizer (qkv_format, VAR_Q/quant.py:34-37) */
-enum varq_layout { VARQ_LAYOUT_BHLC = 0, VARQ_LAYOUT_BLHC = 1 };
+enum varq_layout { VARQ_LAYOUT_BHLC = 0, VARQ_LAYOUT_BLHC = 1,
+                   /* attention calls only: q and the cache as VARQ_LAYOUT_BHLC, out as VARQ_LAYOUT_BLHC */
+                   VARQ_LAYOUT_BHLC_OUT_BLHC = 2 };
 
 /*
  * What the matrix operands of the fused attention hold.
@@ -224,7 +226,11 @@ int varq_dequant(const int32_t *words, const int8_t *codes_i8, const float *scal
  *              [B, Lq, Hq, D], words [B, Lk_stride, Hkv, D*bits/32], scales
  *              [B, Lk_stride, Hkv, D/group] -- the layout of the reference's
  *              flash-attention call (VAR/models/basic_var.py:127-131,157-158) and the
- *              default qkv_format of its quantizer.
+ *              default qkv_format of its quantizer.  VARQ_LAYOUT_BHLC_OUT_BLHC: q and
+ *              the cache as VARQ_LAYOUT_BHLC, out [B, Lq, Hq, D], which is how the
+ *              attention modules hand the result to their output projection
+ *              (VAR/models/basic_var.py:160, Infinity/infinity/models/basic.py:347):
+ *              no transposing copy behind the call.
  *   workspace, workspace_bytes, splits
  *              A launch with few query blocks over a long cache (a small batch, a
  *              step of a few hundred queries) leaves compute units idle or ends in a

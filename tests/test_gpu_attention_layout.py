@@ -63,3 +63,44 @@ def test_stepwise_tables(dev, D, splits):
     torch.cuda.synchronize()
     assert not bool(torch.isnan(a.float()).any())
     assert torch.equal(b.transpose(1, 2), a)
+
+
+@pytest.mark.parametrize('D,group,bits,Lq,Lk,splits', [(128, 128, 4, 150, 700, 1), (128, 128, 4, 150, 700, 3), (128, 64, 8, 16, 2100, 0),
+                                                       (128, 128, 4, 64, 2100, 0), (64, 32, 2, 300, 500, 1), (64, 64, 8, 256, 680, 2)])
+def test_tokens_first_output_of_a_heads_first_call(dev, D, group, bits, Lq, Lk, splits):
+    """out_layout='BLHc' with q and the cache heads first: the same bits as the heads-first
+    output, transposed; rows of heads outside the head map stay untouched.  Covers the general
+    kernel with and without shared keys, the few-queries kernel (16 and 64 queries over 2100
+    keys) and the kernel that combines the shares."""
+    B, Hq = 2, 5
+    heads = [3, 0, 4]
+    gen = torch.Generator(device=dev).manual_seed(D + bits + Lq)
+    k = torch.randn(B, len(heads), Lk, D, device=dev, generator=gen).bfloat16()
+    v = torch.randn(B, len(heads), Lk, D, device=dev, generator=gen).bfloat16()
+    q = torch.randn(B, Hq, Lq, D, device=dev, generator=gen).bfloat16()
+    kq, vq = ops.quant_pack_rows(k, group, bits, True), ops.quant_pack_rows(v, group, bits, True)
+    hm = torch.tensor(heads, dtype=torch.int32, device=dev)
+    note('fused_attn tokens-first out', D, group, bits, Lq, Lk, splits)
+    a = torch.full((B, Hq, Lq, D), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.fused_attn(q, *kq, *vq, bits, bits, Lk, 1 / math.sqrt(D), head_map=hm, out=a, splits=splits)
+    b = torch.full((B, Lq, Hq, D), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.fused_attn(q, *kq, *vq, bits, bits, Lk, 1 / math.sqrt(D), head_map=hm, out=b, splits=splits, out_layout='BLHc')
+    c = ops.fused_attn(q[:, heads].contiguous(), *kq, *vq, bits, bits, Lk, 1 / math.sqrt(D), splits=splits, out_layout='BLHc')
+    torch.cuda.synchronize()
+    assert torch.equal(b.transpose(1, 2), a)
+    assert c.shape == (B, Lq, len(heads), D) and torch.equal(c.transpose(1, 2), a[:, heads])
+    assert bool((b[:, :, [1, 2]] == 7.0).all()) and not bool((b[:, :, heads] == 7.0).all())
+
+
+def test_tokens_first_output_with_tables(dev):
+    B, H, D, bits, L = 2, 3, 64, 8, 700
+    gen = torch.Generator(device=dev).manual_seed(5)
+    kw = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, L, D * bits // 32), device=dev, generator=gen, dtype=torch.int64).int()
+    vw = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, L, D * bits // 32), device=dev, generator=gen, dtype=torch.int64).int()
+    ks, vs = (torch.rand(1, H, D, device=dev, generator=gen) * 0.02 + 0.01 for _ in range(2))
+    q = torch.randn(B, H, 200, D, device=dev, generator=gen).bfloat16()
+    note('fused_attn_channel tokens-first out')
+    a = ops.fused_attn_channel(q, kw, ks, None, vw, vs, None, bits, L, 0.1)
+    b = ops.fused_attn_channel(q, kw, ks, None, vw, vs, None, bits, L, 0.1, out_layout='BLHc')
+    torch.cuda.synchronize()
+    assert b.shape == (B, 200, H, D) and torch.equal(b.transpose(1, 2), a)

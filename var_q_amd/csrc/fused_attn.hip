@@ -100,9 +100,9 @@ struct AttnParams {
   int f16;   // q, out and the MFMA operands are fp16 (host side only: it selects the instantiation)
   int fq_share_blocks;   // few-queries kernel: 32-key blocks per share of the keys
   // memory layout, in rows (a row = the D values of one token of one head):
-  // q/out row = b*q_bs + h*q_hs + i*q_ts, key row = b*kv_bs + slot*kv_hs + j*kv_ts.
+  // q row = b*q_bs + h*q_hs + i*q_ts, out row likewise with o_*, key row = b*kv_bs + slot*kv_hs + j*kv_ts.
   // BHLc: (H*L, L, 1); BLHc (the layout of the flash-attention call): (L*H, 1, H).
-  int64_t q_bs, q_hs, q_ts, kv_bs, kv_hs, kv_ts;
+  int64_t q_bs, q_hs, q_ts, o_bs, o_hs, o_ts, kv_bs, kv_hs, kv_ts;
 };
 
 __device__ __forceinline__ u32 pack_bf16_hi(float lo, float hi) {  // exact for values with <= 8 significant bits
@@ -1190,7 +1190,7 @@ __global__ __launch_bounds__(NWV * 64, WPS) void fused_attn_kernel(AttnParams p)
 #pragma unroll
   for (int s = 0; s < NSVA; ++s) rq[s] = DEQ ? 0.f : __shfl(racc[s], col, 64) + r_run[s];
   if (q_live) {
-    __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D;
+    __bf16 *optr = p.out + (b * p.o_bs + hq * p.o_hs + qrow * p.o_ts) * D;
     // with the keys shared out: the normalized fp32 output and (reference, denominator) of
     // this share, for the combining kernel
     const bool shared_out = p.nsplit > 1;
@@ -1280,7 +1280,7 @@ __global__ __launch_bounds__(256) void combine_splits_kernel(AttnParams p) {
   const int bh = (int)(row / p.Lq), qrow = (int)(row % p.Lq);
   const int b = bh / p.Hkv, hs = bh % p.Hkv;
   const int hq = p.head_map ? p.head_map[hs] : hs;
-  __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D + c0;
+  __bf16 *optr = p.out + (b * p.o_bs + hq * p.o_hs + qrow * p.o_ts) * D + c0;
   *reinterpret_cast<uint2 *>(optr) = make_uint2(pack_io_rne<F16>(acc[0] * inv, acc[1] * inv), pack_io_rne<F16>(acc[2] * inv, acc[3] * inv));
 }
 
@@ -1363,15 +1363,17 @@ int dispatch_groups(const AttnParams &p, int gk, int gv, hipStream_t st) {
 }
 
 int set_layout(AttnParams &p, int layout, const char *who) {
-  if (layout == VARQ_LAYOUT_BHLC) {
+  if (layout == VARQ_LAYOUT_BHLC || layout == VARQ_LAYOUT_BHLC_OUT_BLHC) {
     p.q_bs = (int64_t)p.Hq * p.Lq; p.q_hs = p.Lq; p.q_ts = 1;
     p.kv_bs = (int64_t)p.Hkv * p.Lstride; p.kv_hs = p.Lstride; p.kv_ts = 1;
   } else if (layout == VARQ_LAYOUT_BLHC) {
     p.q_bs = (int64_t)p.Lq * p.Hq; p.q_hs = 1; p.q_ts = p.Hq;
     p.kv_bs = (int64_t)p.Lstride * p.Hkv; p.kv_hs = 1; p.kv_ts = p.Hkv;
   } else {
-    return varq_set_error(VARQ_ERR_INVALID, "%s: layout must be VARQ_LAYOUT_BHLC (0) or VARQ_LAYOUT_BLHC (1), got %d", who, layout);
+    return varq_set_error(VARQ_ERR_INVALID, "%s: layout must be VARQ_LAYOUT_BHLC (0), VARQ_LAYOUT_BLHC (1) or VARQ_LAYOUT_BHLC_OUT_BLHC (2), got %d", who, layout);
   }
+  p.o_bs = p.q_bs; p.o_hs = p.q_hs; p.o_ts = p.q_ts;
+  if (layout == VARQ_LAYOUT_BHLC_OUT_BLHC) { p.o_bs = (int64_t)p.Lq * p.Hq; p.o_hs = 1; p.o_ts = p.Hq; }
   return VARQ_OK;
 }
 
@@ -1871,7 +1873,7 @@ __global__ __launch_bounds__(FQ_NW * 64, 2) void fused_attn_fewq_kernel(AttnPara
     for (int g4 = 0; g4 < 4; ++g4)
       *reinterpret_cast<float4 *>(wptr + 8 * g4) = make_float4(mine[4 * g4] * inv, mine[4 * g4 + 1] * inv, mine[4 * g4 + 2] * inv, mine[4 * g4 + 3] * inv);
   } else {
-    __bf16 *optr = p.out + (b * p.q_bs + hq * p.q_hs + qrow * p.q_ts) * D + wave * 32 + 4 * half;
+    __bf16 *optr = p.out + (b * p.o_bs + hq * p.o_hs + qrow * p.o_ts) * D + wave * 32 + 4 * half;
 #pragma unroll
     for (int g4 = 0; g4 < 4; ++g4)
       *reinterpret_cast<uint2 *>(optr + 8 * g4) =

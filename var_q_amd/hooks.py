@@ -161,8 +161,8 @@ class _QuantizedSelfAttention(nn.Module):
                                               self.group_size, qkv.device, symmetric=self.symmetric)
         mul = None if scale_mul is None else scale_mul.detach().float().reshape(-1).contiguous()
         q = self.packed_cache.append_from_qkv(qkv, mul, l2norm, 1e-12, rope, token_start)
-        o = self.packed_cache.attend(q, scale)                                          # [B,H,L,c]
-        return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(x.dtype)
+        o = self.packed_cache.attend(q, scale, out_layout='BLHc')                       # [B,L,H,c]
+        return o.reshape(B, L, self.num_heads * self.head_dim).to(x.dtype)
 
     def _attn_dtype(self, main_type):
         """dtype of the fused attention: the module's compute dtype where the kernels have it
@@ -190,8 +190,8 @@ class _QuantizedSelfAttention(nn.Module):
                                                   self.group_size, q.device, symmetric=self.symmetric)
             self.packed_cache.append(k, v, layout=self.layout)
             qh = q if self.layout == 'BHLc' else q.transpose(1, 2)
-            o = self.packed_cache.attend(qh.to(self._attn_dtype(out_dtype)).contiguous(), scale)   # [B,H,L,c]
-            return o.transpose(1, 2).reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
+            o = self.packed_cache.attend(qh.to(self._attn_dtype(out_dtype)).contiguous(), scale, out_layout='BLHc')   # [B,L,H,c]
+            return o.reshape(B, L, self.num_heads * self.head_dim).to(out_dtype)
         if self.caching:
             if self.enable_quantization:
                 # (dequantized straight into the attention's dtype: the values `.to(out_dtype)` of

@@ -173,13 +173,17 @@ class PackedKVCache:
         return q_out
 
     def attend(self, q: torch.Tensor, softmax_scale: float, kv_limit: Optional[torch.Tensor] = None,
-               out: Optional[torch.Tensor] = None, exact_codes: bool = False) -> torch.Tensor:
+               out: Optional[torch.Tensor] = None, exact_codes: bool = False, out_layout: str = 'BHLc') -> torch.Tensor:
         """Fused dequant attention of q [B,H,Lq,D] (bf16; fp16 at D=64) over the cached tokens.
         K and V enter the products rounded to q's dtype, as in the reference; exact_codes=True
-        selects the form that does not round them where it exists (see ops.fused_attn)."""
+        selects the form that does not round them where it exists (see ops.fused_attn).
+        out_layout 'BLHc': the result as [B,Lq,H,D], the order an attention module reshapes to
+        [B,Lq,C] for its output projection (no transposing copy)."""
         assert self.len > 0, 'attend on an empty cache: append keys and values first'
+        assert out_layout in ('BHLc', 'BLHc')
         if out is None:
-            out = torch.empty_like(q)
+            B_, H_, Lq_, D_ = q.shape
+            out = torch.empty((B_, Lq_, H_, D_) if out_layout == 'BLHc' else q.shape, dtype=q.dtype, device=q.device)
         asym = not self.symmetric
         many = len(self.classes) > 1
         # side streams for the bit-width classes only where the call is large enough to gain from
@@ -198,7 +202,8 @@ class PackedKVCache:
             # launches share the GPU instead of queueing behind each other half-empty
             args = (q, c.k_words, c.k_scale, c.k_zp if asym else None, c.v_words, c.v_scale, c.v_zp if asym else None,
                     c.bits, c.bits, self.len, softmax_scale)
-            kw = dict(kv_limit=kv_limit, head_map=c.head_map if many else None, out=out, splits=splits, exact_codes=exact_codes)
+            kw = dict(kv_limit=kv_limit, head_map=c.head_map if many else None, out=out, splits=splits, exact_codes=exact_codes,
+                      out_layout=out_layout)
             if side and i:
                 stream = side[i - 1]
                 stream.wait_event(self._fork)

@@ -418,6 +418,22 @@ def _attn_dims(q, k_words, layout):
     return B, Hq, Lq, D, Hkv, Lstride, W
 
 
+def _attn_out(q, out, layout, out_layout, dims):
+    """(layout code of the call, output tensor): out looks like q unless out_layout says
+    tokens first for a heads-first call."""
+    B, Hq, Lq, D = dims
+    if out_layout is None or out_layout == layout:
+        code, shape = _LAYOUTS[layout], q.shape
+    else:
+        assert layout == 'BHLc' and out_layout == 'BLHc', 'out_layout: only tokens-first out of a heads-first call'
+        code, shape = 2, (B, Lq, Hq, D)
+    if out is None:
+        out = torch.empty(shape, dtype=q.dtype, device=q.device)
+    assert out.dtype == q.dtype and tuple(out.shape) == tuple(shape) and out.is_contiguous(), \
+        'out must be contiguous, of the dtype of q and of the shape its layout implies'
+    return code, out
+
+
 def _attn_workspace(lib, B, Hkv, Lq, Lk, D, nseg, splits, device):
     """Device memory for the partial results of a launch that shares keys out (None if the
     library would not); allocated on the current stream, so its reuse after the call is ordered."""
@@ -432,7 +448,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
                k_bits: int, v_bits: int, Lk: int, softmax_scale: float,
                kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
                out: Optional[torch.Tensor] = None, splits: int = 0, layout: str = 'BHLc',
-               exact_codes: bool = False) -> torch.Tensor:
+               exact_codes: bool = False, out_layout: Optional[str] = None) -> torch.Tensor:
     """q [B,Hq,Lq,D] bf16 (or fp16 at D=64, the VAR path); k/v_words [B,Hkv,Lstride,D*bits/32] int32;
     k/v_scale (zp) [B,Hkv,Lstride,D/group] fp32; attends keys 0..Lk-1.
     Returns out [B,Hq,Lq,D] of q's dtype (rows of heads not in head_map are untouched).
@@ -443,6 +459,8 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     group per key at D=128 in bf16 and is ignored elsewhere.
     layout 'BLHc': every tensor has tokens before heads instead ([B,Lq,Hq,D], [B,Lstride,Hkv,...]),
     the layout of the reference's flash-attention call.
+    out_layout 'BLHc' with layout 'BHLc': out is [B,Lq,Hq,D] while q and the cache stay heads
+    first -- what an attention module hands to its output projection, without a transposing copy.
     splits: over how many workgroups the keys of a query block are shared out (0: the
     library decides from the shape, 1: never, 2..8: exactly)."""
     for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_scale, 'k_scale'), (v_scale, 'v_scale')):
@@ -461,9 +479,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
     assert k_scale.dtype == torch.float32 and v_scale.dtype == torch.float32 and k_words.dtype == torch.int32 \
         and v_words.dtype == torch.int32
     assert 0 <= Lk <= Lstride, f'Lk={Lk} outside the cache of {Lstride} tokens'
-    if out is None:
-        out = torch.empty_like(q)
-    assert out.dtype == q.dtype and out.shape == q.shape and out.is_contiguous(), 'out must look like q'
+    code, out = _attn_out(q, out, layout, out_layout, (B, Hq, Lq, D))
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
@@ -479,7 +495,7 @@ def fused_attn(q: torch.Tensor, k_words: torch.Tensor, k_scale: torch.Tensor, k_
                                   k_words.data_ptr(), k_scale.data_ptr(), _ptr(k_zp), k_bits, k_group,
                                   v_words.data_ptr(), v_scale.data_ptr(), _ptr(v_zp), v_bits, v_group,
                                   B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                  _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ATTN_DT[q.dtype],
+                                  _ptr(kv_limit), float(softmax_scale), code, _ATTN_DT[q.dtype],
                                   int(bool(exact_codes)), _ptr(ws), ws_bytes,
                                   int(splits), _stream(q)), 'varq_fused_attn')
     return out
@@ -491,7 +507,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                        bits: int, Lk: int, softmax_scale: float,
                        kv_limit: Optional[torch.Tensor] = None, head_map: Optional[torch.Tensor] = None,
                        out: Optional[torch.Tensor] = None, seg_ends: Optional[Sequence[int]] = None,
-                       splits: int = 0, layout: str = 'BHLc') -> torch.Tensor:
+                       splits: int = 0, layout: str = 'BHLc', out_layout: Optional[str] = None) -> torch.Tensor:
     """Attention over a cache quantized per (head, channel): the scale layout of the
     reference's G_SCALE_HEAD_DIM / G_HEAD_DIM methods (VAR_Q/quant.py:84-88), scalar scales
     (G_TENSOR, G_SCALE) expanded to the table, and the affine per-head-per-dim variant.
@@ -501,7 +517,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
     where the tables change along the keys: a cache filled step by step by the reference's
     append methods has one table per step (VAR_Q/quant.py:196-201).
     With a single table the zero-point of K may be None even for an affine K: it shifts all
-    logits of a query alike.  splits and layout as in fused_attn."""
+    logits of a query alike.  splits, layout and out_layout as in fused_attn."""
     for t, n in ((q, 'q'), (k_words, 'k_words'), (v_words, 'v_words'), (k_chan_scale, 'k_chan_scale'),
                  (v_chan_scale, 'v_chan_scale')):
         _gpu(t, n)
@@ -522,9 +538,7 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                 f'{n} must be fp32 [nseg, Hkv, D] (more tables than segments are allowed)'
     assert k_words.dtype == torch.int32 and v_words.dtype == torch.int32
     assert 0 <= Lk <= Lstride, f'Lk={Lk} outside the cache of {Lstride} tokens'
-    if out is None:
-        out = torch.empty_like(q)
-    assert out.dtype == q.dtype and out.shape == q.shape and out.is_contiguous(), 'out must look like q'
+    code, out = _attn_out(q, out, layout, out_layout, (B, Hq, Lq, D))
     if kv_limit is not None:
         _gpu(kv_limit, 'kv_limit')
         assert kv_limit.dtype == torch.int32 and kv_limit.numel() == Lq and kv_limit.is_contiguous()
@@ -540,6 +554,6 @@ def fused_attn_channel(q: torch.Tensor, k_words: torch.Tensor, k_chan_scale: tor
                                           k_words.data_ptr(), k_chan_scale.data_ptr(), _ptr(k_chan_zp),
                                           v_words.data_ptr(), v_chan_scale.data_ptr(), _ptr(v_chan_zp),
                                           nseg, ends, bits, B, Hq, Hkv, _ptr(head_map), Lq, Lk, Lstride, D,
-                                          _ptr(kv_limit), float(softmax_scale), _LAYOUTS[layout], _ATTN_DT[q.dtype],
+                                          _ptr(kv_limit), float(softmax_scale), code, _ATTN_DT[q.dtype],
                                           _ptr(ws), ws_bytes, int(splits), _stream(q)), 'varq_fused_attn_channel')
     return out
