@@ -294,3 +294,37 @@ def test_dropin_module_dequantizes_into_the_attention_dtype(dev, layout, method,
         x = torch.randn(2, n, C, device=dev, dtype=dtype)
         assert torch.equal(a_mod(x), b_mod(x))
     assert isinstance(a_mod.k_quant, VAR_Q) and not isinstance(b_mod.k_quant, VAR_Q)
+
+
+def test_parameter_only_tensors_are_kept_for_one_cached_schedule(dev):
+    """Under no_grad and kv_caching(True) the qkv bias and the per-head multiplier are built once
+    per schedule; the outputs are those of the module that rebuilds them every call, and a
+    parameter changed between two schedules is seen by the next one."""
+    torch.manual_seed(11)
+    C, H = 256, 4
+    kw = dict(embed_dim=C, num_heads=H, layout='BLHc', q_bits=4, quant_method='G_GROUP', group_size=64, symmetric=False,
+              enable_quantization=True, max_tokens=40, fused=True, fused_producer=True)
+    a_mod = hooks.VarSelfAttention(0, **kw).to(dev).to(torch.bfloat16)
+    b_mod = hooks.VarSelfAttention(0, **kw).to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        a_mod.q_bias.normal_(); a_mod.v_bias.normal_()
+    b_mod.load_state_dict(a_mod.state_dict())
+    xs = [torch.randn(2, n, C, device=dev, dtype=torch.bfloat16) for n in (1, 4, 9, 16)]
+    for round_ in range(2):
+        a_mod.kv_caching(True)
+        b_mod.kv_caching(True)
+        for x in xs:
+            note('hooks session tensors', round_, x.shape[1])
+            with torch.no_grad():
+                a = a_mod(x)
+            with torch.enable_grad():             # nothing is kept while gradients are recorded
+                b = b_mod(x)
+            assert torch.equal(a, b.detach())
+        assert len(a_mod._session) >= 2 and len(b_mod._session) == 0
+        a_mod.kv_caching(False)
+        b_mod.kv_caching(False)
+        assert a_mod._session == {}
+        with torch.no_grad():                     # a new multiplier and bias for the second schedule
+            for m in (a_mod, b_mod):
+                m.scale_mul_1H11.fill_(1.25)
+                m.q_bias.mul_(0.5)

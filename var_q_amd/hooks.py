@@ -118,6 +118,7 @@ class _QuantizedSelfAttention(nn.Module):
         self.caching, self.cached_k, self.cached_v = enable, None, None
         self.k_quant = self.v_quant = None
         self.packed_cache = None
+        self._session = {}          # tensors derived from the parameters alone, kept while a schedule is cached
         if enable and self.enable_quantization and self.fused is not True:
             kw = dict(quant_bits=self.q_bits, qkv_format=self.layout, quant_method=self.quant_method, blk_idx=self.block_idx)
             if self.quant_method == 'G_GROUP' or not self.symmetric:
@@ -130,8 +131,21 @@ class _QuantizedSelfAttention(nn.Module):
 
     def _qkv(self, x):
         B, L, _ = x.shape
-        bias = torch.cat((self.q_bias, self.zero_k_bias, self.v_bias))
-        return F.linear(x, self.mat_qkv.weight.to(x.dtype), bias.to(x.dtype)).view(B, L, 3, self.num_heads, self.head_dim)
+        bias = self._per_session(('qkv bias', x.dtype),
+                                 lambda: torch.cat((self.q_bias, self.zero_k_bias, self.v_bias)).to(x.dtype))
+        return F.linear(x, self.mat_qkv.weight.to(x.dtype), bias).view(B, L, 3, self.num_heads, self.head_dim)
+
+    def _per_session(self, key, make):
+        """make() once per cached schedule (kv_caching(True) .. kv_caching(False): inference, the
+        parameters do not change under it), every time otherwise, as the reference's modules do
+        (VAR/models/basic_var.py:122, :138): a handful of tiny launches per call that cost the
+        small scales more host time than their attention takes."""
+        if not self.caching or torch.is_grad_enabled():
+            return make()
+        session = self.__dict__.setdefault('_session', {})
+        if key not in session:
+            session[key] = make()
+        return session[key]
 
     def _project(self, x):
         qkv = self._qkv(x)
@@ -159,7 +173,7 @@ class _QuantizedSelfAttention(nn.Module):
         if self.packed_cache is None:
             self.packed_cache = PackedKVCache(B, self.num_heads, self.max_tokens, self.head_dim, self.q_bits,
                                               self.group_size, qkv.device, symmetric=self.symmetric)
-        mul = None if scale_mul is None else scale_mul.detach().float().reshape(-1).contiguous()
+        mul = None if scale_mul is None else self._per_session('scale_mul fp32', lambda: scale_mul().detach().float().reshape(-1).contiguous())
         q = self.packed_cache.append_from_qkv(qkv, mul, l2norm, 1e-12, rope, token_start)
         o = self.packed_cache.attend(q, scale, out_layout='BLHc')                       # [B,L,H,c]
         return o.reshape(B, L, self.num_heads * self.head_dim).to(x.dtype)
@@ -233,7 +247,7 @@ class VarSelfAttention(_QuantizedSelfAttention):
 
     def forward(self, x: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         if self.caching and self.fused_producer:
-            mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp() if self.attn_l2_norm else None
+            mul = (lambda: self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp()) if self.attn_l2_norm else None
             o = self._fused_from_qkv(x, self.scale, mul, self.attn_l2_norm, None, None, attn_bias)
             return self.proj(o.to(self.proj.weight.dtype))
         q, k, v = self._project(x)
@@ -274,10 +288,11 @@ class InfinitySelfAttention(_QuantizedSelfAttention):
         """rope = (cos, sin) from rope2d_tables for the whole schedule; token_start =
         number of tokens of the scales before this one."""
         if self.caching and self.fused_producer:
-            mul = self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp() if self.cos_attn else None
+            mul = (lambda: self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp()) if self.cos_attn else None
             rope_dev = None
             if rope is not None:
-                rope_dev = tuple(t.to(x.device, torch.float32).contiguous() for t in rope)
+                rope_dev = self._per_session(('rope', id(rope[0]), id(rope[1])),
+                                             lambda: tuple(t.to(x.device, torch.float32).contiguous() for t in rope))
             o = self._fused_from_qkv(x, self.scale, mul, self.cos_attn, rope_dev, token_start, attn_bias)
             return self.proj(o.to(self.proj.weight.dtype))
         q, k, v = self._project(x)
