@@ -291,8 +291,7 @@ class InfinitySelfAttention(_QuantizedSelfAttention):
             mul = (lambda: self.scale_mul_1H11.clamp_max(self.max_scale_mul).exp()) if self.cos_attn else None
             rope_dev = None
             if rope is not None:
-                rope_dev = self._per_session(('rope', id(rope[0]), id(rope[1])),
-                                             lambda: tuple(t.to(x.device, torch.float32).contiguous() for t in rope))
+                rope_dev = tuple(t.to(x.device, torch.float32).contiguous() for t in rope)   # (no copies for fp32 tables on the device)
             o = self._fused_from_qkv(x, self.scale, mul, self.cos_attn, rope_dev, token_start, attn_bias)
             return self.proj(o.to(self.proj.weight.dtype))
         q, k, v = self._project(x)
